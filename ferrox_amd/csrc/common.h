@@ -1,0 +1,99 @@
+// Shared by every kernel library of the engine (gfx950 only).
+//
+// Each library is a plain shared object with `extern "C"` entry points that take
+// raw device pointers and a HIP stream; Python calls them through ctypes.  An
+// entry point checks its sizes on the host before it launches anything and
+// returns 0, or a non-zero code after storing a message for fx_last_error().
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <math.h>
+
+#define FX_API extern "C" __attribute__((visibility("default")))
+
+// element types as the Python side numbers them
+enum FxDtype { FX_F32 = 0, FX_BF16 = 1 };
+
+static thread_local char fx_err_buf[512];
+
+static int fx_fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(fx_err_buf, sizeof(fx_err_buf), fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+#define FX_DEFINE_LAST_ERROR() \
+    FX_API const char* fx_last_error() { return fx_err_buf; }
+
+#define FX_REQUIRE(cond, ...)                      \
+    do {                                           \
+        if (!(cond)) return fx_fail(__VA_ARGS__);  \
+    } while (0)
+
+#define FX_CHECK_LAUNCH(name)                                                     \
+    do {                                                                          \
+        hipError_t e_ = hipGetLastError();                                        \
+        if (e_ != hipSuccess) return fx_fail("%s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+// ---- bfloat16 as raw bits --------------------------------------------------
+struct bf16 {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_float(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16 float_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    bf16 r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r.bits = (uint16_t)((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r.bits = (uint16_t)(u >> 16);
+    }
+    return r;
+}
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16 v) { return bf16_to_float(v); }
+__device__ __forceinline__ void from_float(float* p, float v) { *p = v; }
+__device__ __forceinline__ void from_float(bf16* p, float v) { *p = float_to_bf16(v); }
+
+// load one element of a tensor whose element type is only known at run time
+__device__ __forceinline__ float load_as_float(const void* p, int dtype, size_t i) {
+    return dtype == FX_F32 ? ((const float*)p)[i] : bf16_to_float(((const bf16*)p)[i]);
+}
+
+// ---- wave (64 lanes) and block reductions in a fixed order ------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// sum over a block of NW waves; every thread gets the result.  `red` has NW floats.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) s += red[i];
+    return s;
+}
+
+static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

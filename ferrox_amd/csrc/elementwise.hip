@@ -1,0 +1,266 @@
+// Row-wise kernels: embedding gather, RMSNorm, rotary + cache write, residual
+// add, casts, the weighted sum of routed expert outputs.
+//
+// The residual stream `h` is float32 in both precisions; normed activations and
+// q/k/v are in the activation type T (float or bf16).  Statistics, angles and
+// sums are computed in float32.
+#include "common.h"
+
+FX_DEFINE_LAST_ERROR()
+
+// ---------------------------------------------------------------------------
+// embedding: h[t, :] = table[ids[t], :]   (no scale; ferrox-models/src/decoder.rs:1279-1284)
+// ---------------------------------------------------------------------------
+template <typename W>
+__global__ void embed_kernel(const W* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ h, int H, int V) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= V) {  // the host rejects such ids; never read outside the table
+        for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = __int_as_float(0x7fc00000);
+        return;
+    }
+    const W* row = table + (size_t)id * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = to_float(row[c]);
+}
+
+FX_API int fx_embed(void* stream, int w_dtype, const void* table, const int* ids, float* h,
+                    int T, int H, int V) {
+    FX_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (w_dtype == FX_F32)
+        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, h, H, V);
+    else if (w_dtype == FX_BF16)
+        embed_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)table, ids, h, H, V);
+    else
+        return fx_fail("embed: unknown table dtype %d", w_dtype);
+    FX_CHECK_LAUNCH("embed");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, multiply order x*s*w
+// (ferrox-core/src/matmul.rs:62-69).  Input rows are float32 (the residual
+// stream), optionally gathered through `rows`; output is T.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
+                                                      const void* __restrict__ w, int w_dtype,
+                                                      T* __restrict__ out, int H, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* x = h + (size_t)(rows ? rows[r] : r) * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) {
+        float v = x[c];
+        ss += v * v;
+    }
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += 256)
+        from_float(out + (size_t)r * H + c, x[c] * scale * load_as_float(w, w_dtype, c));
+}
+
+FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* rows, const void* w,
+                      int w_dtype, void* out, int R, int H, float eps) {
+    FX_REQUIRE(R >= 0 && H > 0, "rmsnorm: bad sizes R=%d H=%d", R, H);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "rmsnorm: unknown weight dtype %d", w_dtype);
+    if (R == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == FX_F32)
+        rmsnorm_kernel<float><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, H, eps);
+    else if (out_dtype == FX_BF16)
+        rmsnorm_kernel<bf16><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, H, eps);
+    else
+        return fx_fail("rmsnorm: unknown output dtype %d", out_dtype);
+    FX_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Rotary position encoding of q and k, and the write of k and v into the pages.
+//
+// Split-half pairing (i, i + rot/2), angle = pos * theta^(-2i/rot)
+// (ferrox-core/src/attention.rs:20-32); `interleaved` pairs (2i, 2i+1) instead.
+// rot = 0 rotates nothing.  v is never rotated.  Key pages hold
+// [page][kv_head][slot][head_dim]; value pages hold the transpose
+// [page][kv_head][head_dim][slot], which is what the attention kernels read.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+    T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
+    const int* __restrict__ positions, const int* __restrict__ token_seq,
+    const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    const int half = rot >> 1;
+    T* k_dst = nullptr;
+    T* v_dst = nullptr;
+    int slot = 0;
+    if (k_pages) {
+        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+        slot = pos % bs;
+        k_dst = k_pages + (size_t)page * nkv * bs * hd;
+        v_dst = v_pages + (size_t)page * nkv * hd * bs;
+    }
+    // rotated pairs of q (in place) and k (into the page)
+    const int n_pairs = (nh + nkv) * half;
+    for (int i = threadIdx.x; i < n_pairs; i += 256) {
+        const int head = i / half, p = i % half;
+        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
+        float sn, cs;
+        sincosf((float)pos * freq, &sn, &cs);
+        const int ia = interleaved ? 2 * p : p;
+        const int ib = interleaved ? 2 * p + 1 : p + half;
+        if (head < nh) {
+            T* row = q + (size_t)t * ldq + (size_t)head * hd;
+            const float a = to_float(row[ia]), b = to_float(row[ib]);
+            from_float(row + ia, a * cs - b * sn);
+            from_float(row + ib, a * sn + b * cs);
+        } else if (k_dst) {
+            const int kh = head - nh;
+            const T* row = k + (size_t)t * ldk + (size_t)kh * hd;
+            const float a = to_float(row[ia]), b = to_float(row[ib]);
+            T* dst = k_dst + ((size_t)kh * bs + slot) * hd;
+            from_float(dst + ia, a * cs - b * sn);
+            from_float(dst + ib, a * sn + b * cs);
+        }
+    }
+    if (!k_dst) return;
+    // the part of k beyond the rotated dimensions, and v
+    const int tail = hd - rot;
+    for (int i = threadIdx.x; i < nkv * tail; i += 256) {
+        const int kh = i / tail, d = rot + i % tail;
+        k_dst[((size_t)kh * bs + slot) * hd + d] = k[(size_t)t * ldk + (size_t)kh * hd + d];
+    }
+    for (int i = threadIdx.x; i < nkv * hd; i += 256) {
+        const int kh = i / hd, d = i % hd;
+        v_dst[((size_t)kh * hd + d) * bs + slot] = v[(size_t)t * ldv + i];
+    }
+}
+
+FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const void* k, int ldk,
+                            const void* v, int ldv, const int* positions, const int* token_seq,
+                            const int* block_table, int max_blocks, void* k_pages, void* v_pages,
+                            int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
+    FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
+    FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
+    FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FX_F32)
+        rope_kv_write_kernel<float><<<T, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
+                                                      positions, token_seq, block_table, max_blocks,
+                                                      (float*)k_pages, (float*)v_pages, nh, nkv, hd, bs, rot,
+                                                      interleaved, theta);
+    else if (dtype == FX_BF16)
+        rope_kv_write_kernel<bf16><<<T, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
+                                                     positions, token_seq, block_table, max_blocks,
+                                                     (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, bs, rot,
+                                                     interleaved, theta);
+    else
+        return fx_fail("rope_kv_write: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("rope_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// h[t, :] += y[t, :]  (float32 sum), y of either type.  Used by parts that have
+// no fused epilogue of their own.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__ y, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) h[i] += to_float(y[i]);
+}
+
+FX_API int fx_residual_add(void* stream, int y_dtype, float* h, const void* y, long n) {
+    FX_REQUIRE(n >= 0, "residual_add: bad size");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 65536) blocks = 65536;
+    if (y_dtype == FX_F32)
+        residual_add_kernel<float><<<blocks, 256, 0, s>>>(h, (const float*)y, (size_t)n);
+    else if (y_dtype == FX_BF16)
+        residual_add_kernel<bf16><<<blocks, 256, 0, s>>>(h, (const bf16*)y, (size_t)n);
+    else
+        return fx_fail("residual_add: unknown dtype %d", y_dtype);
+    FX_CHECK_LAUNCH("residual_add");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// casts between float32 and bf16
+// ---------------------------------------------------------------------------
+template <typename A, typename B>
+__global__ void cast_kernel(const A* __restrict__ a, B* __restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) from_float(b + i, to_float(a[i]));
+}
+
+FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, long n) {
+    FX_REQUIRE(n >= 0, "cast: bad size");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 65536) blocks = 65536;
+    if (src_dtype == FX_F32 && dst_dtype == FX_BF16)
+        cast_kernel<float, bf16><<<blocks, 256, 0, s>>>((const float*)src, (bf16*)dst, (size_t)n);
+    else if (src_dtype == FX_BF16 && dst_dtype == FX_F32)
+        cast_kernel<bf16, float><<<blocks, 256, 0, s>>>((const bf16*)src, (float*)dst, (size_t)n);
+    else
+        return fx_fail("cast: unsupported pair %d -> %d", src_dtype, dst_dtype);
+    FX_CHECK_LAUNCH("cast");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Weighted sum of the routed experts' outputs into the residual stream:
+//   h[t, :] += sum_j w[t, j] * y[inv[t*k + j], :]
+// in ascending j, the selection order (ferrox-moe/src/lib.rs:735-745).
+// y is float32 [n_sorted, H].
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                          const int* __restrict__ inv, const float* __restrict__ w,
+                                                          int H, int k) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < H; c += 256) {
+        float acc = 0.f;
+        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)inv[t * k + j] * H + c];
+        h[(size_t)t * H + c] += acc;
+    }
+}
+
+FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv, const float* w,
+                          int T, int H, int k) {
+    FX_REQUIRE(T >= 0 && H > 0 && k > 0, "moe_combine: bad sizes");
+    if (T == 0) return 0;
+    moe_combine_kernel<<<T, 256, 0, (hipStream_t)stream>>>(h, y, inv, w, H, k);
+    FX_CHECK_LAUNCH("moe_combine");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// fill a buffer of 32-bit words (used instead of a memset so that callers may
+// record it into a HIP graph)
+// ---------------------------------------------------------------------------
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+FX_API int fx_fill_u32(void* stream, void* p, unsigned v, long n) {
+    FX_REQUIRE(n >= 0, "fill: bad size");
+    if (n == 0) return 0;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 65536) blocks = 65536;
+    fill_u32_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((uint32_t*)p, v, (size_t)n);
+    FX_CHECK_LAUNCH("fill");
+    return 0;
+}

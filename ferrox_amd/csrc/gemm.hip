@@ -1,0 +1,378 @@
+// Matrix products  C[m, n] = sum_k A[m, k] * W[n, k]  (weights are [out, in] as
+// the checkpoint stores them; ferrox-core/src/matmul.rs:5-8) with fused epilogues,
+// for plain and for expert-grouped rows.
+//
+//  * bfloat16: MFMA 16x16x32 tiles, float32 accumulators.
+//  * float32 : FMA in float32 only (no reduced-precision matrix mode).
+//
+// In both, one output element is accumulated over k in ascending order with a
+// single accumulator, whatever the tile shape and whatever else is in the batch,
+// so a row's result does not depend on how many rows are computed with it.
+//
+// Grouped mode: rows are sorted by expert; expert e owns rows
+// [expert_offsets[e], expert_offsets[e+1]) and the weights at W + e * w_stride.
+// Dual mode: two weight matrices (gate, up) are multiplied at once and the
+// epilogue stores silu(gate) * up  (ferrox-moe/src/lib.rs:655-658).
+#include "common.h"
+
+FX_DEFINE_LAST_ERROR()
+
+enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_RESID = 2, EPI_SILU_MUL = 3 };
+
+struct GemmArgs {
+    const void* A;
+    long lda;
+    const void* W;
+    long w_stride;      // elements between experts (grouped)
+    long up_offset;     // elements from the gate matrix to the up matrix (dual)
+    const void* bias;   // [N] or null
+    int bias_dtype;
+    void* C;
+    long ldc;
+    const float* row_scale;  // [M] or null, multiplies the product before it is added (EPI_RESID)
+    const int* a_rows;       // [M] or null: row of A to read for logical row m
+    const int* expert_offsets;  // [E+1] or null
+    int E;
+    int M, N, K;
+    int vec_ok;  // 16-byte loads are legal for A and W
+};
+
+// block -> (first logical row, end of rows, expert).  Plain: tiles of TM rows.
+// Grouped: walk the experts' tile counts; blocks past the last tile get r0 = -1.
+template <int TM>
+__device__ __forceinline__ void locate_rows(const GemmArgs& g, int tile, int& r0, int& r_end, int& expert) {
+    if (!g.expert_offsets) {
+        r0 = tile * TM;
+        r_end = g.M;
+        expert = 0;
+        if (r0 >= g.M) r0 = -1;
+        return;
+    }
+    int acc = 0;
+    r0 = -1;
+    r_end = 0;
+    expert = 0;
+    for (int e = 0; e < g.E; ++e) {
+        const int b = g.expert_offsets[e], en = g.expert_offsets[e + 1];
+        const int nt = (en - b + TM - 1) / TM;
+        if (tile < acc + nt) {
+            r0 = b + (tile - acc) * TM;
+            r_end = en;
+            expert = e;
+            return;
+        }
+        acc += nt;
+    }
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+// ===========================================================================
+// bfloat16 on MFMA
+// ===========================================================================
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+#define BK 64
+#define LDS_STRIDE (BK + 8)  // bf16 elements; keeps 16-byte reads of 16 rows on distinct banks
+
+__device__ __forceinline__ uint4 load_chunk(const bf16* row, int k, int K, int vec_ok) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (!row || k >= K) return v;
+    if (vec_ok && k + 8 <= K) return *(const uint4*)(row + k);
+    uint16_t tmp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tmp[i] = (k + i < K) ? row[k + i].bits : (uint16_t)0;
+    v.x = tmp[0] | ((uint32_t)tmp[1] << 16);
+    v.y = tmp[2] | ((uint32_t)tmp[3] << 16);
+    v.z = tmp[4] | ((uint32_t)tmp[5] << 16);
+    v.w = tmp[6] | ((uint32_t)tmp[7] << 16);
+    return v;
+}
+
+// TM x TN block tile (TN counts weight rows: in dual mode half of them are gate
+// rows and half up rows, interleaved in groups of 16), 4 waves of WM x WN.
+template <int TM, int TN, int WM, int WN, bool DUAL, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
+    constexpr int WAVES_N = TN / WN;
+    static_assert((TM / WM) * WAVES_N == 4, "four waves per block");
+    constexpr int MT = WM / 16, NT = WN / 16;
+    constexpr int NA = (TM * 8 + 255) / 256, NB = (TN * 8 + 255) / 256;
+    constexpr int OUT_TN = DUAL ? TN / 2 : TN;
+    __shared__ __attribute__((aligned(16))) bf16 As[TM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16 Bs[TN * LDS_STRIDE];
+
+    int r0, r_end, expert;
+    locate_rows<TM>(g, blockIdx.y, r0, r_end, expert);
+    if (r0 < 0) return;
+    const int n0 = blockIdx.x * OUT_TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const bf16* Abase = (const bf16*)g.A;
+    const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
+
+    // the row each of this thread's chunks comes from stays the same for all k
+    const bf16* a_src[NA];
+    const bf16* b_src[NB];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const int c = tid + i * 256, row = c >> 3;
+        a_src[i] = nullptr;
+        if (c < TM * 8 && r0 + row < r_end) {
+            const int m = r0 + row;
+            a_src[i] = Abase + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        const int c = tid + i * 256, row = c >> 3;
+        b_src[i] = nullptr;
+        if (c < TN * 8) {
+            if (DUAL) {
+                const int col = n0 + (row >> 5) * 16 + (row & 15);
+                if (col < g.N) b_src[i] = Wbase + (size_t)col * g.K + (((row >> 4) & 1) ? g.up_offset : 0);
+            } else {
+                if (n0 + row < g.N) b_src[i] = Wbase + (size_t)(n0 + row) * g.K;
+            }
+        }
+    }
+
+    f32x4_t acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    uint4 a_reg[NA], b_reg[NB];
+    const int kc = (tid & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) a_reg[i] = load_chunk(a_src[i], kc, g.K, g.vec_ok);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) b_reg[i] = load_chunk(b_src[i], kc, g.K, g.vec_ok);
+
+    for (int k0 = 0; k0 < g.K; k0 += BK) {
+        __syncthreads();  // the previous tile has been read
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int c = tid + i * 256;
+            if (c < TM * 8) *(uint4*)(As + (c >> 3) * LDS_STRIDE + kc) = a_reg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const int c = tid + i * 256;
+            if (c < TN * 8) *(uint4*)(Bs + (c >> 3) * LDS_STRIDE + kc) = b_reg[i];
+        }
+        __syncthreads();
+        if (k0 + BK < g.K) {  // fetch the next tile while this one is multiplied
+#pragma unroll
+            for (int i = 0; i < NA; ++i) a_reg[i] = load_chunk(a_src[i], k0 + BK + kc, g.K, g.vec_ok);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) b_reg[i] = load_chunk(b_src[i], k0 + BK + kc, g.K, g.vec_ok);
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks) {
+            const int koff = ks * 32 + (lane >> 4) * 8;
+            bf16x8_t af[MT], bfr[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                af[i] = *(const bf16x8_t*)(As + (wm * WM + i * 16 + (lane & 15)) * LDS_STRIDE + koff);
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                bfr[j] = *(const bf16x8_t*)(Bs + (wn * WN + j * 16 + (lane & 15)) * LDS_STRIDE + koff);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
+            if (m >= r_end) continue;
+            if (DUAL) {
+#pragma unroll
+                for (int j = 0; j < NT; j += 2) {
+                    const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
+                    if (n < g.N)
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(acc[i][j][r]) * acc[i][j + 1][r]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const int n = n0 + wn * WN + j * 16 + (lane & 15);
+                    if (n >= g.N) continue;
+                    float v = acc[i][j][r];
+                    if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
+                    if (EPI == EPI_STORE) {
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
+                    } else if (EPI == EPI_STORE_F32) {
+                        ((float*)g.C)[(size_t)m * g.ldc + n] = v;
+                    } else {
+                        if (g.row_scale) v *= g.row_scale[m];
+                        ((float*)g.C)[(size_t)m * g.ldc + n] += v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ===========================================================================
+// float32 with FMA
+// ===========================================================================
+#define FK 16
+// 64 x 64 outputs per block, 256 threads, 4 x 4 per thread.
+template <bool DUAL, int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
+    __shared__ float As[FK][64 + 4];
+    __shared__ float Bs[DUAL ? 2 : 1][FK][64 + 4];
+    int r0, r_end, expert;
+    locate_rows<64>(g, blockIdx.y, r0, r_end, expert);
+    if (r0 < 0) return;
+    const int n0 = blockIdx.x * 64;
+    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+    const float* Abase = (const float*)g.A;
+    const float* Wbase = (const float*)g.W + (size_t)expert * g.w_stride;
+
+    // loader: element idx = tid + i*256 of a 64 x 16 tile, k fastest
+    const float* a_src[4];
+    const float* b_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (tid + i * 256) >> 4;
+        a_src[i] = nullptr;
+        b_src[i] = nullptr;
+        if (r0 + row < r_end) {
+            const int m = r0 + row;
+            a_src[i] = Abase + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda;
+        }
+        if (n0 + row < g.N) b_src[i] = Wbase + (size_t)(n0 + row) * g.K;
+    }
+    const int kk = tid & 15;
+
+    float acc[4][4] = {}, acc2[4][4] = {};
+    for (int k0 = 0; k0 < g.K; k0 += FK) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = (tid + i * 256) >> 4;
+            const bool kin = k0 + kk < g.K;
+            As[kk][row] = (a_src[i] && kin) ? a_src[i][k0 + kk] : 0.f;
+            Bs[0][kk][row] = (b_src[i] && kin) ? b_src[i][k0 + kk] : 0.f;
+            if (DUAL) Bs[1][kk][row] = (b_src[i] && kin) ? b_src[i][g.up_offset + k0 + kk] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < FK; ++k) {
+            float a[4], b[4], b2[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[0][k][tx * 4 + j];
+            if (DUAL) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b2[j] = Bs[1][k][tx * 4 + j];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                    if (DUAL) acc2[i][j] = fmaf(a[i], b2[j], acc2[i][j]);
+                }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = r0 + ty * 4 + i;
+        if (m >= r_end) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= g.N) continue;
+            float v = acc[i][j];
+            float* out = (float*)g.C + (size_t)m * g.ldc + n;
+            if (DUAL) {
+                *out = silu_f(v) * acc2[i][j];
+            } else {
+                if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
+                if (EPI == EPI_RESID) {
+                    if (g.row_scale) v *= g.row_scale[m];
+                    *out += v;
+                } else {
+                    *out = v;
+                }
+            }
+        }
+    }
+}
+
+// ===========================================================================
+// host side
+// ===========================================================================
+template <int TM, int TN, int WM, int WN>
+static void launch_bf16(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
+    const bool dual = epi == EPI_SILU_MUL;
+    dim3 grid(ceil_div(g.N, dual ? TN / 2 : TN), m_tiles);
+    switch (epi) {
+        case EPI_STORE: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_STORE><<<grid, 256, 0, s>>>(g); break;
+        case EPI_STORE_F32: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_STORE_F32><<<grid, 256, 0, s>>>(g); break;
+        case EPI_RESID: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_RESID><<<grid, 256, 0, s>>>(g); break;
+        default: gemm_bf16_kernel<TM, TN, WM, WN, true, EPI_SILU_MUL><<<grid, 256, 0, s>>>(g); break;
+    }
+}
+
+// dtype: type of A and W.  C is: T for EPI_STORE and EPI_SILU_MUL, float32 otherwise.
+// rows_hint: in grouped mode, the expected number of rows per expert (chooses the tile).
+FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
+                   long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
+                   const float* row_scale, const int* a_rows, const int* expert_offsets, int E,
+                   int M, int N, int K) {
+    FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
+    FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
+    FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    FX_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%ld ldc=%ld too small for K=%d N=%d", lda, ldc, K, N);
+    FX_REQUIRE(!(epi == EPI_SILU_MUL && bias), "gemm: the gate/up epilogue takes no bias");
+    FX_REQUIRE(!expert_offsets || E > 0, "gemm: grouped mode needs E > 0");
+    FX_REQUIRE(!bias || bias_dtype == FX_F32 || bias_dtype == FX_BF16, "gemm: unknown bias dtype %d", bias_dtype);
+    if (M == 0) return 0;
+    GemmArgs g;
+    g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
+    g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
+    g.a_rows = a_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
+    hipStream_t s = (hipStream_t)stream;
+    const int nonempty = expert_offsets ? (E < M ? E : M) : 0;
+    if (dtype == FX_F32) {
+        g.vec_ok = 0;
+        const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
+        dim3 grid(ceil_div(N, 64), m_tiles);
+        switch (epi) {
+            case EPI_STORE:
+            case EPI_STORE_F32: gemm_f32_kernel<false, EPI_STORE_F32><<<grid, 256, 0, s>>>(g); break;
+            case EPI_RESID: gemm_f32_kernel<false, EPI_RESID><<<grid, 256, 0, s>>>(g); break;
+            default: gemm_f32_kernel<true, EPI_SILU_MUL><<<grid, 256, 0, s>>>(g); break;
+        }
+        FX_CHECK_LAUNCH("gemm_f32");
+        return 0;
+    }
+    g.vec_ok = (K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
+               (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+    const long per_group = expert_offsets ? (M + E - 1) / E : M;
+    if (per_group <= 16) {
+        const int m_tiles = M / 16 + (expert_offsets ? nonempty : (M % 16 != 0));
+        launch_bf16<16, 256, 16, 64>(g, epi, m_tiles, s);
+    } else if (per_group <= 64) {
+        const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
+        launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
+    } else {
+        const int m_tiles = M / 128 + (expert_offsets ? nonempty : (M % 128 != 0));
+        launch_bf16<128, 128, 64, 64>(g, epi, m_tiles, s);
+    }
+    FX_CHECK_LAUNCH("gemm_bf16");
+    return 0;
+}

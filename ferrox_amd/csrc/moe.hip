@@ -1,0 +1,199 @@
+// Routing of tokens to experts.
+//
+//  fx_router_topk : router logits (float32 sums), a gating function over all
+//                   experts, the k best, optional renormalisation; and the
+//                   scalar sigmoid gate of a shared expert.
+//  fx_moe_align   : sorts the (token, slot) pairs by expert with a stable
+//                   counting sort, so that a grouped matrix product sees each
+//                   expert's rows together.
+#include "common.h"
+
+FX_DEFINE_LAST_ERROR()
+
+#define E_MAX 1024
+#define K_MAX 32
+#define NEG_INFINITY_F (-INFINITY)
+
+enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
+
+// One block of 256 threads per token.
+//   logits[e] = sum_c x[c] * Wr[e, c]            (no bias; ferrox-models/src/decoder.rs:2915)
+//   softmax over all E with max subtraction, then the k largest probabilities,
+//   weights = those probabilities, divided by their sum if `renorm`
+//   (ferrox-moe/src/lib.rs:333-355).  Ties: higher probability first, then the
+//   lower expert index (the rule of ferrox-metal/src/gpu.rs:686-699).
+//   GATE_SIGMOID scores each expert with 1/(1+exp(-logit)) instead
+//   (ferrox-moe/src/lib.rs:100-121).
+//   gate_out[t] = sigmoid(sum_c x[c] * shared_gate[c])  (decoder.rs:2670-2672).
+template <typename T>
+__global__ __launch_bounds__(256) void router_topk_kernel(
+    const T* __restrict__ x, long ldx, const void* __restrict__ Wr, int w_dtype,
+    const void* __restrict__ shared_gate, int sg_dtype, int H, int E, int k, int renorm, int gating,
+    int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ gate_out) {
+    extern __shared__ float xs[];         // H floats
+    __shared__ float score[E_MAX];
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int c = tid; c < H; c += 256) xs[c] = to_float(x[(size_t)t * ldx + c]);
+    __syncthreads();
+    for (int e = wave; e < E; e += 4) {
+        float acc = 0.f;
+        for (int c = lane; c < H; c += 64) acc = fmaf(xs[c], load_as_float(Wr, w_dtype, (size_t)e * H + c), acc);
+        acc = wave_sum(acc);
+        if (lane == 0) score[e] = acc;
+    }
+    if (shared_gate) {
+        float acc = 0.f;
+        for (int c = tid; c < H; c += 256) acc = fmaf(xs[c], load_as_float(shared_gate, sg_dtype, c), acc);
+        acc = block_sum<4>(acc, red);
+        if (tid == 0) gate_out[t] = 1.0f / (1.0f + expf(-acc));
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // gating over all experts, by one wave
+    if (gating == GATE_SOFTMAX) {
+        float mx = NEG_INFINITY_F;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, score[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float ex = expf(score[e] - mx);
+            score[e] = ex;
+            sum += ex;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += 64) score[e] = score[e] / sum;
+    } else {
+        for (int e = lane; e < E; e += 64) score[e] = 1.0f / (1.0f + expf(-score[e]));
+    }
+    __builtin_amdgcn_wave_barrier();
+    // k rounds of "largest remaining", lower index on ties
+    float wsum = 0.f;
+    float my_w = 0.f;  // lane j keeps the weight of selection j
+    for (int j = 0; j < k; ++j) {
+        float best = -1.f;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float v = score[e];
+            if (v > best) {  // ascending e within a lane: the first maximum is kept
+                best = v;
+                bi = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ob > best || (ob == best && oi < bi)) {
+                best = ob;
+                bi = oi;
+            }
+        }
+        if (lane == j) my_w = best;
+        if (lane == 0) {
+            ids[t * k + j] = bi;
+            score[bi] = -2.f;  // scores are >= 0; taken out of the race
+        }
+        wsum += best;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    if (lane < k) weights[t * k + lane] = renorm ? my_w / wsum : my_w;
+}
+
+FX_API int fx_router_topk(void* stream, int x_dtype, const void* x, long ldx, const void* Wr, int w_dtype,
+                          const void* shared_gate, int sg_dtype, int T, int H, int E, int k, int renorm,
+                          int gating, int* ids, float* weights, float* gate_out) {
+    FX_REQUIRE(x_dtype == FX_F32 || x_dtype == FX_BF16, "router: unknown activation dtype %d", x_dtype);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "router: unknown weight dtype %d", w_dtype);
+    FX_REQUIRE(T >= 0 && H > 0, "router: bad sizes T=%d H=%d", T, H);
+    FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
+    FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
+    FX_REQUIRE(H <= 12288, "router: hidden size %d exceeds this kernel's 12288", H);
+    FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
+    FX_REQUIRE(!shared_gate || gate_out, "router: shared gate given without an output");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t shm = (size_t)H * sizeof(float);
+    if (x_dtype == FX_F32)
+        router_topk_kernel<float><<<T, 256, shm, s>>>((const float*)x, ldx, Wr, w_dtype, shared_gate, sg_dtype, H, E, k,
+                                                      renorm, gating, ids, weights, gate_out);
+    else
+        router_topk_kernel<bf16><<<T, 256, shm, s>>>((const bf16*)x, ldx, Wr, w_dtype, shared_gate, sg_dtype, H, E, k,
+                                                     renorm, gating, ids, weights, gate_out);
+    FX_CHECK_LAUNCH("router_topk");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Stable counting sort of n = T*k (token, slot) pairs by expert, one block.
+//   expert_offsets[E+1] : rows of expert e are [off[e], off[e+1])
+//   sorted_token[i]     : token of sorted row i
+//   inv[t*k + j]        : sorted row of pair (t, j)
+// Thread th owns the contiguous pairs [th*c, (th+1)*c) and counts them per
+// expert in its own row cnt[th][.]; thread e then turns column e into running
+// sums over th; a scan over the experts' totals gives the offsets; each thread
+// walks its pairs again and places them.  The order inside an expert is the
+// order of the pairs, whatever the number of threads.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E,
+                                                        int* __restrict__ expert_offsets,
+                                                        int* __restrict__ sorted_token, int* __restrict__ inv) {
+    extern __shared__ int lds[];
+    int* offs = lds;                              // E + 1
+    uint16_t* cnt = (uint16_t*)(lds + E + 1);     // [rows][E]
+    const int nt = blockDim.x, th = threadIdx.x;
+    const int c = max(1, (n + nt - 1) / nt);
+    const int rows = min(nt, (n + c - 1) / c);    // threads that own at least one pair
+    const int b = min(n, th * c), b_end = min(n, (th + 1) * c);
+    for (int i = th; i < rows * E; i += nt) cnt[i] = 0;
+    __syncthreads();
+    for (int i = b; i < b_end; ++i) {
+        const int e = ids[i];
+        if (e >= 0 && e < E) cnt[th * E + e] += 1;
+    }
+    __syncthreads();
+    for (int e = th; e < E; e += nt) {
+        int run = 0;
+        for (int r = 0; r < rows; ++r) {
+            const int v = cnt[r * E + e];
+            cnt[r * E + e] = (uint16_t)run;
+            run += v;
+        }
+        offs[e + 1] = run;  // total of expert e, scanned below
+    }
+    __syncthreads();
+    if (th == 0) {
+        int run = 0;
+        offs[0] = 0;
+        for (int e = 0; e < E; ++e) {
+            run += offs[e + 1];
+            offs[e + 1] = run;
+        }
+    }
+    __syncthreads();
+    for (int e = th; e <= E; e += nt) expert_offsets[e] = offs[e];
+    for (int i = b; i < b_end; ++i) {
+        const int e = ids[i];
+        if (e >= 0 && e < E) {
+            const int dst = offs[e] + cnt[th * E + e];
+            cnt[th * E + e] += 1;
+            sorted_token[dst] = i / k;
+            inv[i] = dst;
+        }
+    }
+}
+
+FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
+                        int* sorted_token, int* inv) {
+    FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
+    FX_REQUIRE(E >= 1, "moe_align: E=%d", E);
+    int nt = 256;
+    while (nt > 64 && (size_t)nt * E * 2 + (E + 1) * 4 > 48 * 1024) nt >>= 1;
+    const size_t shm = (size_t)nt * E * 2 + (E + 1) * 4;
+    FX_REQUIRE(shm <= 48 * 1024, "moe_align: %d experts exceed this kernel's limit of about 380", E);
+    FX_REQUIRE((n + nt - 1) / nt < 65536, "moe_align: %d pairs are too many for one block", n);
+    moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, expert_offsets, sorted_token, inv);
+    FX_CHECK_LAUNCH("moe_align");
+    return 0;
+}

@@ -1,0 +1,128 @@
+"""The Python entry point: an `Engine` over one model on one GPU.
+
+    engine = Engine("/path/to/model")                      # config.json + safetensors
+    engine = Engine(config=cfg_dict, random_weights=0)     # seeded random weights, no files
+    ids = engine.generate([[1, 2, 3]], max_new_tokens=16, temperature=0.0)
+
+Generation follows the reference's loop (ferrox-cli/src/run.rs:651-676,
+ferrox-server/src/batch_scheduler.rs:158-243): prefill, then sample -> append ->
+forward until EOS, the token limit or the context limit; here all requests share
+one continuously batched step.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+
+import torch
+
+from ..sampling.sampler import SamplingParams, sample_rows
+from .loading import load_model, parse_dtype, random_model
+from .runner import ModelRunner, StepEntry
+from .scheduler import Request, Scheduler
+
+
+@dataclass
+class Completion:
+    token_ids: list
+    finish_reason: str
+    n_prompt_tokens: int
+    n_preempted: int = 0
+
+
+class Engine:
+    def __init__(self, model_dir: str | None = None, *, config=None, random_weights: int | None = None,
+                 dtype="bfloat16", device="cuda:0", block_size: int = 64, num_pages: int | None = None,
+                 max_seqs: int = 64, max_tokens_per_step: int = 2048, prefill_chunk: int = 512,
+                 ctx_size: int = 0):
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; this engine has no CPU path")
+        self.dtype = parse_dtype(dtype)
+        if model_dir is not None:
+            self.model = load_model(model_dir, self.dtype, device)
+        elif config is not None and random_weights is not None:
+            self.model = random_model(config, int(random_weights), self.dtype, device)
+        else:
+            raise ValueError("give a model folder, or a configuration together with random_weights=<seed>")
+        spec = self.model.spec
+        self.context_limit = ctx_size if ctx_size > 0 else spec.max_positions      # run.rs:551-559
+        if num_pages is None:        # room for max_seqs requests of half the context each, at least one full
+            num_pages = max(-(-self.context_limit // block_size) + 1,
+                            max_seqs * (-(-self.context_limit // block_size)) // 2)
+        self.runner = ModelRunner(self.model, block_size=block_size, num_pages=num_pages, max_seqs=max_seqs)
+        self.max_seqs = max_seqs
+        self.max_tokens_per_step = max_tokens_per_step
+        self.prefill_chunk = prefill_chunk
+        self.eos_token_id = spec.eos_token_id
+        self.last_stats: dict = {}
+
+    @property
+    def vocab_size(self) -> int:
+        return self.model.spec.vocab_size
+
+    def step(self, entries: list):
+        """Direct access to the step function (entries are `StepEntry`s whose pages are reserved)."""
+        return self.runner.step(entries)
+
+    def generate(self, prompts: list, max_new_tokens: int = 128, temperature: float = 0.0, top_k: int = 0,
+                 top_p: float = 1.0, repetition_penalty: float = 1.0, presence_penalty: float = 0.0,
+                 frequency_penalty: float = 0.0, seed: int = 0, ignore_eos: bool = False,
+                 eos_token_id: int | None = None) -> list:
+        """Token ids generated for each prompt (a list of token ids), in order."""
+        return [c.token_ids for c in self.generate_detailed(
+            prompts, max_new_tokens, SamplingParams(temperature, top_k, top_p, repetition_penalty,
+                                                    presence_penalty, frequency_penalty, seed),
+            ignore_eos=ignore_eos, eos_token_id=eos_token_id)]
+
+    def generate_detailed(self, prompts: list, max_new_tokens, params: SamplingParams | list | None = None,
+                          ignore_eos: bool = False, eos_token_id: int | None = None) -> list:
+        """`params` may be one `SamplingParams` for all or one per prompt; `max_new_tokens` likewise.
+        Request i draws from a generator seeded with its own params.seed."""
+        eos = eos_token_id if eos_token_id is not None else self.eos_token_id
+        sched = Scheduler(self.runner, max_tokens_per_step=self.max_tokens_per_step,
+                          prefill_chunk=self.prefill_chunk, max_seqs=self.max_seqs,
+                          context_limit=self.context_limit, vocab_size=self.vocab_size)
+        reqs = []
+        for i, p in enumerate(prompts):
+            sp = params[i] if isinstance(params, (list, tuple)) else (params or SamplingParams())
+            mx = max_new_tokens[i] if isinstance(max_new_tokens, (list, tuple)) else max_new_tokens
+            if mx < 0:                                   # -1: fill the context (run.rs:609-614)
+                mx = self.context_limit - len(p)
+            mx = min(mx, self.context_limit - len(p))
+            r = Request(i, [int(t) for t in p], mx, SamplingParams(**vars(sp)), eos, ignore_eos)
+            reqs.append(r)
+            sched.add(r)
+        t0 = time.time()
+        n_steps = n_tokens = 0
+        try:
+            while sched.has_work():
+                batch = sched.schedule()
+                if not batch:
+                    if sched.has_work():
+                        raise RuntimeError("scheduler made no progress")
+                    break
+                entries = [StepEntry(s.request.id, sched.step_tokens(s), [s.n_tokens - 1] if s.samples else [])
+                           for s in batch]
+                logits = self.runner.step(entries)
+                sampled = {}
+                rows = [s.request for s in batch if s.samples]
+                if rows:
+                    toks = sample_rows(logits, [r.params for r in rows], [r.rng for r in rows],
+                                       [r.generated for r in rows])
+                    sampled = {r.id: t for r, t in zip(rows, toks)}
+                sched.commit(batch, sampled)
+                n_steps += 1
+                n_tokens += sum(s.n_tokens for s in batch)
+        finally:
+            for r in list(sched.running):
+                self.runner.release(r.id)
+        self.last_stats = {"steps": n_steps, "tokens": n_tokens, "seconds": time.time() - t0,
+                           "preemptions": sched.n_preemptions}
+        return [Completion(r.generated, r.finish_reason or "aborted", len(r.prompt), r.n_preempted) for r in reqs]
+
+
+def generate(model_dir: str, prompts: list, **kw) -> list:
+    """One-call form: load the model folder, generate, return the token ids."""
+    engine_kw = {k: kw.pop(k) for k in ("dtype", "device", "block_size", "num_pages", "max_seqs",
+                                        "max_tokens_per_step", "prefill_chunk", "ctx_size") if k in kw}
+    return Engine(model_dir, **engine_kw).generate(prompts, **kw)

@@ -1,0 +1,103 @@
+"""A model built from a `ModelSpec`: embedding, blocks, the order they run in,
+final norm and head.  It owns the weights; the cache belongs to the runner."""
+from __future__ import annotations
+
+import torch
+
+from ..parts.base import (BLOCKS, EMBEDDINGS, HEADS, NORMS, LayerCache, ModelSpec, StepContext, walk_params,
+                          walk_parts)
+from ..weights.loader import check_names, upload
+
+
+def group_key(mixer):
+    """Mixers with the same need share pages' ids: all keys, or the last W."""
+    return ("window", int(mixer.window)) if mixer.window else ("full",)
+
+
+class Model:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = EMBEDDINGS.build(spec.embedding)
+        self.blocks = []
+        for ls in spec.layers:
+            cls = BLOCKS.get(ls.block)
+            missing = set(cls.slots) - set(ls.parts)
+            if missing:
+                raise ValueError(f"layer {ls.prefix!r}: block '{ls.block}' needs parts {sorted(missing)}")
+            parts = {slot: reg.build(ls.parts[slot]) for slot, reg in cls.slots.items()}
+            self.blocks.append(cls(parts, {slot: ls.parts[slot].prefix for slot in cls.slots}))
+        self.final_norm = NORMS.build(spec.final_norm)
+        self.head = HEADS.build(spec.head)
+        self.schedule = list(spec.schedule)
+        for i, e in enumerate(self.schedule):
+            if not 0 <= e.layer < len(self.blocks):
+                raise ValueError(f"schedule entry {i} names layer {e.layer}; the model has {len(self.blocks)}")
+            if e.cache is not None:
+                if not 0 <= e.cache < i or self.schedule[e.cache].cache is not None:
+                    raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache}, which must be an "
+                                     f"earlier entry with a cache of its own")
+                a, b = self.blocks[e.layer].mixer, self.blocks[self.schedule[e.cache].layer].mixer
+                if group_key(a) != group_key(b) or a.page_shapes(16) != b.page_shapes(16):
+                    raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache}: "
+                                     f"their mixers keep different pages")
+        self.act_dtype = None
+        self.device = None
+
+    # ---- parameters ------------------------------------------------------
+    def _roots(self):
+        yield self.spec.embedding.prefix, self.embedding
+        for ls, block in zip(self.spec.layers, self.blocks):
+            yield ls.prefix, block
+        yield self.spec.final_norm.prefix, self.final_norm
+        yield self.spec.head.prefix, self.head
+
+    def named_params(self) -> dict:
+        out = {}
+        for prefix, root in self._roots():
+            for name, spec, _, _ in walk_params(root, prefix):
+                if name in out:
+                    raise ValueError(f"two parts claim the tensor '{name}'")
+                out[name] = spec
+        return out
+
+    def kernel_libraries(self) -> list:
+        libs = []
+        for prefix, root in self._roots():
+            for _, part in walk_parts(root, prefix):
+                for lib in part.kernel_libraries:
+                    if lib not in libs:
+                        libs.append(lib)
+        return libs
+
+    def load(self, source, act_dtype: torch.dtype, device, where: str = "") -> None:
+        """Check every name and shape first (one error for all), then upload part by part."""
+        if hasattr(source, "expect"):
+            source.expect(self.named_params())
+        check_names(self.named_params(), source, where)
+        device = torch.device(device)
+        for prefix, root in self._roots():
+            for pfx, part in walk_parts(root, prefix):
+                part.load(lambda local, _p=pfx: upload(source, _p + local, act_dtype, device))
+        if getattr(self.head, "tied", False):
+            self.head.tie(self.embedding)
+        self.act_dtype, self.device = act_dtype, device
+
+    # ---- cache needs -----------------------------------------------------
+    def cache_groups(self) -> dict:
+        """group key -> window, over the mixers that keep pages."""
+        groups = {}
+        for e in self.schedule:
+            m = self.blocks[e.layer].mixer
+            if m.page_shapes(16):
+                groups[group_key(m)] = m.window
+        return groups
+
+    # ---- forward ---------------------------------------------------------
+    def forward(self, ctx: StepContext, caches: list):
+        h = self.embedding.forward(ctx.token_ids)
+        for i, e in enumerate(self.schedule):
+            self.blocks[e.layer].forward(h, ctx, caches[i])
+        if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
+            return None
+        x = self.final_norm.forward(h, ctx, rows=ctx.logit_rows)
+        return self.head.forward(x)

@@ -1,0 +1,292 @@
+"""Python faces of the HIP kernels: argument checks, then one ctypes call.
+
+Tensors live on the GPU; the kernels run on torch's current stream.  There is no
+other implementation behind these functions: a tensor on the CPU, or a missing
+library, raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from .csrc.build import load_library
+
+FX_F32, FX_BF16 = 0, 1
+EPI_STORE, EPI_STORE_F32, EPI_RESID, EPI_SILU_MUL = 0, 1, 2, 3
+GATE_SOFTMAX, GATE_SIGMOID = 0, 1
+ROPE_NEOX, ROPE_INTERLEAVED = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return FX_F32
+    if dt == torch.bfloat16:
+        return FX_BF16
+    raise KernelError(f"kernels take float32 and bfloat16 tensors, not {dt}")
+
+
+def _p(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise KernelError("kernel called with a tensor that is not on the GPU")
+    return c_void_p(t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_sigs = {
+    ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
+    ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float],
+    ("elementwise", "fx_rope_kv_write"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float],
+    ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
+    ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
+    ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
+    ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
+    ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
+                          c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
+    ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
+                                     c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float],
+    ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
+                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                      c_int, c_int, c_int, c_int, c_int, c_float,
+                                      c_void_p, c_void_p, c_int, c_int],
+    ("moe", "fx_router_topk"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int,
+                                c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
+}
+_fns: dict = {}
+
+
+def _fn(lib: str, name: str):
+    key = (lib, name)
+    entry = _fns.get(key)
+    if entry is None:
+        handle = load_library(lib)
+        f = getattr(handle, name)
+        f.argtypes = _sigs[key]
+        f.restype = c_int
+        entry = _fns[key] = (f, handle)
+    return entry
+
+
+def _call(lib: str, name: str, *args) -> None:
+    f, handle = _fn(lib, name)
+    if f(*args):
+        raise KernelError(handle.fx_last_error().decode())
+
+
+def _i32(t, what):
+    if t is not None and t.dtype != torch.int32:
+        raise KernelError(f"{what} must be int32, got {t.dtype}")
+    return t
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """h[t] = table[ids[t]] as float32."""
+    V, H = table.shape
+    T = ids.numel()
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _call("elementwise", "fx_embed", _stream(), dtype_code(table.dtype), _p(table), _p(_i32(ids, "ids")), _p(out), T, H, V)
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rows of float32 `h` (all, or those in `rows`) normed into `out_dtype`."""
+    if h.dtype != torch.float32 or not h.is_contiguous():
+        raise KernelError("rmsnorm reads a contiguous float32 residual stream")
+    H = h.shape[-1]
+    if weight.numel() != H:
+        raise KernelError(f"rmsnorm weight has {weight.numel()} elements for width {H}")
+    R = h.shape[0] if rows is None else rows.numel()
+    if out is None:
+        out = torch.empty((R, H), dtype=out_dtype, device=h.device)
+    _call("elementwise", "fx_rmsnorm", _stream(), dtype_code(out_dtype), _p(h), _p(_i32(rows, "rows")), _p(weight),
+          dtype_code(weight.dtype), _p(out), R, H, float(eps))
+    return out
+
+
+def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads,
+                  head_dim, block_size, rotary_dim, theta, interleaved=False) -> None:
+    """Rotate q in place; rotate k and write it and v into the pages (skipped when k_pages is None).
+    q, k, v are 2-D views [T, heads*head_dim] with unit inner stride."""
+    T = q.shape[0]
+    for t in (q, k, v):
+        if t.stride(-1) != 1 or t.dtype != q.dtype:
+            raise KernelError("rope_kv_write wants q, k, v of one dtype with unit inner stride")
+    if k_pages is not None:
+        if k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+            raise KernelError("cache pages and activations differ in dtype")
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (n_kv_heads, head_dim, block_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_pages.shape)}, {tuple(v_pages.shape)}; expected "
+                              f"[pages,{n_kv_heads},{block_size},{head_dim}] and [pages,{n_kv_heads},{head_dim},{block_size}]")
+    _call("elementwise", "fx_rope_kv_write", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(k), k.stride(0),
+          _p(v), v.stride(0), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
+          _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
+          _p(k_pages), _p(v_pages), T, n_heads, n_kv_heads, head_dim, block_size, rotary_dim,
+          1 if interleaved else 0, float(theta))
+
+
+def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:
+    """h += y, summed in float32."""
+    if h.dtype != torch.float32 or h.shape != y.shape or not h.is_contiguous() or not y.is_contiguous():
+        raise KernelError("residual_add wants a contiguous float32 h and a y of the same shape")
+    _call("elementwise", "fx_residual_add", _stream(), dtype_code(y.dtype), _p(h), _p(y), h.numel())
+
+
+def cast(src: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    if src.dtype == dtype:
+        return src
+    src = src.contiguous()
+    dst = torch.empty(src.shape, dtype=dtype, device=src.device)
+    _call("elementwise", "fx_cast", _stream(), dtype_code(src.dtype), _p(src), dtype_code(dtype), _p(dst), src.numel())
+    return dst
+
+
+def fill_u32(t: torch.Tensor, value: int = 0) -> None:
+    if not t.is_contiguous() or t.element_size() * t.numel() % 4:
+        raise KernelError("fill_u32 wants a contiguous buffer of whole 32-bit words")
+    _call("elementwise", "fx_fill_u32", _stream(), _p(t), value, t.element_size() * t.numel() // 4)
+
+
+def moe_combine(h, y_sorted, inv, weights, top_k) -> None:
+    """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]]."""
+    T, H = h.shape
+    if y_sorted.dtype != torch.float32 or h.dtype != torch.float32:
+        raise KernelError("moe_combine works on float32")
+    _call("elementwise", "fx_moe_combine", _stream(), _p(h), _p(y_sorted), _p(_i32(inv, "inv")), _p(weights), T, H, top_k)
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: torch.Tensor | None = None,
+         bias: torch.Tensor | None = None, row_scale: torch.Tensor | None = None,
+         a_rows: torch.Tensor | None = None, expert_offsets: torch.Tensor | None = None,
+         n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0) -> torch.Tensor:
+    """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
+
+    `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
+    EPI_STORE stores in a's dtype (+bias); EPI_STORE_F32 stores float32; EPI_RESID adds the
+    product (times row_scale[m]) into the float32 `out`; EPI_SILU_MUL multiplies two
+    matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores silu(gate)*up.
+    `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.
+    """
+    if a.dtype != w.dtype:
+        raise KernelError(f"gemm: activations are {a.dtype}, weights {w.dtype}")
+    if a.dim() != 2 or a.stride(1) != 1:
+        raise KernelError("gemm: activations must be 2-D with unit inner stride")
+    if not w.is_contiguous():
+        raise KernelError("gemm: weights must be contiguous")
+    K = a.shape[1]
+    grouped = expert_offsets is not None
+    if grouped:
+        if w.dim() != 3:
+            raise KernelError("gemm: grouped weights must be [E, N, K]")
+        E, n_w, kw = w.shape
+        w_stride = n_w * kw
+    else:
+        if w.dim() != 2:
+            raise KernelError("gemm: weights must be [N, K]")
+        E, (n_w, kw), w_stride = 0, w.shape, 0
+    if kw != K:
+        raise KernelError(f"gemm: inner sizes differ, activations {K}, weights {kw}")
+    M = n_rows if n_rows is not None else a.shape[0]
+    if epilogue == EPI_SILU_MUL:
+        N = n_out if n_out is not None else n_w // 2
+        if up_offset == 0:
+            up_offset = N * K
+        if up_offset // K + N > n_w:
+            raise KernelError("gemm: gate/up rows exceed the weight matrix")
+    else:
+        N = n_out if n_out is not None else n_w
+    out_dtype = a.dtype if epilogue in (EPI_STORE, EPI_SILU_MUL) else torch.float32
+    if out is None:
+        if epilogue == EPI_RESID:
+            raise KernelError("gemm: the residual epilogue needs `out`")
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if out.dtype != out_dtype or out.dim() != 2 or out.stride(1) != 1 or out.shape[0] < M or out.shape[1] < N:
+        raise KernelError(f"gemm: output {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {out_dtype}")
+    if bias is not None and bias.numel() != N:
+        raise KernelError(f"gemm: bias has {bias.numel()} elements for {N} columns")
+    _call("gemm", "fx_gemm", _stream(), dtype_code(a.dtype), epilogue, _p(a), a.stride(0), _p(w), w_stride, up_offset,
+          _p(bias), dtype_code(bias.dtype) if bias is not None else 0, _p(out), out.stride(0),
+          _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K)
+    return out
+
+
+def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
+                    n_heads, n_kv_heads, head_dim, block_size, window, scale) -> None:
+    _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
+          _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
+          _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
+          _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
+          int(window or 0), float(scale))
+
+
+def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
+                     n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=256) -> None:
+    n = item_seq.numel()
+    splits = max(1, -(-max_kv_len // chunk))
+    part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((n, n_heads, splits, 2), dtype=torch.float32, device=q.device)
+    _call("attention", "fx_attn_decode", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
+          _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
+          _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")), n,
+          n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
+          _p(part_o), _p(part_ml), splits, chunk)
+
+
+def router_topk(x, router_w, top_k, renorm, gating=GATE_SOFTMAX, shared_gate=None):
+    """Returns (ids int32 [T,k], weights float32 [T,k], gate float32 [T] or None)."""
+    T, H = x.shape
+    E = router_w.shape[0]
+    if router_w.shape[1] != H or not router_w.is_contiguous() or x.stride(1) != 1:
+        raise KernelError("router: weight must be contiguous [E, H] and x [T, H]")
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=x.device)
+    weights = torch.empty((T, top_k), dtype=torch.float32, device=x.device)
+    gate = torch.empty((T,), dtype=torch.float32, device=x.device) if shared_gate is not None else None
+    _call("moe", "fx_router_topk", _stream(), dtype_code(x.dtype), _p(x), x.stride(0), _p(router_w),
+          dtype_code(router_w.dtype), _p(shared_gate), dtype_code(shared_gate.dtype) if shared_gate is not None else 0,
+          T, H, E, top_k, 1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
+    return ids, weights, gate
+
+
+def moe_align(ids: torch.Tensor, n_experts: int):
+    """Returns (expert_offsets [E+1], sorted_token [n], inv [n]) for ids [T, k]."""
+    T, k = ids.shape
+    n = T * k
+    dev = ids.device
+    offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
+    sorted_token = torch.empty((n,), dtype=torch.int32, device=dev)
+    inv = torch.empty((n,), dtype=torch.int32, device=dev)
+    _call("moe", "fx_moe_align", _stream(), _p(_i32(ids, "ids")), n, k, n_experts, _p(offsets), _p(sorted_token), _p(inv))
+    return offsets, sorted_token, inv
+
+
+def sample(logits: torch.Tensor, *, temperature=None, draw=None, top_k=None, top_p=None, rep_penalty=None,
+           presence=None, frequency=None, hist=None, hist_start=None) -> torch.Tensor:
+    """One token per row of float32 logits [R, V]; all per-row parameters are device tensors or None
+    (None: greedy / option off)."""
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be float32 [R, V] with unit inner stride")
+    R, V = logits.shape
+    work = torch.empty((R, V), dtype=torch.float32, device=logits.device)
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _call("sampling", "fx_sample", _stream(), _p(logits), logits.stride(0), _p(work), R, V,
+          _p(temperature), _p(_i32(top_k, "top_k")), _p(top_p), _p(rep_penalty), _p(presence), _p(frequency),
+          _p(draw), _p(_i32(hist, "hist")), _p(_i32(hist_start, "hist_start")), _p(out))
+    return out

@@ -1,0 +1,114 @@
+"""Causal grouped-query attention over the paged cache.
+
+Per token (ferrox-models/src/decoder.rs:3224-3560): q, k, v = W x + b, the bias
+added before the rotation; q and k rotated by the position encoding; k and v
+written into the pages; the query attends to its sequence's pages (its own
+position included, through the cache just written); the heads' outputs go
+through o_proj (no bias) into the residual stream.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import ops
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec
+from .linear import Linear, same_dtype
+
+TILE_Q = 16   # queries per work item of the tiled kernel
+
+
+def attention_items(ctx):
+    """Work items of a step, shared by all attention layers: sequences with one
+    new token go to the split decode kernel, the others are cut into tiles of
+    TILE_Q consecutive queries."""
+    dec_seq, dec_tok, t_seq, t_tok, t_n = [], [], [], [], []
+    max_kv = 1
+    for s in range(ctx.n_seqs):
+        b, e = ctx.q_starts[s], ctx.q_starts[s + 1]
+        if e - b == 1:
+            dec_seq.append(s)
+            dec_tok.append(b)
+            max_kv = max(max_kv, ctx.kv_lens[s])
+        else:
+            for t0 in range(b, e, TILE_Q):
+                t_seq.append(s)
+                t_tok.append(t0)
+                t_n.append(min(TILE_Q, e - t0))
+    flat = dec_seq + dec_tok + t_seq + t_tok + t_n
+    dev = torch.tensor(flat, dtype=torch.int32, device=ctx.device) if flat else None
+    nd, nt = len(dec_seq), len(t_seq)
+    items = {"n_decode": nd, "n_tiles": nt, "max_kv": max_kv}
+    if nd:
+        items["dec_seq"], items["dec_tok"] = dev[:nd], dev[nd:2 * nd]
+    if nt:
+        o = 2 * nd
+        items["tile_seq"], items["tile_tok"], items["tile_n"] = dev[o:o + nt], dev[o + nt:o + 2 * nt], dev[o + 2 * nt:]
+    return items
+
+
+@MIXERS.register("paged_attention")
+class PagedAttention(Mixer):
+    kernel_libraries = ("elementwise", "gemm", "attention")
+
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, bias: bool,
+                 position: PartSpec, window: int | None = None, scale: float | None = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError(f"head_dim {head_dim}: the attention kernels take multiples of 16 from 16 to 256")
+        self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
+        self.bias = bool(bias)
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # attention.rs:433
+        self.position = POSITION_ENCODINGS.build(position)
+        self.qw, self.kvw = n_heads * head_dim, n_kv_heads * head_dim
+        self.qkv = self.o_proj = None
+
+    def children(self):
+        return [("", self.position)]
+
+    def param_specs(self):
+        H = self.hidden_size
+        specs = {"q_proj.weight": ParamSpec((self.qw, H)), "k_proj.weight": ParamSpec((self.kvw, H)),
+                 "v_proj.weight": ParamSpec((self.kvw, H)), "o_proj.weight": ParamSpec((H, self.qw))}
+        if self.bias:
+            specs.update({"q_proj.bias": ParamSpec((self.qw,)), "k_proj.bias": ParamSpec((self.kvw,)),
+                          "v_proj.bias": ParamSpec((self.kvw,))})
+        return specs
+
+    def load(self, fetch):
+        w = torch.cat(same_dtype([fetch("q_proj.weight"), fetch("k_proj.weight"), fetch("v_proj.weight")]), dim=0)
+        b = None
+        if self.bias:
+            b = torch.cat(same_dtype([fetch("q_proj.bias"), fetch("k_proj.bias"), fetch("v_proj.bias")]), dim=0)
+        self.qkv = Linear(w, b)
+        self.o_proj = Linear(fetch("o_proj.weight"))
+
+    def page_shapes(self, block_size: int) -> dict:
+        return {"k": (self.n_kv_heads, block_size, self.head_dim),
+                "v": (self.n_kv_heads, self.head_dim, block_size)}
+
+    def forward(self, x, ctx, cache, residual) -> None:
+        qkv = self.qkv(x)
+        q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
+        table = ctx.block_tables[cache.group]
+        k_pages, v_pages = cache.pages["k"], cache.pages["v"]
+        rot = self.position.rotary()
+        if rot is None:
+            self.position.apply(q, k, ctx)
+            rot = (0, 1.0, False)
+        ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
+                          k_pages if cache.writes else None, v_pages if cache.writes else None,
+                          self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1], rot[2])
+        out = torch.empty((ctx.n_tokens, self.qw), dtype=x.dtype, device=x.device)
+        items = ctx.memo("attention_items", lambda: attention_items(ctx))
+        common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
+        if items["n_tiles"]:
+            ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
+                                items["tile_seq"], items["tile_tok"], items["tile_n"], *common)
+        if items["n_decode"]:
+            ops.attention_decode(q, out, k_pages, v_pages, table, ctx.positions,
+                                 items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"])
+        self.o_proj(out, epilogue=ops.EPI_RESID, out=residual)

@@ -1,0 +1,234 @@
+"""What a model is put together from, and the registries the parts are found in.
+
+A model is data: a `ModelSpec` lists an embedding, layers (each a block made of
+a mixer, a feed-forward and norms, every one a `PartSpec` = kind + arguments),
+the order in which the layers run (`schedule`), a final norm and a head.  The
+builder looks each kind up in a registry and constructs it from its arguments;
+no part knows which model it is in.  Another part becomes available by
+registering a class under a new kind; nothing else changes.
+
+Interfaces (all tensors on the GPU; `h` is the float32 residual stream [T, H],
+`x` an activation [T, H] in `ctx.act_dtype`):
+
+  Norm             forward(h, ctx, rows=None) -> x
+  PositionEncoding rotary() -> (rotary_dim, theta, interleaved) when the attention
+                   kernels can apply it themselves, else None and
+                   apply(q, k, ctx) -> None rotates q [T, nh*hd], k [T, nkv*hd] in place
+  Mixer            window (None or int), page_shapes(block_size) -> {name: shape},
+                   state_shapes() -> {name: (shape, dtype)},
+                   forward(x, ctx, cache, residual) -> None   (adds its output into residual)
+  FeedForward      forward(x, ctx, residual) -> None
+  Block            forward(h, ctx, cache) -> None
+  every part       param_specs() -> {local name: ParamSpec}, load(fetch), kernel_libraries
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable
+
+import torch
+
+
+# --------------------------------------------------------------------------
+# specs: the data a model is described with
+# --------------------------------------------------------------------------
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: tuple
+    init: str = "normal"      # 'normal' (std from the writer), 'ones', 'zeros'
+    integer: bool = False     # integer tables are kept as int32
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    args: dict = field(default_factory=dict)
+    prefix: str = ""          # joined to the owner's prefix to form tensor names
+
+
+@dataclass
+class LayerSpec:
+    block: str                # kind of block, e.g. 'prenorm'
+    prefix: str               # e.g. 'model.layers.3.'
+    parts: dict               # slot name -> PartSpec
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    layer: int                # index into ModelSpec.layers; a layer may be named twice
+    cache: int | None = None  # None: a cache of this entry's own; j: read the cache of entry j
+
+
+@dataclass
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    embedding: PartSpec
+    layers: list
+    schedule: list
+    final_norm: PartSpec
+    head: PartSpec
+    max_positions: int
+    eos_token_id: int | None = None
+
+
+# --------------------------------------------------------------------------
+# registries
+# --------------------------------------------------------------------------
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: dict[str, type] = {}
+
+    def register(self, kind: str):
+        def deco(cls):
+            self._items[kind] = cls
+            cls.kind = kind
+            return cls
+        return deco
+
+    def build(self, spec: PartSpec, **extra):
+        cls = self._items.get(spec.kind)
+        if cls is None:
+            raise KeyError(f"no {self.what} of kind '{spec.kind}' is registered "
+                           f"(known: {', '.join(sorted(self._items)) or 'none'})")
+        return cls(**spec.args, **extra)
+
+    def get(self, kind: str) -> type:
+        if kind not in self._items:
+            raise KeyError(f"no {self.what} of kind '{kind}' is registered "
+                           f"(known: {', '.join(sorted(self._items)) or 'none'})")
+        return self._items[kind]
+
+    def __contains__(self, kind):
+        return kind in self._items
+
+    def kinds(self):
+        return sorted(self._items)
+
+
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")
+
+
+# --------------------------------------------------------------------------
+# what a step hands to the parts
+# --------------------------------------------------------------------------
+@dataclass
+class StepContext:
+    """One batch of (request, its next tokens), flattened.
+
+    Token t belongs to sequence token_seq[t] (a row of the block tables and of
+    slot_ids) and stands at positions[t].  Sequence s owns tokens
+    [q_starts[s], q_starts[s+1]) and holds kv_lens[s] positions after the step.
+    """
+    n_tokens: int
+    n_seqs: int
+    act_dtype: torch.dtype
+    device: torch.device
+    token_ids: torch.Tensor            # int32 [T]
+    positions: torch.Tensor            # int32 [T]
+    token_seq: torch.Tensor            # int32 [T]
+    q_starts: list                     # host, n_seqs + 1
+    kv_lens: list                      # host, n_seqs
+    slot_ids: torch.Tensor             # int32 [n_seqs]
+    slots: list                        # host copy
+    block_tables: dict                 # group key -> int32 [n_seqs, max_blocks]
+    block_size: int
+    logit_rows: torch.Tensor | None = None   # int32 [R] token indices whose logits are wanted
+    _memo: dict = field(default_factory=dict)
+
+    def memo(self, key, make: Callable):
+        """Per-step data that several layers share (built by the first that asks)."""
+        if key not in self._memo:
+            self._memo[key] = make()
+        return self._memo[key]
+
+    def q_len(self, s: int) -> int:
+        return self.q_starts[s + 1] - self.q_starts[s]
+
+
+@dataclass
+class LayerCache:
+    """The part of the cache one schedule entry sees."""
+    pages: dict                        # name -> [num_pages, *page_shape]
+    state: dict                        # name -> [n_slots, *state_shape]
+    group: object                      # key into ctx.block_tables (None if the mixer has no pages)
+    block_size: int
+    writes: bool = True                # False: the pages belong to another entry, read only
+
+
+# --------------------------------------------------------------------------
+# base classes
+# --------------------------------------------------------------------------
+class Part:
+    kernel_libraries: tuple = ()
+
+    def param_specs(self) -> dict:
+        return {}
+
+    def load(self, fetch: Callable[[str], torch.Tensor]) -> None:
+        """`fetch(local name)` returns the tensor on the device.  Floating tensors come
+        in the activation type, except those stored in float32, which stay float32."""
+
+    def children(self) -> list:
+        """Sub-parts as [(prefix, part)]; a child's tensors are named prefix + its local names."""
+        return []
+
+
+def walk_params(part: "Part", prefix: str = ""):
+    """Yields (full tensor name, ParamSpec, owning part, local name) of a part and its children."""
+    for local, spec in part.param_specs().items():
+        yield prefix + local, spec, part, local
+    for child_prefix, child in part.children():
+        yield from walk_params(child, prefix + child_prefix)
+
+
+def walk_parts(part: "Part", prefix: str = ""):
+    """Yields (prefix, part) for a part and its children."""
+    yield prefix, part
+    for child_prefix, child in part.children():
+        yield from walk_parts(child, prefix + child_prefix)
+
+
+class Norm(Part):
+    def forward(self, h, ctx: StepContext, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary(self):
+        return None
+
+    def apply(self, q, k, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    window: int | None = None
+
+    def page_shapes(self, block_size: int) -> dict:
+        return {}
+
+    def state_shapes(self) -> dict:
+        return {}
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, residual) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, ctx: StepContext, residual) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, h, ctx: StepContext, cache: LayerCache) -> None:
+        raise NotImplementedError

@@ -1,0 +1,31 @@
+"""Dense gated feed-forward: down( silu(gate x) * (up x) )
+(ferrox-moe/src/lib.rs:655-658; dense layers: ferrox-models/src/decoder.rs:2902-2913)."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import FEED_FORWARDS, FeedForward, ParamSpec
+from .linear import Linear, same_dtype
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    kernel_libraries = ("gemm",)
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.gate_up = self.down = None
+
+    def param_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        return {"gate_proj.weight": ParamSpec((I, H)), "up_proj.weight": ParamSpec((I, H)),
+                "down_proj.weight": ParamSpec((H, I))}
+
+    def load(self, fetch):
+        self.gate_up = Linear(torch.cat(same_dtype([fetch("gate_proj.weight"), fetch("up_proj.weight")]), dim=0))
+        self.down = Linear(fetch("down_proj.weight"))
+
+    def forward(self, x, ctx, residual, row_scale=None) -> None:
+        act = self.gate_up(x, epilogue=ops.EPI_SILU_MUL)
+        self.down(act, epilogue=ops.EPI_RESID, out=residual, row_scale=row_scale)

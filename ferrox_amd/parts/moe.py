@@ -1,0 +1,76 @@
+"""Sparse mixture of experts with an optional gated shared expert.
+
+Per token (ferrox-models/src/decoder.rs:2895-2924, 2567-2682): router logits
+r = W_r x; a gating function over all experts and the k best of them
+(ferrox-moe/src/lib.rs:333-355); each chosen expert is a gated feed-forward
+(lib.rs:655-658); their outputs are summed with the routing weights in selection
+order (lib.rs:735-745); a shared expert, scaled by sigmoid(w_g . x), is added
+(decoder.rs:2660-2679).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import FEED_FORWARDS, FeedForward, ParamSpec
+from .linear import matmul, same_dtype
+from .mlp import SwiGLU
+
+GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
+
+
+@FEED_FORWARDS.register("sparse_moe")
+class SparseMoE(FeedForward):
+    kernel_libraries = ("elementwise", "gemm", "moe")
+
+    def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
+                 norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
+                 shared_gate: bool = True):
+        if not 1 <= top_k <= n_experts:
+            raise ValueError(f"top_k {top_k} must lie in 1..{n_experts}")
+        if gating not in GATINGS:
+            raise ValueError(f"gating '{gating}' is not one of {sorted(GATINGS)}")
+        self.hidden_size, self.n_experts, self.top_k = int(hidden_size), int(n_experts), int(top_k)
+        self.expert_intermediate_size = int(expert_intermediate_size)
+        self.norm_topk_prob, self.gating = bool(norm_topk_prob), GATINGS[gating]
+        self.shared = SwiGLU(hidden_size, shared_intermediate_size) if shared_intermediate_size > 0 else None
+        self.has_shared_gate = bool(shared_gate) and self.shared is not None
+        self.router = self.w_gate_up = self.w_down = self.shared_gate_w = None
+
+    def children(self):
+        return [("shared_expert.", self.shared)] if self.shared is not None else []
+
+    def param_specs(self):
+        H, I = self.hidden_size, self.expert_intermediate_size
+        specs = {"gate.weight": ParamSpec((self.n_experts, H))}
+        for e in range(self.n_experts):
+            specs[f"experts.{e}.gate_proj.weight"] = ParamSpec((I, H))
+            specs[f"experts.{e}.up_proj.weight"] = ParamSpec((I, H))
+            specs[f"experts.{e}.down_proj.weight"] = ParamSpec((H, I))
+        if self.has_shared_gate:
+            specs["shared_expert_gate.weight"] = ParamSpec((1, H))
+        return specs
+
+    def load(self, fetch):
+        self.router = fetch("gate.weight").contiguous()
+        gu, dn = [], []
+        for e in range(self.n_experts):
+            gu.append(torch.cat(same_dtype([fetch(f"experts.{e}.gate_proj.weight"),
+                                            fetch(f"experts.{e}.up_proj.weight")]), dim=0))
+            dn.append(fetch(f"experts.{e}.down_proj.weight"))
+        self.w_gate_up = torch.stack(same_dtype(gu)).contiguous()     # [E, 2*I, H]
+        self.w_down = torch.stack(same_dtype(dn)).contiguous()        # [E, H, I]
+        if self.has_shared_gate:
+            self.shared_gate_w = fetch("shared_expert_gate.weight").reshape(-1).contiguous()
+
+    def forward(self, x, ctx, residual) -> None:
+        T = x.shape[0]
+        ids, weights, gate = ops.router_topk(x, self.router, self.top_k, self.norm_topk_prob, self.gating,
+                                             self.shared_gate_w)
+        offsets, sorted_token, inv = ops.moe_align(ids, self.n_experts)
+        act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
+                     expert_offsets=offsets, n_rows=T * self.top_k)
+        y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets)
+        ops.moe_combine(residual, y, inv, weights, self.top_k)
+        if self.shared is not None:
+            self.shared.forward(x, ctx, residual, row_scale=gate)

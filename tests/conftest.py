@@ -1,0 +1,63 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+# Two tiny configurations that differ in every size and option.
+TINY_A = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 4,
+    "num_experts": 8, "num_experts_per_tok": 2, "norm_topk_prob": False, "moe_intermediate_size": 32,
+    "shared_expert_intermediate_size": 96, "intermediate_size": 128, "decoder_sparse_step": 1,
+    "mlp_only_layers": [], "vocab_size": 256, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 128, "use_sliding_window": False, "sliding_window": 32768,
+    "max_window_layers": 2, "tie_word_embeddings": False,
+}
+TINY_B = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 3, "hidden_size": 96, "num_attention_heads": 3, "num_key_value_heads": 1,
+    "num_experts": 6, "num_experts_per_tok": 3, "norm_topk_prob": True, "moe_intermediate_size": 48,
+    "shared_expert_intermediate_size": 64, "intermediate_size": 160, "decoder_sparse_step": 2,
+    "mlp_only_layers": [0], "vocab_size": 384, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
+    "max_position_embeddings": 256, "use_sliding_window": True, "sliding_window": 16,
+    "max_window_layers": 1, "tie_word_embeddings": True,
+}
+# a third one: GQA with groups of 2, head_dim 48, widths that are no power of two
+TINY_C = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 2, "hidden_size": 120, "num_attention_heads": 6, "num_key_value_heads": 3,
+    "head_dim": 48, "num_experts": 5, "num_experts_per_tok": 1, "norm_topk_prob": True,
+    "moe_intermediate_size": 40, "shared_expert_intermediate_size": 0, "intermediate_size": 72,
+    "decoder_sparse_step": 1, "mlp_only_layers": [1], "vocab_size": 331, "rope_theta": 50000.0,
+    "rms_norm_eps": 3e-6, "max_position_embeddings": 512, "use_sliding_window": True, "sliding_window": 40,
+    "max_window_layers": 0, "tie_word_embeddings": False,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+
+
+@pytest.fixture(scope="session")
+def model_folders(tmp_path_factory):
+    """name, dtype -> folder with config.json and model.safetensors (made once a session)."""
+    made = {}
+
+    def get(name: str, dtype: str = "float32") -> str:
+        key = (name, dtype)
+        if key not in made:
+            from ferrox_amd.engine.loading import write_random_model
+            cfg, seed = TINY[name]
+            folder = str(tmp_path_factory.mktemp(f"tiny{name}_{dtype}"))
+            write_random_model(dict(cfg), folder, seed, dtype)
+            made[key] = folder
+        return made[key]
+
+    return get

@@ -1,0 +1,135 @@
+"""The engine against the plain implementation, on the GPU: the same requests whole, with the
+last 32 tokens decoded one by one, in portions of changing size, and mixed with other requests
+under a pool so small that pages are used again; in float32 and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import replay_util as ru
+from conftest import ROOT, TINY
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [1, 7, 16, 33, 70, 45], "B": [3, 17, 40, 64, 90, 120], "C": [2, 35, 66, 130, 51]}
+# float32: the engine differs from a float64 computation by float32 rounding only.
+# bfloat16: weights are the same bfloat16 values on both sides; activations are rounded to 8 bits
+# of mantissa at every matrix product, and logits are of the order 0.1 .. 0.5.
+TOL = {"float32": (2e-5, 1e-4), "bfloat16": (2e-2, 2e-2)}
+
+_runners = {}
+
+
+def runner_for(model_folders, name, dtype, block_size, num_pages):
+    from ferrox_amd.engine.loading import load_model
+    from ferrox_amd.engine.runner import ModelRunner
+    folder = model_folders(name, dtype)
+    key = (name, dtype)
+    if key not in _runners:
+        _runners[key] = load_model(folder, dtype, "cuda:0")
+    return folder, ModelRunner(_runners[key], block_size=block_size, num_pages=num_pages, max_seqs=4)
+
+
+def requests_for(name):
+    cfg, seed = TINY[name]
+    return ru.make_requests(cfg["vocab_size"], LENGTHS[name], 100 + seed)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_prompts(model_folders, name, dtype):
+    folder, runner = runner_for(model_folders, name, dtype, block_size=16, num_pages=16)
+    reqs = requests_for(name)
+    got = ru.run_trace(runner, ru.trace_whole(reqs))
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_tokens_one_by_one(model_folders, name, dtype):
+    folder, runner = runner_for(model_folders, name, dtype, block_size=8, num_pages=24)
+    reqs = requests_for(name)
+    got = ru.run_trace(runner, ru.trace_tail_decode(reqs))
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} tail-decode")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(model_folders, name, dtype):
+    folder, runner = runner_for(model_folders, name, dtype, block_size=8, num_pages=24)
+    reqs = requests_for(name)
+    got = ru.run_trace(runner, ru.trace_portions(reqs))
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_page_reuse(model_folders, name, dtype):
+    reqs = requests_for(name)
+    steps = ru.trace_mixed(reqs, seed=7)
+    bs = 8
+    pages = ru.max_live_tokens(steps, bs) // bs          # exactly what the live requests need
+    folder, runner = runner_for(model_folders, name, dtype, block_size=bs, num_pages=pages)
+    got = ru.run_trace(runner, steps)
+    assert runner.manager.n_free_pages() == pages
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} mixed")
+
+
+@pytest.mark.parametrize("dtype", ["float32"])
+def test_cuts_agree_bitwise_in_float32(model_folders, dtype):
+    """Beyond closeness to the plain model: float32 logits of a position are the same bits however
+    the tokens were cut, except where single tokens go through the split decode kernel."""
+    folder, runner = runner_for(model_folders, "B", dtype, block_size=8, num_pages=40)
+    reqs = requests_for("B")
+    a = ru.run_trace(runner, ru.trace_whole(reqs))
+    b = ru.run_trace(runner, ru.trace_portions(reqs))
+    for key in a:
+        assert torch.equal(a[key], b[key]), f"position {key}: whole and portions differ in float32"
+
+
+def test_trace_run_program(model_folders, tmp_path):
+    """bin/trace_run as a user runs it: steps on stdin, `done <step>` lines, <step>.f32 files."""
+    folder = model_folders("B", "float32")
+    reqs = requests_for("B")
+    steps = ru.trace_mixed(reqs, seed=3)
+    for i, st in enumerate(steps):
+        st["step"] = i
+    out = tmp_path / "logits"
+    n_tokens = ru.max_live_tokens(steps, 64)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype",
+                           "float32", "--out", str(out), "--max-tokens", str(n_tokens)],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                          timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    import numpy as np
+    vocab = TINY["B"][0]["vocab_size"]
+    got, pos = {}, {}
+    for st in steps:
+        arr = np.fromfile(out / f"{st['step']}.f32", dtype="<f4").reshape(-1, vocab)
+        row = 0
+        for e in st["entries"]:
+            pos.setdefault(e["id"], 0)
+            for w in e["want"]:
+                got[(e["id"], pos[e["id"]] + w)] = torch.from_numpy(arr[row].copy())
+                row += 1
+            pos[e["id"]] += len(e["tokens"])
+        assert row == arr.shape[0]
+    ru.compare(got, folder, reqs, *TOL["float32"], "trace_run B float32 mixed")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(model_folders, name):
+    import plain_qwen2moe as plain
+    from ferrox_amd.engine.api import Engine
+    folder = model_folders(name, "float32")
+    cfg, w = plain.load_folder(folder)
+    prompts = list(ru.make_requests(cfg["vocab_size"], [1, 7, 16, 33], 5).values())
+    engine = Engine(folder, dtype="float32", block_size=16, num_pages=24, max_seqs=4,
+                    max_tokens_per_step=32, prefill_chunk=24)
+    got = engine.generate(prompts, max_new_tokens=16, temperature=0.0)
+    for p, g in zip(prompts, got):
+        assert g == plain.greedy_generate(cfg, w, p, 16)

@@ -1,0 +1,247 @@
+"""Each kernel alone against a plain float64 reference, at sizes other than the engine's."""
+import math
+import random
+
+import pytest
+import torch
+
+import plain_qwen2moe as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, dtype, what, k=1):
+    """float32: rounding of sums of k products; bfloat16: inputs are exact, the output is rounded once."""
+    got, want = got.double().cpu(), want.double().cpu()
+    scale = float(want.abs().max()) + 1e-30
+    tol = (1e-5 if dtype == torch.float32 else 1e-2) * scale
+    err = float((got - want).abs().max())
+    assert err <= tol, f"{what}: max error {err:.3e} > {tol:.3e} (scale {scale:.3e})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 100, 96), (16, 256, 128), (17, 257, 200), (33, 72, 40),
+                                    (64, 64, 64), (130, 300, 520), (257, 129, 1032), (3, 50, 100)])
+def test_gemm_plain_and_epilogues(dtype, M, N, K):
+    from ferrox_amd import ops
+    a, w = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1)
+    bias = rnd(N, dtype=dtype, seed=2)
+    ref = a.double() @ w.double().T
+    close(ops.gemm(a, w), ref, dtype, "store")
+    close(ops.gemm(a, w, bias=bias), ref + bias.double(), dtype, "store+bias")
+    close(ops.gemm(a, w, epilogue=ops.EPI_STORE_F32, bias=bias), ref + bias.double(), torch.float32 if dtype == torch.float32 else dtype, "f32 store")
+    h = rnd(M, N, seed=3)
+    h0 = h.clone()
+    scale = rnd(M, seed=4)
+    ops.gemm(a, w, epilogue=ops.EPI_RESID, out=h, row_scale=scale)
+    close(h, h0.double() + ref * scale.double()[:, None], dtype, "residual")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,I,K", [(1, 32, 64), (7, 48, 96), (40, 100, 72), (200, 176, 256)])
+def test_gemm_gate_up(dtype, M, I, K):
+    from ferrox_amd import ops
+    a, w = rnd(M, K, dtype=dtype), rnd(2 * I, K, dtype=dtype, seed=1, scale=0.5)
+    g, u = a.double() @ w[:I].double().T, a.double() @ w[I:].double().T
+    close(ops.gemm(a, w, epilogue=ops.EPI_SILU_MUL), plain.silu(g) * u, dtype, "silu(gate)*up")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,k,I,H", [(1, 4, 2, 32, 64), (9, 6, 3, 48, 96), (70, 5, 1, 40, 120), (300, 8, 2, 64, 128),
+                                        (64, 3, 2, 24, 72)])
+def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
+    """router ids -> align -> grouped gate/up -> grouped down -> combine, against per-token loops."""
+    from ferrox_amd import ops
+    x = rnd(T, H, dtype=dtype)
+    w_gu, w_dn = rnd(E, 2 * I, H, dtype=dtype, seed=1, scale=0.3), rnd(E, H, I, dtype=dtype, seed=2, scale=0.3)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    wts = torch.rand(T, k, generator=g).to(DEV)
+    offsets, sorted_token, inv = ops.moe_align(ids, E)
+    # the sort: offsets are the counts' prefix sums; every pair sits in its expert's range; order is stable
+    counts = torch.bincount(ids.flatten().long().cpu(), minlength=E)
+    assert offsets.cpu().tolist() == [0] + torch.cumsum(counts, 0).tolist()
+    inv_c, st_c, ids_c = inv.cpu(), sorted_token.cpu(), ids.cpu()
+    assert sorted(inv_c.tolist()) == list(range(T * k))
+    for i in range(T * k):
+        e = int(ids_c.flatten()[i])
+        assert offsets[e] <= inv_c[i] < offsets[e + 1] and st_c[inv_c[i]] == i // k
+    for e in range(E):
+        seg = [i for i in range(T * k) if int(ids_c.flatten()[i]) == e]
+        assert [int(inv_c[i]) for i in seg] == list(range(int(offsets[e]), int(offsets[e + 1])))
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets)
+    h = torch.zeros(T, H, device=DEV)
+    ops.moe_combine(h, y, inv, wts, k)
+    ref = torch.zeros(T, H, dtype=torch.float64)
+    xd, gud, dnd = x.double().cpu(), w_gu.double().cpu(), w_dn.double().cpu()
+    for t in range(T):
+        for j in range(k):
+            e = int(ids_c[t, j])
+            a = plain.silu(xd[t] @ gud[e, :I].T) * (xd[t] @ gud[e, I:].T)
+            if dtype == torch.bfloat16:
+                a = a.to(torch.bfloat16).double()       # the engine stores the activation in bfloat16
+            ref[t] += float(wts[t, j]) * (a @ dnd[e].T)
+    close(h, ref, dtype, "moe")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_and_embed(dtype):
+    from ferrox_amd import ops
+    for T, H, eps in [(1, 64, 1e-6), (5, 96, 1e-5), (3, 1000, 1e-3), (2, 4100, 1e-6)]:
+        h = rnd(T, H, scale=3.0)
+        w = rnd(H, dtype=dtype, seed=1)
+        ref = plain.rms_norm(h.double().cpu(), w.double().cpu(), eps)
+        close(ops.rmsnorm(h, w, eps, dtype), ref, dtype, f"rmsnorm {T}x{H}")
+        rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+        close(ops.rmsnorm(h, w, eps, dtype, rows=rows), ref[[T - 1, 0]], dtype, "rmsnorm rows")
+    table = rnd(50, 72, dtype=dtype)
+    ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.embed(table, ids), table[ids.long()].float())
+
+
+def paged_setup(dtype, nh, nkv, hd, bs, seq_lens, theta, rot, n_pages, seed=0):
+    """Random q, k, v for whole sequences; pages filled through rope_kv_write with a shuffled page order."""
+    from ferrox_amd import ops
+    rng = random.Random(seed)
+    free = list(range(n_pages))
+    rng.shuffle(free)
+    max_blocks = max(-(-L // bs) for L in seq_lens)
+    table = torch.zeros(len(seq_lens), max_blocks, dtype=torch.int32)
+    toks = []
+    for s, L in enumerate(seq_lens):
+        for b in range(-(-L // bs)):
+            table[s, b] = free.pop()
+        toks += [(s, p) for p in range(L)]
+    T = len(toks)
+    q, k, v = rnd(T, nh * hd, dtype=dtype), rnd(T, nkv * hd, dtype=dtype, seed=1), rnd(T, nkv * hd, dtype=dtype, seed=2)
+    k_pages = torch.zeros(n_pages, nkv, bs, hd, dtype=dtype, device=DEV)
+    v_pages = torch.zeros(n_pages, nkv, hd, bs, dtype=dtype, device=DEV)
+    pos = torch.tensor([p for _, p in toks], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([s for s, _ in toks], dtype=torch.int32, device=DEV)
+    q_rot = q.clone()
+    ops.rope_kv_write(q_rot, k, v, pos, seq, table.to(DEV), k_pages, v_pages, nh, nkv, hd, bs, rot, theta)
+    return q, k, v, q_rot, k_pages, v_pages, table.to(DEV), pos, seq, toks
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,bs,rot,theta", [(4, 4, 16, 16, 16, 1e4), (3, 1, 32, 8, 32, 1e6), (6, 3, 48, 4, 24, 5e4),
+                                                    (2, 2, 128, 64, 128, 1e6), (8, 2, 80, 16, 80, 1e4)])
+def test_rope_and_cache_write(dtype, nh, nkv, hd, bs, rot, theta):
+    seq_lens = [5, 2 * bs + 3, 1]
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, seq_lens, theta, rot, 12)
+    qd, kd = q.double().cpu().reshape(-1, nh, hd), k.double().cpu().reshape(-1, nkv, hd)
+    for t, (s, p) in enumerate(toks):
+        want_q = torch.cat([plain.rope_neox(qd[t][:, :rot], p, theta), qd[t][:, rot:]], dim=-1)
+        close(q_rot[t].reshape(nh, hd), want_q, dtype, f"q rope token {t}")
+        want_k = torch.cat([plain.rope_neox(kd[t][:, :rot], p, theta), kd[t][:, rot:]], dim=-1)
+        page = int(table[s, p // bs])
+        close(k_pages[page, :, p % bs, :], want_k, dtype, f"k page token {t}")
+        assert torch.equal(v_pages[page, :, :, p % bs].reshape(-1), v[t]), f"v page token {t}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,bs,window", [(4, 4, 16, 16, 0), (3, 1, 32, 8, 16), (6, 3, 48, 4, 40), (2, 2, 128, 64, 0),
+                                                 (8, 2, 80, 16, 7), (4, 1, 256, 32, 100)])
+def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
+    """Whole sequences through the tiled kernel, and their last tokens again through the decode
+    kernel, against the plain attention on the same rotated, rounded q/k/v."""
+    from ferrox_amd import ops
+    seq_lens = [70, 1, 33, 150]
+    theta = 1e4
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, seq_lens, theta, hd, 64)
+    T = len(toks)
+    scale = 1.0 / math.sqrt(hd)
+    # reference from what the pages hold
+    ref = torch.zeros(T, nh, hd, dtype=torch.float64)
+    starts = [0]
+    for L in seq_lens:
+        starts.append(starts[-1] + L)
+    kp, vp, tab = k_pages.double().cpu(), v_pages.double().cpu(), table.cpu()
+    for s, L in enumerate(seq_lens):
+        ks = torch.stack([kp[int(tab[s, p // bs]), :, p % bs, :] for p in range(L)])
+        vs = torch.stack([vp[int(tab[s, p // bs]), :, :, p % bs] for p in range(L)])
+        qs = q_rot[starts[s]:starts[s + 1]].double().cpu().reshape(L, nh, hd)
+        ref[starts[s]:starts[s + 1]] = plain.causal_attention(qs, ks, vs, nh, nkv, window or None)
+    ref = ref.reshape(T, nh * hd)
+    # tiles of up to 16 queries
+    t_seq, t_tok, t_n = [], [], []
+    for s, L in enumerate(seq_lens):
+        for t0 in range(0, L, 16):
+            t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(16, L - t0))
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    out = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
+    ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale)
+    close(out, ref, dtype, "tiled attention")
+    # the last token of every sequence as a single query
+    out2 = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
+    last = [starts[s + 1] - 1 for s in range(len(seq_lens))]
+    for chunk in (64, 256):
+        ops.attention_decode(q_rot, out2, k_pages, v_pages, table, pos, i32(list(range(len(seq_lens)))), i32(last),
+                             nh, nkv, hd, bs, window, scale, max_kv_len=max(seq_lens), chunk=chunk)
+        close(out2[last], ref[last], dtype, f"decode attention chunk {chunk}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,H,E,k,renorm", [(1, 64, 8, 2, False), (7, 96, 6, 3, True), (33, 200, 60, 4, False),
+                                             (5, 128, 130, 8, True), (4, 72, 5, 5, False)])
+def test_router(dtype, T, H, E, k, renorm):
+    from ferrox_amd import ops
+    x, wr, sg = rnd(T, H, dtype=dtype), rnd(E, H, dtype=dtype, seed=1, scale=0.3), rnd(H, dtype=dtype, seed=2, scale=0.2)
+    ids, w, gate = ops.router_topk(x, wr, k, renorm, shared_gate=sg)
+    xd, wd = x.double().cpu(), wr.double().cpu()
+    for t in range(T):
+        want_ids, want_w = plain.route_top_k(wd @ xd[t], k, renorm)
+        assert ids[t].tolist() == want_ids, f"token {t}: experts {ids[t].tolist()} != {want_ids}"
+        close(w[t], want_w, torch.float32, f"router weights token {t}")
+    close(gate, torch.sigmoid(xd @ sg.double().cpu()), torch.float32, "shared gate")
+
+
+def test_router_golden_vector():
+    """logits 1..8, k=3, no renormalisation -> experts [7, 6, 5], weights [0.6323223, 0.2326232,
+    0.0855683] (the vector of the reference's own test, ferrox-moe/src/lib.rs:863-893)."""
+    from ferrox_amd import ops
+    x = torch.zeros(1, 8, device=DEV)
+    x[0, 0] = 1.0
+    wr = torch.zeros(8, 8, device=DEV)
+    wr[:, 0] = torch.arange(1, 9, dtype=torch.float32)
+    ids, w, _ = ops.router_topk(x, wr, 3, False)
+    assert ids[0].tolist() == [7, 6, 5]
+    assert torch.allclose(w[0].cpu(), torch.tensor([0.6323223, 0.2326232, 0.0855683]), atol=1e-6)
+    ids, w, _ = ops.router_topk(x, torch.zeros(8, 8, device=DEV), 3, True)      # all equal: lowest indices
+    assert ids[0].tolist() == [0, 1, 2] and torch.allclose(w[0].cpu(), torch.full((3,), 1 / 3))
+
+
+def test_sampling_kernel():
+    from ferrox_amd import ops
+    V = 1000
+    logits = rnd(6, V, scale=3.0)
+    assert ops.sample(logits).tolist() == logits.argmax(-1).tolist()
+    tie = torch.zeros(1, V, device=DEV)
+    tie[0, [17, 400]] = 5.0
+    assert ops.sample(tie).tolist() == [17]
+    # seeded sampling against the plain sampler, option by option
+    cases = [dict(temperature=0.8), dict(temperature=1.3, top_k=5), dict(temperature=0.7, top_p=0.6),
+             dict(temperature=1.0, top_k=50, top_p=0.9, repetition_penalty=1.3),
+             dict(temperature=0.0, repetition_penalty=2.0, presence_penalty=0.5, frequency_penalty=0.25),
+             dict(temperature=0.9, top_k=1)]
+    hist = [int(logits[0].argmax()), 3, 3, 999, int(logits[0].argmax())]
+    for case in cases:
+        for trial in range(12):
+            rng_a = plain.XorShift64(trial + 1)
+            want = plain.sample(logits[0].double().cpu().tolist(), rng_a, history=hist, **case)
+            u = plain.XorShift64(trial + 1).next_f32()
+            f = lambda v: torch.tensor([v], dtype=torch.float32, device=DEV)
+            got = ops.sample(logits[:1], temperature=f(case.get("temperature", 0.0)), draw=f(u),
+                             top_k=torch.tensor([case.get("top_k", 0)], dtype=torch.int32, device=DEV),
+                             top_p=f(case.get("top_p", 1.0)), rep_penalty=f(case.get("repetition_penalty", 1.0)),
+                             presence=f(case.get("presence_penalty", 0.0)), frequency=f(case.get("frequency_penalty", 0.0)),
+                             hist=torch.tensor(hist, dtype=torch.int32, device=DEV),
+                             hist_start=torch.tensor([0, len(hist)], dtype=torch.int32, device=DEV)).tolist()[0]
+            assert got == want, f"{case} trial {trial}: kernel {got}, plain {want}"
