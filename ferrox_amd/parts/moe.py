@@ -22,6 +22,7 @@ GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
 @FEED_FORWARDS.register("sparse_moe")
 class SparseMoE(FeedForward):
     kernel_libraries = ("elementwise", "gemm", "moe")
+    record = None      # a list here collects every call's expert ids (measurement only)
 
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
                  norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
@@ -67,6 +68,8 @@ class SparseMoE(FeedForward):
         T = x.shape[0]
         ids, weights, gate = ops.router_topk(x, self.router, self.top_k, self.norm_topk_prob, self.gating,
                                              self.shared_gate_w)
+        if SparseMoE.record is not None:
+            SparseMoE.record.append(ids)
         offsets, sorted_token, inv = ops.moe_align(ids, self.n_experts)
         act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
                      expert_offsets=offsets, n_rows=T * self.top_k)
