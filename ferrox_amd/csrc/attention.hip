@@ -231,6 +231,215 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// bfloat16 on MFMA (head_dim and block size multiples of 16).
+//
+// One wave owns 16 "rows" that share one kv head: 16 consecutive queries of one
+// head (prefill), or the query heads of one kv group for a single token
+// (decode).  For a tile of 64 keys it computes S^T = K Q^T with K as the A
+// operand, so that the accumulator of lane (row = lane%16, g = lane/16) holds 16
+// scores of its own row; the softmax runs on those registers, and the same
+// registers, rounded to bfloat16, are the A operand of O += P V (16x16x16 MFMA,
+// whose lane (row, g) supplies k = 4g..4g+3).  To make that work, A-row i of key
+// block kb reads key 16*(i/4) + 4*kb + i%4 of the tile, and the B operand reads
+// 16 consecutive keys 16g..16g+15 of a transposed value row.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    return (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
+}
+
+template <int HD>   // compile-time bound of head_dim (a.hd <= HD)
+struct WaveAttn {
+    static constexpr int KS = HD / 32;   // k-steps of S^T = K Q^T
+    static constexpr int CB = HD / 16;   // column blocks of O
+    float m, l;                          // running max and sum of this lane's row
+    f32x4_t o[CB];                       // lane (j, g): O[row 4g+r][16*cb + j]
+    bf16x8_t qf[KS];                     // lane (row, g): Q[row][32u + 8g ..]
+
+    __device__ __forceinline__ void init(const bf16* qrow, int hd) {
+        m = NEG_INF;
+        l = 0.f;
+        const int g = threadIdx.x >> 4 & 3;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) o[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            const int d = 32 * u + 8 * g;
+            uint4 v = (qrow && d < hd) ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
+            qf[u] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+
+    // keys [kt0, kt0 + 64); this lane's row sees key t iff lo <= t <= hi (hi < lo: row unused)
+    __device__ __forceinline__ void tile(const AttnArgs& a, const int* bt, int kvh, int kt0, int kv_begin, int kv_end,
+                                         int lo, int hi) {
+        const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
+        const int hd = a.hd, bs = a.bs;
+        f32x4_t sc[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            const int key = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
+            const bf16* kr = nullptr;
+            if (key >= kv_begin && key < kv_end)
+                kr = (const bf16*)a.k_pages + (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd;
+#pragma unroll
+            for (int u = 0; u < KS; ++u) {
+                const int d = 32 * u + 8 * g;
+                const uint4 v = (kr && d < hd) ? *(const uint4*)(kr + d) : make_uint4(0, 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, v), qf[u], sc[kb], 0, 0, 0);
+            }
+        }
+        // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
+        float mt = NEG_INF;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kt0 + 16 * g + 4 * kb + r;
+                const float v = (key >= lo && key <= hi) ? sc[kb][r] * a.scale : NEG_INF;
+                sc[kb][r] = v;
+                mt = fmaxf(mt, v);
+            }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
+        float ps = 0.f;
+        uint2 pk[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[r] = (sc[kb][r] == NEG_INF) ? 0.f : expf(sc[kb][r] - m_new);
+                ps += p[r];
+            }
+            pk[kb] = make_uint2(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]));
+        }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * alpha + ps;
+        m = m_new;
+        // the accumulators hold rows 4g+r: fetch their factors from the lanes that own those rows
+        float al[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
+        // values: 16 consecutive keys kt0 + 16g .. of transposed row d = 16*cb + li
+        const int kg = kt0 + 16 * g;
+        const bool vload = kg < kv_end && kg + 16 > kv_begin;
+        const bf16* vbase = nullptr;
+        if (vload) vbase = (const bf16*)a.v_pages + ((size_t)bt[kg / bs] * a.nkv + kvh) * hd * bs + kg % bs;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const int d = 16 * cb + li;
+            uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
+            if (vbase && d < hd) {
+                v0 = *(const uint4*)(vbase + (size_t)d * bs);
+                v1 = *(const uint4*)(vbase + (size_t)d * bs + 8);
+            }
+            f32x4_t acc = o[cb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] *= al[r];
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[0]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.x, v0.y)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[1]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.z, v0.w)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[2]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.x, v1.y)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[3]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.z, v1.w)), acc, 0, 0, 0);
+            o[cb] = acc;
+        }
+    }
+};
+
+// prefill: item = up to 16 consecutive queries of one sequence; block = one wave = (item, head)
+template <int HD>
+__global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
+    const int item = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+    const int kvh = h / (a.nh / a.nkv);
+    const int tok0 = a.item_tok[item], n = a.item_n[item];
+    const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
+    const int hd = a.hd;
+    const int pmin = a.positions[tok0], pmax = a.positions[tok0 + n - 1];
+    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_end = pmax + 1;
+    int lo = 1, hi = 0;
+    const bf16* qrow = nullptr;
+    if (li < n) {
+        hi = a.positions[tok0 + li];
+        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * hd;
+    }
+    WaveAttn<HD> w;
+    w.init(qrow, hd);
+    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        const float lr = __shfl(w.l, row, 64);
+        if (row < n) {
+#pragma unroll
+            for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
+                const int d = 16 * cb + li;
+                if (d < hd) from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * hd + d, w.o[cb][r] / lr);
+            }
+        }
+    }
+}
+
+// decode: item = one token; block = one wave = (item, kv head x group block of 16 query heads, split)
+template <int HD>
+__global__ __launch_bounds__(64) void attn_mfma_decode_kernel(AttnArgs a) {
+    const int item = blockIdx.x, split = blockIdx.z, lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+    const int group = a.nh / a.nkv, gblocks = (group + 15) / 16;
+    const int kvh = blockIdx.y / gblocks, hb = blockIdx.y % gblocks;
+    const int tok = a.item_tok[item];
+    const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
+    const int hd = a.hd;
+    const int p = a.positions[tok];
+    const int kv_begin = max(a.window > 0 ? max(0, p - a.window + 1) : 0, split * a.chunk);
+    const int kv_end = min(p + 1, (split + 1) * a.chunk);
+    const int n = min(16, group - hb * 16);        // query heads in this block
+    const int h0 = kvh * group + hb * 16;
+    const bool empty = kv_begin >= kv_end;
+    WaveAttn<HD> w;
+    const bool row_ok = li < n;
+    w.init(row_ok && !empty ? (const bf16*)a.q + (size_t)tok * a.ldq + (size_t)(h0 + li) * hd : nullptr, hd);
+    if (!empty) {
+        const int lo = row_ok ? kv_begin : 1, hi = row_ok ? kv_end - 1 : 0;
+        for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
+    }
+    if (li < n && g == 0) {
+        float* pml = a.part_ml + (((size_t)item * a.nh + h0 + li) * a.splits + split) * 2;
+        pml[0] = empty ? NEG_INF : w.m;
+        pml[1] = empty ? 0.f : w.l;
+    }
+    if (empty) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        if (row < n) {
+            float* po = a.part_o + (((size_t)item * a.nh + h0 + row) * a.splits + split) * hd;
+#pragma unroll
+            for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
+                const int d = 16 * cb + li;
+                if (d < hd) po[d] = w.o[cb][r];
+            }
+        }
+    }
+}
+
+static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
+    return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
+           (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
+}
+
+// ---------------------------------------------------------------------------
 static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "%s: unknown dtype %d", who, dtype);
     FX_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: n_heads %d must be a multiple of n_kv_heads %d", who, nh, nkv);
@@ -253,10 +462,16 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
     dim3 grid(n_items, nh);
+    hipStream_t s = (hipStream_t)stream;
     if (dtype == FX_F32)
-        attn_tile_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(a);
-    else
-        attn_tile_kernel<bf16><<<grid, 64, 0, (hipStream_t)stream>>>(a);
+        attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages) && hd % 16 == 0) {
+        if (hd <= 32) attn_mfma_tile_kernel<32><<<grid, 64, 0, s>>>(a);
+        else if (hd <= 64) attn_mfma_tile_kernel<64><<<grid, 64, 0, s>>>(a);
+        else if (hd <= 128) attn_mfma_tile_kernel<128><<<grid, 64, 0, s>>>(a);
+        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);
+    } else
+        attn_tile_kernel<bf16><<<grid, 64, 0, s>>>(a);
     FX_CHECK_LAUNCH("attn_tiles");
     return 0;
 }
@@ -282,6 +497,14 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     if (dtype == FX_F32) {
         attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<float><<<grid2, 64, 0, s>>>(a);
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
+        const int group = nh / nkv;
+        dim3 gridm(n_items, nkv * ((group + 15) / 16), splits);
+        if (hd <= 32) attn_mfma_decode_kernel<32><<<gridm, 64, 0, s>>>(a);
+        else if (hd <= 64) attn_mfma_decode_kernel<64><<<gridm, 64, 0, s>>>(a);
+        else if (hd <= 128) attn_mfma_decode_kernel<128><<<gridm, 64, 0, s>>>(a);
+        else attn_mfma_decode_kernel<256><<<gridm, 64, 0, s>>>(a);
+        attn_decode_merge_kernel<bf16><<<grid2, 64, 0, s>>>(a);
     } else {
         attn_decode_kernel<bf16><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<bf16><<<grid2, 64, 0, s>>>(a);

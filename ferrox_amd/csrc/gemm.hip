@@ -222,6 +222,110 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Few rows (decode): the weights are streamed once from memory straight into
+// MFMA operands, no LDS staging.  A block owns 16 output columns (16 rows of W)
+// and up to 16*MT logical rows; its WAVES waves split K between them in pieces
+// of 128 and their partial sums are added in wave order through LDS.  Lane
+// (i = lane%16, g = lane/16) reads 64 contiguous bytes of W row n0+i per piece,
+// so the four g-lanes of a row cover 256 contiguous bytes; the activations use
+// the same k -> lane assignment, which is all the MFMA needs to be right.
+// W is the A operand: the accumulator of lane (m = lane%16, g) holds
+// C[m][n0 + 4g + r], r = 0..3.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint4 load16(const bf16* row, int k, int K) {
+    return (row && k < K) ? *(const uint4*)(row + k) : make_uint4(0, 0, 0, 0);
+}
+
+template <int MT, int WAVES, bool DUAL, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
+    constexpr int NACC = MT * (DUAL ? 2 : 1);
+    __shared__ f32x4_t red[WAVES][NACC][64];
+    int r0, r_end, expert;
+    locate_rows<16 * MT>(g, blockIdx.y, r0, r_end, expert);
+    if (r0 < 0) return;
+    const int n0 = blockIdx.x * 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, grp = lane >> 4;
+    const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
+    const bf16* wrow = (n0 + li < g.N) ? Wbase + (size_t)(n0 + li) * g.K : nullptr;
+    const bf16* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = r0 + mt * 16 + li;
+        xrow[mt] = (m < r_end) ? (const bf16*)g.A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : nullptr;
+    }
+    f32x4_t acc[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    const int n_super = (g.K + 127) / 128;
+    const int per = (n_super + WAVES - 1) / WAVES;
+    const int s_end = min(n_super, (wave + 1) * per);
+    for (int s = wave * per; s < s_end; ++s) {
+        const int kb = s * 128 + grp * 32;
+        uint4 w[4], wu[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            w[u] = load16(wrow, kb + 8 * u, g.K);
+            if (DUAL) wu[u] = load16(wrow ? wrow + g.up_offset : nullptr, kb + 8 * u, g.K);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            uint4 x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = load16(xrow[mt], kb + 8 * u, g.K);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[u]);
+                if (DUAL) {
+                    acc[2 * mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[u]), xb, acc[2 * mt], 0, 0, 0);
+                    acc[2 * mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wu[u]), xb, acc[2 * mt + 1], 0, 0, 0);
+                } else {
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[u]), xb, acc[mt], 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) red[wave][a][lane] = acc[a];
+    __syncthreads();
+    for (int idx = tid; idx < MT * 64; idx += WAVES * 64) {
+        const int mt = idx >> 6, L = idx & 63;
+        f32x4_t v = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v2 = v;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            if (DUAL) {
+                v += red[w][2 * mt][L];
+                v2 += red[w][2 * mt + 1][L];
+            } else {
+                v += red[w][mt][L];
+            }
+        }
+        const int m = r0 + mt * 16 + (L & 15);
+        if (m >= r_end) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n0 + (L >> 4) * 4 + r;
+            if (n >= g.N) continue;
+            float o = v[r];
+            if (DUAL) {
+                from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(o) * v2[r]);
+                continue;
+            }
+            if (g.bias) o += load_as_float(g.bias, g.bias_dtype, n);
+            if (EPI == EPI_STORE) {
+                from_float((bf16*)g.C + (size_t)m * g.ldc + n, o);
+            } else if (EPI == EPI_STORE_F32) {
+                ((float*)g.C)[(size_t)m * g.ldc + n] = o;
+            } else {
+                if (g.row_scale) o *= g.row_scale[m];
+                ((float*)g.C)[(size_t)m * g.ldc + n] += o;
+            }
+        }
+    }
+}
+
 // ===========================================================================
 // float32 with FMA
 // ===========================================================================
@@ -327,6 +431,30 @@ static void launch_bf16(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) 
     }
 }
 
+template <int MT, int WAVES>
+static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
+    dim3 grid(ceil_div(g.N, 16), m_tiles);
+    switch (epi) {
+        case EPI_STORE: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_STORE><<<grid, WAVES * 64, 0, s>>>(g); break;
+        case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
+        case EPI_RESID: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_RESID><<<grid, WAVES * 64, 0, s>>>(g); break;
+        default:
+            if constexpr (MT * 2 * WAVES <= 32)
+                gemm_bf16_skinny_kernel<MT, WAVES, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
+            break;
+    }
+}
+
+static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int m_tiles, hipStream_t s) {
+    if (mt == 1) {
+        if (eight) launch_skinny_cfg<1, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<1, 4>(g, epi, m_tiles, s);
+    } else if (mt == 2) {
+        if (eight) launch_skinny_cfg<2, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<2, 4>(g, epi, m_tiles, s);
+    } else {
+        if (eight) launch_skinny_cfg<4, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<4, 4>(g, epi, m_tiles, s);
+    }
+}
+
 // dtype: type of A and W.  C is: T for EPI_STORE and EPI_SILU_MUL, float32 otherwise.
 // rows_hint: in grouped mode, the expected number of rows per expert (chooses the tile).
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
@@ -363,10 +491,17 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.vec_ok = (K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
                (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
-    if (per_group <= 16) {
-        const int m_tiles = M / 16 + (expert_offsets ? nonempty : (M % 16 != 0));
-        launch_bf16<16, 256, 16, 64>(g, epi, m_tiles, s);
-    } else if (per_group <= 64) {
+    if (g.vec_ok && per_group <= 64) {
+        const int mt = per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4);
+        const int m_tiles = M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
+        const long blocks = (long)ceil_div(N, 16) * m_tiles;
+        const bool dual = epi == EPI_SILU_MUL;
+        const bool eight = blocks < 1024 && mt * (dual ? 2 : 1) <= 4 && K >= 2048;
+        launch_skinny(g, epi, mt, eight, m_tiles, s);
+        FX_CHECK_LAUNCH("gemm_bf16_skinny");
+        return 0;
+    }
+    if (per_group <= 64) {
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else {

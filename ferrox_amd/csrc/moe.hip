@@ -36,11 +36,49 @@ __global__ __launch_bounds__(256) void router_topk_kernel(
     const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (int c = tid; c < H; c += 256) xs[c] = to_float(x[(size_t)t * ldx + c]);
     __syncthreads();
-    for (int e = wave; e < E; e += 4) {
-        float acc = 0.f;
-        for (int c = lane; c < H; c += 64) acc = fmaf(xs[c], load_as_float(Wr, w_dtype, (size_t)e * H + c), acc);
-        acc = wave_sum(acc);
-        if (lane == 0) score[e] = acc;
+    // four experts at a time per wave, 8 weights per lane and step, so that many loads are in flight;
+    // the order of the sums depends on H alone
+    const bool vec = (H % 8 == 0) && (((uintptr_t)Wr) % 16 == 0);
+    for (int e0 = wave * 4; e0 < E; e0 += 16) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        if (vec) {
+            for (int c = lane * 8; c < H; c += 512) {
+                float xv[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] = xs[c + i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = e0 + j;
+                    if (e >= E) continue;
+                    if (w_dtype == FX_BF16) {
+                        const uint4 v = *(const uint4*)((const bf16*)Wr + (size_t)e * H + c);
+                        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            acc[j] = fmaf(xv[2 * i], __uint_as_float(u[i] << 16), acc[j]);
+                            acc[j] = fmaf(xv[2 * i + 1], __uint_as_float(u[i] & 0xffff0000u), acc[j]);
+                        }
+                    } else {
+                        const float4 a = *(const float4*)((const float*)Wr + (size_t)e * H + c);
+                        const float4 b = *(const float4*)((const float*)Wr + (size_t)e * H + c + 4);
+                        acc[j] = fmaf(xv[0], a.x, acc[j]); acc[j] = fmaf(xv[1], a.y, acc[j]);
+                        acc[j] = fmaf(xv[2], a.z, acc[j]); acc[j] = fmaf(xv[3], a.w, acc[j]);
+                        acc[j] = fmaf(xv[4], b.x, acc[j]); acc[j] = fmaf(xv[5], b.y, acc[j]);
+                        acc[j] = fmaf(xv[6], b.z, acc[j]); acc[j] = fmaf(xv[7], b.w, acc[j]);
+                    }
+                }
+            }
+        } else {
+            for (int c = lane; c < H; c += 64)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (e0 + j < E) acc[j] = fmaf(xs[c], load_as_float(Wr, w_dtype, (size_t)(e0 + j) * H + c), acc[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float v = wave_sum(acc[j]);
+            if (lane == 0 && e0 + j < E) score[e0 + j] = v;
+        }
     }
     if (shared_gate) {
         float acc = 0.f;

@@ -119,7 +119,16 @@ def swiglu_mlp(x, w_gate, w_up, w_down) -> torch.Tensor:
     return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
 
 
-def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w):
+def router_margin(logits: torch.Tensor, k: int) -> float:
+    """Relative gap between the k-th and the (k+1)-th probability: how far the choice of
+    experts is from flipping (1.0 if all experts are chosen)."""
+    p = torch.softmax(logits, 0).sort(descending=True).values
+    if k >= p.shape[0]:
+        return 1.0
+    return float((p[k - 1] - p[k]) / p[k - 1])
+
+
+def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w, margins=None):
     """One token through the sparse block.
 
     Router logits r = router . x with no bias (ferrox-models/src/decoder.rs:2915),
@@ -130,6 +139,8 @@ def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w
     """
     logits = router_w @ x
     ids, w = route_top_k(logits, k, norm_topk_prob)
+    if margins is not None:
+        margins.append(router_margin(logits, k))
     out = torch.zeros_like(x)
     for j, e in enumerate(ids):
         g, u, d = experts[e]
@@ -180,13 +191,17 @@ def load_folder(folder: str, dtype=torch.float64):
     return cfg, weights
 
 
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0) -> torch.Tensor:
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0, margins=None) -> torch.Tensor:
     """Logits[T, V] of one whole sequence (ferrox-models/src/decoder.rs:3014-3678
     followed by the head on every row, decoder.rs:2952-2973).
 
     `start_pos` shifts every position (used by the shift-invariance test only).
+    `margins`, a list of T floats if given, receives for every position the smallest
+    `router_margin` over the sparse layers.
     """
     T = len(tokens)
+    if margins is not None:
+        margins[:] = [1.0] * T
     nh = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads", nh)
     hd = head_dim_of(cfg)
@@ -223,11 +238,15 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0)
                           w[p + "mlp.shared_expert.up_proj.weight"],
                           w[p + "mlp.shared_expert.down_proj.weight"])
                 gate_w = w[p + "mlp.shared_expert_gate.weight"]
+            layer_margins = [] if margins is not None else None
             f = torch.stack([
                 moe_ffn_token(x2[t], w[p + "mlp.gate.weight"], experts,
                               cfg["num_experts_per_tok"], cfg.get("norm_topk_prob", False),
-                              shared, gate_w)
+                              shared, gate_w, layer_margins)
                 for t in range(T)])
+            if margins is not None:
+                for t in range(T):
+                    margins[t] = min(margins[t], layer_margins[t])
         else:                                                                        # dense layer: decoder.rs:2902-2913
             f = swiglu_mlp(x2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                            w[p + "mlp.down_proj.weight"])

@@ -134,23 +134,33 @@ def _plain_model(folder: str):
 _plain_cache: dict = {}
 
 
-def plain_logits(folder: str, tokens) -> torch.Tensor:
+def plain_logits(folder: str, tokens, with_margins: bool = False):
     key = (folder, tuple(tokens))
     if key not in _plain_cache:
         cfg, w = _plain_model(folder)
-        _plain_cache[key] = plain.forward(cfg, w, list(tokens))
-    return _plain_cache[key]
+        margins = []
+        _plain_cache[key] = (plain.forward(cfg, w, list(tokens), margins=margins), margins)
+    return _plain_cache[key] if with_margins else _plain_cache[key][0]
 
 
-def compare(got: dict, folder: str, requests: dict, atol: float, rtol: float, what: str) -> float:
-    """Every (request, position) of `got` against the plain implementation; returns the largest error."""
-    worst, worst_at = 0.0, None
+def compare(got: dict, folder: str, requests: dict, atol: float, rtol: float, what: str,
+            min_margin: float = 0.0) -> float:
+    """Every (request, position) of `got` against the plain implementation; returns the largest error.
+
+    `min_margin` > 0 (bfloat16 only): positions where the plain router's k-th and (k+1)-th
+    probabilities lie closer than this relative gap are not compared: there the choice of experts
+    is decided by rounding, and either choice is a right answer.  They must stay a small minority."""
+    worst, worst_at, skipped, total = 0.0, None, 0, 0
     for rid, toks in requests.items():
-        ref = plain_logits(folder, toks)
+        ref, margins = plain_logits(folder, toks, with_margins=True)
         for p in range(len(toks)):
             assert (rid, p) in got, f"{what}: no logits for request {rid} position {p}"
             g = got[(rid, p)].double()
             assert torch.isfinite(g).all(), f"{what}: non-finite logits for {rid} position {p}"
+            total += 1
+            if margins[p] < min_margin:
+                skipped += 1
+                continue
             err = (g - ref[p]).abs()
             bound = atol + rtol * ref[p].abs()
             if (err > bound).any():
@@ -159,5 +169,6 @@ def compare(got: dict, folder: str, requests: dict, atol: float, rtol: float, wh
                                      f"plain {float(ref[p][i]):.7f}, |diff| {float(err[i]):.3e} > {float(bound[i]):.3e}")
             if float(err.max()) > worst:
                 worst, worst_at = float(err.max()), (rid, p)
-    print(f"[{what}] largest |engine - plain| = {worst:.3e} at {worst_at}")
+    assert skipped <= 0.15 * total, f"{what}: {skipped} of {total} positions have a near-tie in the router"
+    print(f"[{what}] largest |engine - plain| = {worst:.3e} at {worst_at}; {skipped}/{total} near-ties not compared")
     return worst

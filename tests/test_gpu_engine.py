@@ -19,6 +19,9 @@ LENGTHS = {"A": [1, 7, 16, 33, 70, 45], "B": [3, 17, 40, 64, 90, 120], "C": [2, 
 # bfloat16: weights are the same bfloat16 values on both sides; activations are rounded to 8 bits
 # of mantissa at every matrix product, and logits are of the order 0.1 .. 0.5.
 TOL = {"float32": (5e-6, 2e-5), "bfloat16": (2e-2, 2e-2)}
+# bfloat16 rounding moves a router probability by about 1 part in 1000; positions whose top-k choice
+# hangs on less than five times that in the plain model are left out of the bfloat16 comparison.
+MARGIN = {"float32": 0.0, "bfloat16": 0.005}
 
 _runners = {}
 
@@ -44,7 +47,7 @@ def test_whole_prompts(model_folders, name, dtype):
     folder, runner = runner_for(model_folders, name, dtype, block_size=16, num_pages=16)
     reqs = requests_for(name)
     got = ru.run_trace(runner, ru.trace_whole(reqs))
-    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} whole")
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} whole", MARGIN[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -53,7 +56,7 @@ def test_last_tokens_one_by_one(model_folders, name, dtype):
     folder, runner = runner_for(model_folders, name, dtype, block_size=8, num_pages=24)
     reqs = requests_for(name)
     got = ru.run_trace(runner, ru.trace_tail_decode(reqs))
-    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} tail-decode")
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} tail-decode", MARGIN[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -62,7 +65,7 @@ def test_portions_of_changing_size(model_folders, name, dtype):
     folder, runner = runner_for(model_folders, name, dtype, block_size=8, num_pages=24)
     reqs = requests_for(name)
     got = ru.run_trace(runner, ru.trace_portions(reqs))
-    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} portions")
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} portions", MARGIN[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -75,7 +78,7 @@ def test_mixed_batches_with_page_reuse(model_folders, name, dtype):
     folder, runner = runner_for(model_folders, name, dtype, block_size=bs, num_pages=pages)
     got = ru.run_trace(runner, steps)
     assert runner.manager.n_free_pages() == pages
-    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} mixed")
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} mixed", MARGIN[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32"])
