@@ -255,6 +255,7 @@ template <int HD>   // compile-time bound of head_dim (a.hd <= HD)
 struct WaveAttn {
     static constexpr int KS = HD / 32;   // k-steps of S^T = K Q^T
     static constexpr int CB = HD / 16;   // column blocks of O
+    static constexpr bool EARLY_V = HD <= 128;   // registers allow the values to be fetched before the scores
     float m, l;                          // running max and sum of this lane's row
     f32x4_t o[CB];                       // lane (j, g): O[row 4g+r][16*cb + j]
     bf16x8_t qf[KS];                     // lane (row, g): Q[row][32u + 8g ..]
@@ -278,10 +279,28 @@ struct WaveAttn {
                                          int lo, int hi) {
         const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
         const int hd = a.hd, bs = a.bs;
+        // values first, so that they arrive while the scores are computed: 16 consecutive keys
+        // kt0 + 16g .. of transposed row d = 16*cb + li
+        const int kg = kt0 + 16 * g;
+        const bf16* vbase = nullptr;
+        if (kg < kv_end && kg + 16 > kv_begin)
+            vbase = (const bf16*)a.v_pages + ((size_t)bt[kg / bs] * a.nkv + kvh) * hd * bs + kg % bs;
+        uint4 vv[EARLY_V ? CB : 1][2];
+        if (EARLY_V) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int d = 16 * cb + li;
+                vv[cb][0] = vv[cb][1] = make_uint4(0, 0, 0, 0);
+                if (vbase && d < hd) {
+                    vv[cb][0] = *(const uint4*)(vbase + (size_t)d * bs);
+                    vv[cb][1] = *(const uint4*)(vbase + (size_t)d * bs + 8);
+                }
+            }
+        }
         f32x4_t sc[4];
+        uint4 kf[4][KS];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
             const int key = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
             const bf16* kr = nullptr;
             if (key >= kv_begin && key < kv_end)
@@ -289,9 +308,15 @@ struct WaveAttn {
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
                 const int d = 32 * u + 8 * g;
-                const uint4 v = (kr && d < hd) ? *(const uint4*)(kr + d) : make_uint4(0, 0, 0, 0);
-                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, v), qf[u], sc[kb], 0, 0, 0);
+                kf[kb][u] = (kr && d < hd) ? *(const uint4*)(kr + d) : make_uint4(0, 0, 0, 0);
             }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < KS; ++u)
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[kb][u]), qf[u], sc[kb], 0, 0, 0);
         }
         // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
         float mt = NEG_INF;
@@ -328,18 +353,19 @@ struct WaveAttn {
         float al[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
-        // values: 16 consecutive keys kt0 + 16g .. of transposed row d = 16*cb + li
-        const int kg = kt0 + 16 * g;
-        const bool vload = kg < kv_end && kg + 16 > kv_begin;
-        const bf16* vbase = nullptr;
-        if (vload) vbase = (const bf16*)a.v_pages + ((size_t)bt[kg / bs] * a.nkv + kvh) * hd * bs + kg % bs;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
-            const int d = 16 * cb + li;
-            uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
-            if (vbase && d < hd) {
-                v0 = *(const uint4*)(vbase + (size_t)d * bs);
-                v1 = *(const uint4*)(vbase + (size_t)d * bs + 8);
+            uint4 v0, v1;
+            if (EARLY_V) {
+                v0 = vv[cb][0];
+                v1 = vv[cb][1];
+            } else {
+                const int d = 16 * cb + li;
+                v0 = v1 = make_uint4(0, 0, 0, 0);
+                if (vbase && d < hd) {
+                    v0 = *(const uint4*)(vbase + (size_t)d * bs);
+                    v1 = *(const uint4*)(vbase + (size_t)d * bs + 8);
+                }
             }
             f32x4_t acc = o[cb];
 #pragma unroll

@@ -105,13 +105,18 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         k_dst = k_pages + (size_t)page * nkv * bs * hd;
         v_dst = v_pages + (size_t)page * nkv * hd * bs;
     }
+    // one (cos, sin) per rotated pair of this token, shared by all heads
+    __shared__ float cs_s[512], sn_s[512];
+    for (int p = threadIdx.x; p < half; p += 256) {
+        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
+        sincosf((float)pos * freq, &sn_s[p], &cs_s[p]);
+    }
+    __syncthreads();
     // rotated pairs of q (in place) and k (into the page)
     const int n_pairs = (nh + nkv) * half;
     for (int i = threadIdx.x; i < n_pairs; i += 256) {
         const int head = i / half, p = i % half;
-        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
-        float sn, cs;
-        sincosf((float)pos * freq, &sn, &cs);
+        const float cs = cs_s[p], sn = sn_s[p];
         const int ia = interleaved ? 2 * p : p;
         const int ib = interleaved ? 2 * p + 1 : p + half;
         if (head < nh) {
@@ -146,7 +151,7 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
                             const int* block_table, int max_blocks, void* k_pages, void* v_pages,
                             int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
     FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
-    FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
+    FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0 && rot <= 1024, "rope_kv_write: rotary dim %d must be even, <= head_dim %d and <= 1024", rot, hd);
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;

@@ -1,6 +1,6 @@
 // Routing of tokens to experts.
 //
-//  fx_router_topk : router logits (float32 sums), a gating function over all
+//  fx_router_select : from float32 router logits, a gating function over all
 //                   experts, the k best, optional renormalisation; and the
 //                   scalar sigmoid gate of a shared expert.
 //  fx_moe_align   : sorts the (token, slot) pairs by expert with a stable
@@ -16,93 +16,41 @@ FX_DEFINE_LAST_ERROR()
 
 enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
 
-// One block of 256 threads per token.
-//   logits[e] = sum_c x[c] * Wr[e, c]            (no bias; ferrox-models/src/decoder.rs:2915)
+// One wave per token, four tokens per block.  Input: float32 router logits
+// [T, ld] (products of the activations with the router matrix, no bias;
+// ferrox-models/src/decoder.rs:2915), optionally with the shared expert's gate
+// logit in column E.
 //   softmax over all E with max subtraction, then the k largest probabilities,
 //   weights = those probabilities, divided by their sum if `renorm`
 //   (ferrox-moe/src/lib.rs:333-355).  Ties: higher probability first, then the
 //   lower expert index (the rule of ferrox-metal/src/gpu.rs:686-699).
 //   GATE_SIGMOID scores each expert with 1/(1+exp(-logit)) instead
 //   (ferrox-moe/src/lib.rs:100-121).
-//   gate_out[t] = sigmoid(sum_c x[c] * shared_gate[c])  (decoder.rs:2670-2672).
-template <typename T>
-__global__ __launch_bounds__(256) void router_topk_kernel(
-    const T* __restrict__ x, long ldx, const void* __restrict__ Wr, int w_dtype,
-    const void* __restrict__ shared_gate, int sg_dtype, int H, int E, int k, int renorm, int gating,
-    int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ gate_out) {
-    extern __shared__ float xs[];         // H floats
-    __shared__ float score[E_MAX];
-    __shared__ float red[4];
-    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int c = tid; c < H; c += 256) xs[c] = to_float(x[(size_t)t * ldx + c]);
-    __syncthreads();
-    // four experts at a time per wave, 8 weights per lane and step, so that many loads are in flight;
-    // the order of the sums depends on H alone
-    const bool vec = (H % 8 == 0) && (((uintptr_t)Wr) % 16 == 0);
-    for (int e0 = wave * 4; e0 < E; e0 += 16) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        if (vec) {
-            for (int c = lane * 8; c < H; c += 512) {
-                float xv[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) xv[i] = xs[c + i];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int e = e0 + j;
-                    if (e >= E) continue;
-                    if (w_dtype == FX_BF16) {
-                        const uint4 v = *(const uint4*)((const bf16*)Wr + (size_t)e * H + c);
-                        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            acc[j] = fmaf(xv[2 * i], __uint_as_float(u[i] << 16), acc[j]);
-                            acc[j] = fmaf(xv[2 * i + 1], __uint_as_float(u[i] & 0xffff0000u), acc[j]);
-                        }
-                    } else {
-                        const float4 a = *(const float4*)((const float*)Wr + (size_t)e * H + c);
-                        const float4 b = *(const float4*)((const float*)Wr + (size_t)e * H + c + 4);
-                        acc[j] = fmaf(xv[0], a.x, acc[j]); acc[j] = fmaf(xv[1], a.y, acc[j]);
-                        acc[j] = fmaf(xv[2], a.z, acc[j]); acc[j] = fmaf(xv[3], a.w, acc[j]);
-                        acc[j] = fmaf(xv[4], b.x, acc[j]); acc[j] = fmaf(xv[5], b.y, acc[j]);
-                        acc[j] = fmaf(xv[6], b.z, acc[j]); acc[j] = fmaf(xv[7], b.w, acc[j]);
-                    }
-                }
-            }
-        } else {
-            for (int c = lane; c < H; c += 64)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (e0 + j < E) acc[j] = fmaf(xs[c], load_as_float(Wr, w_dtype, (size_t)(e0 + j) * H + c), acc[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float v = wave_sum(acc[j]);
-            if (lane == 0 && e0 + j < E) score[e0 + j] = v;
-        }
-    }
-    if (shared_gate) {
-        float acc = 0.f;
-        for (int c = tid; c < H; c += 256) acc = fmaf(xs[c], load_as_float(shared_gate, sg_dtype, c), acc);
-        acc = block_sum<4>(acc, red);
-        if (tid == 0) gate_out[t] = 1.0f / (1.0f + expf(-acc));
-    }
-    __syncthreads();
-    if (wave != 0) return;
-    // gating over all experts, by one wave
+//   gate_out[t] = sigmoid(logits[t, E])  (decoder.rs:2670-2672).
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, int T, int E,
+                                                            int k, int renorm, int gating, int* __restrict__ ids,
+                                                            float* __restrict__ weights, float* __restrict__ gate_out) {
+    __shared__ float score_all[4][E_MAX];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;
+    float* score = score_all[wave];
+    const float* row = logits + (size_t)t * ld;
+    if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E]));
     if (gating == GATE_SOFTMAX) {
         float mx = NEG_INFINITY_F;
-        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, score[e]);
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, row[e]);
         mx = wave_max(mx);
         float sum = 0.f;
         for (int e = lane; e < E; e += 64) {
-            const float ex = expf(score[e] - mx);
+            const float ex = expf(row[e] - mx);
             score[e] = ex;
             sum += ex;
         }
         sum = wave_sum(sum);
         for (int e = lane; e < E; e += 64) score[e] = score[e] / sum;
     } else {
-        for (int e = lane; e < E; e += 64) score[e] = 1.0f / (1.0f + expf(-score[e]));
+        for (int e = lane; e < E; e += 64) score[e] = 1.0f / (1.0f + expf(-row[e]));
     }
     __builtin_amdgcn_wave_barrier();
     // k rounds of "largest remaining", lower index on ties
@@ -139,27 +87,17 @@ __global__ __launch_bounds__(256) void router_topk_kernel(
     if (lane < k) weights[t * k + lane] = renorm ? my_w / wsum : my_w;
 }
 
-FX_API int fx_router_topk(void* stream, int x_dtype, const void* x, long ldx, const void* Wr, int w_dtype,
-                          const void* shared_gate, int sg_dtype, int T, int H, int E, int k, int renorm,
-                          int gating, int* ids, float* weights, float* gate_out) {
-    FX_REQUIRE(x_dtype == FX_F32 || x_dtype == FX_BF16, "router: unknown activation dtype %d", x_dtype);
-    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "router: unknown weight dtype %d", w_dtype);
-    FX_REQUIRE(T >= 0 && H > 0, "router: bad sizes T=%d H=%d", T, H);
+FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, int E, int k, int renorm,
+                            int gating, int* ids, float* weights, float* gate_out) {
+    FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
     FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
     FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
-    FX_REQUIRE(H <= 12288, "router: hidden size %d exceeds this kernel's 12288", H);
+    FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
-    FX_REQUIRE(!shared_gate || gate_out, "router: shared gate given without an output");
     if (T == 0) return 0;
-    hipStream_t s = (hipStream_t)stream;
-    const size_t shm = (size_t)H * sizeof(float);
-    if (x_dtype == FX_F32)
-        router_topk_kernel<float><<<T, 256, shm, s>>>((const float*)x, ldx, Wr, w_dtype, shared_gate, sg_dtype, H, E, k,
-                                                      renorm, gating, ids, weights, gate_out);
-    else
-        router_topk_kernel<bf16><<<T, 256, shm, s>>>((const bf16*)x, ldx, Wr, w_dtype, shared_gate, sg_dtype, H, E, k,
-                                                     renorm, gating, ids, weights, gate_out);
-    FX_CHECK_LAUNCH("router_topk");
+    router_select_kernel<<<(T + 3) / 4, 256, 0, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
+                                                                     gate_out);
+    FX_CHECK_LAUNCH("router_select");
     return 0;
 }
 

@@ -62,8 +62,8 @@ _sigs = {
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
                                       c_void_p, c_void_p, c_int, c_int],
-    ("moe", "fx_router_topk"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int,
-                                c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+                                  c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
@@ -247,7 +247,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
         chunk = 256
         if q.dtype == torch.bfloat16:
             pairs = n * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
-            want = max(1, 2048 // max(1, pairs))
+            want = max(1, 4096 // max(1, pairs))
             chunk = 64
             while chunk < 4096 and -(-max_kv_len // chunk) > want:
                 chunk *= 2
@@ -261,18 +261,19 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
           _p(part_o), _p(part_ml), splits, chunk)
 
 
-def router_topk(x, router_w, top_k, renorm, gating=GATE_SOFTMAX, shared_gate=None):
-    """Returns (ids int32 [T,k], weights float32 [T,k], gate float32 [T] or None)."""
-    T, H = x.shape
-    E = router_w.shape[0]
-    if router_w.shape[1] != H or not router_w.is_contiguous() or x.stride(1) != 1:
-        raise KernelError("router: weight must be contiguous [E, H] and x [T, H]")
-    ids = torch.empty((T, top_k), dtype=torch.int32, device=x.device)
-    weights = torch.empty((T, top_k), dtype=torch.float32, device=x.device)
-    gate = torch.empty((T,), dtype=torch.float32, device=x.device) if shared_gate is not None else None
-    _call("moe", "fx_router_topk", _stream(), dtype_code(x.dtype), _p(x), x.stride(0), _p(router_w),
-          dtype_code(router_w.dtype), _p(shared_gate), dtype_code(shared_gate.dtype) if shared_gate is not None else 0,
-          T, H, E, top_k, 1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
+def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+    """From float32 router logits [T, >= E (+1)]: (ids int32 [T,k], weights float32 [T,k],
+    gate float32 [T] = sigmoid(logits[:, E]) or None)."""
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("router_select: logits must be float32 [T, E] with unit inner stride")
+    T = logits.shape[0]
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
+    gate = torch.empty((T,), dtype=torch.float32, device=logits.device) if has_gate else None
+    if logits.shape[1] < n_experts + (1 if has_gate else 0):
+        raise KernelError(f"router_select: {logits.shape[1]} columns for {n_experts} experts")
+    _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), T, n_experts, top_k,
+          1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
     return ids, weights, gate
 
 

@@ -36,7 +36,7 @@ class SparseMoE(FeedForward):
         self.norm_topk_prob, self.gating = bool(norm_topk_prob), GATINGS[gating]
         self.shared = SwiGLU(hidden_size, shared_intermediate_size) if shared_intermediate_size > 0 else None
         self.has_shared_gate = bool(shared_gate) and self.shared is not None
-        self.router = self.w_gate_up = self.w_down = self.shared_gate_w = None
+        self.router = self.w_gate_up = self.w_down = None
 
     def children(self):
         return [("shared_expert.", self.shared)] if self.shared is not None else []
@@ -53,7 +53,7 @@ class SparseMoE(FeedForward):
         return specs
 
     def load(self, fetch):
-        self.router = fetch("gate.weight").contiguous()
+        router = fetch("gate.weight")
         gu, dn = [], []
         for e in range(self.n_experts):
             gu.append(torch.cat(same_dtype([fetch(f"experts.{e}.gate_proj.weight"),
@@ -61,13 +61,15 @@ class SparseMoE(FeedForward):
             dn.append(fetch(f"experts.{e}.down_proj.weight"))
         self.w_gate_up = torch.stack(same_dtype(gu)).contiguous()     # [E, 2*I, H]
         self.w_down = torch.stack(same_dtype(dn)).contiguous()        # [E, H, I]
-        if self.has_shared_gate:
-            self.shared_gate_w = fetch("shared_expert_gate.weight").reshape(-1).contiguous()
+        if self.has_shared_gate:     # the gate's row rides along as column E of the router product
+            router = torch.cat(same_dtype([router, fetch("shared_expert_gate.weight").reshape(1, -1)]), dim=0)
+        self.router = router.contiguous()
 
     def forward(self, x, ctx, residual) -> None:
         T = x.shape[0]
-        ids, weights, gate = ops.router_topk(x, self.router, self.top_k, self.norm_topk_prob, self.gating,
-                                             self.shared_gate_w)
+        logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
+        ids, weights, gate = ops.router_select(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
+                                               self.has_shared_gate)
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
         offsets, sorted_token, inv = ops.moe_align(ids, self.n_experts)

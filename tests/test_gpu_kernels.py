@@ -192,9 +192,11 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
 @pytest.mark.parametrize("T,H,E,k,renorm", [(1, 64, 8, 2, False), (7, 96, 6, 3, True), (33, 200, 60, 4, False),
                                              (5, 128, 130, 8, True), (4, 72, 5, 5, False)])
 def test_router(dtype, T, H, E, k, renorm):
+    """router matrix product + selection, with the shared expert's gate as an extra row"""
     from ferrox_amd import ops
     x, wr, sg = rnd(T, H, dtype=dtype), rnd(E, H, dtype=dtype, seed=1, scale=0.3), rnd(H, dtype=dtype, seed=2, scale=0.2)
-    ids, w, gate = ops.router_topk(x, wr, k, renorm, shared_gate=sg)
+    logits = ops.gemm(x, torch.cat([wr, sg[None]]).contiguous(), epilogue=ops.EPI_STORE_F32)
+    ids, w, gate = ops.router_select(logits, E, k, renorm, has_gate=True)
     xd, wd = x.double().cpu(), wr.double().cpu()
     for t in range(T):
         want_ids, want_w = plain.route_top_k(wd @ xd[t], k, renorm)
@@ -207,18 +209,19 @@ def test_router_golden_vector():
     """logits 1..8, k=3, no renormalisation -> experts [7, 6, 5], weights [0.6323223, 0.2326232,
     0.0855683] (the vector of the reference's own test, ferrox-moe/src/lib.rs:863-893)."""
     from ferrox_amd import ops
-    x = torch.zeros(1, 8, device=DEV)
-    x[0, 0] = 1.0
-    wr = torch.zeros(8, 8, device=DEV)
-    wr[:, 0] = torch.arange(1, 9, dtype=torch.float32)
-    ids, w, _ = ops.router_topk(x, wr, 3, False)
+    logits = torch.arange(1, 9, dtype=torch.float32, device=DEV)[None].contiguous()
+    ids, w, _ = ops.router_select(logits, 8, 3, False)
     assert ids[0].tolist() == [7, 6, 5]
     assert torch.allclose(w[0].cpu(), torch.tensor([0.6323223, 0.2326232, 0.0855683]), atol=1e-4)   # its tolerance
     assert abs(float(w[0].sum()) - 0.9505138) < 1e-4
     exact = torch.softmax(torch.arange(1, 9, dtype=torch.float64), 0).flip(0)[:3]
     assert torch.allclose(w[0].cpu().double(), exact, atol=1e-6)
-    ids, w, _ = ops.router_topk(x, torch.zeros(8, 8, device=DEV), 3, True)      # all equal: lowest indices
+    ids, w, _ = ops.router_select(logits, 8, 3, True)              # renormalised: the same experts, sum 1
+    assert ids[0].tolist() == [7, 6, 5] and abs(float(w[0].sum()) - 1.0) < 1e-6
+    ids, w, _ = ops.router_select(torch.zeros(1, 8, device=DEV), 8, 3, True)     # all equal: lowest indices
     assert ids[0].tolist() == [0, 1, 2] and torch.allclose(w[0].cpu(), torch.full((3,), 1 / 3))
+    ids, w, _ = ops.router_select(torch.tensor([[0.1, 5.0, 0.2, 3.0, -1.0]], device=DEV), 5, 2, False)
+    assert ids[0].tolist() == [1, 3]                               # ferrox-moe/src/lib.rs:834-841
 
 
 def test_sampling_kernel():
