@@ -120,11 +120,17 @@ class CacheManager:
     def __contains__(self, req) -> bool:
         return req in self.seqs
 
+    def _seq(self, req) -> Sequence:
+        seq = self.seqs.get(req)
+        if seq is None:
+            raise ValueError(f"request {req!r} is not admitted")
+        return seq
+
     def length(self, req) -> int:
-        return self.seqs[req].length
+        return self._seq(req).length
 
     def slot(self, req) -> int:
-        return self.seqs[req].slot
+        return self._seq(req).slot
 
     def table(self, req, key) -> list:
         return self.groups[key].tables[req]
@@ -142,7 +148,7 @@ class CacheManager:
 
     def extend(self, req, new_len: int) -> bool:
         """Pages for positions [length, new_len) in every group, all or nothing; sets the length."""
-        seq = self.seqs[req]
+        seq = self._seq(req)
         if new_len < seq.length:
             raise ValueError("a sequence cannot shrink")
         need = self.pages_needed(req, new_len)
@@ -158,7 +164,7 @@ class CacheManager:
         """Give back pages that a window has passed: every query from now on stands at
         position >= length and sees keys t with position - t < W, so t >= length - W + 1.
         Returns the number of pages freed."""
-        seq = self.seqs[req]
+        seq = self._seq(req)
         freed = 0
         for g in self.groups.values():
             if g.window is None:

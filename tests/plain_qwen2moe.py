@@ -128,6 +128,17 @@ def router_margin(logits: torch.Tensor, k: int) -> float:
     return float((p[k - 1] - p[k]) / p[k - 1])
 
 
+def combine_expert_outputs(routed, shared, hidden_dim: int, dtype=torch.float64) -> torch.Tensor:
+    """sum of weight * routed output in the given order, then the shared outputs
+    (ferrox-moe/src/lib.rs:735-752).  `routed`: list of (vector, weight)."""
+    out = torch.zeros(hidden_dim, dtype=dtype)
+    for vec, weight in routed:
+        out = out + vec * weight
+    for vec in shared:
+        out = out + vec
+    return out
+
+
 def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w, margins=None):
     """One token through the sparse block.
 
@@ -141,18 +152,15 @@ def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w
     ids, w = route_top_k(logits, k, norm_topk_prob)
     if margins is not None:
         margins.append(router_margin(logits, k))
-    out = torch.zeros_like(x)
-    for j, e in enumerate(ids):
-        g, u, d = experts[e]
-        out = out + swiglu_mlp(x, g, u, d) * w[j]
+    routed = [(swiglu_mlp(x, *experts[e]), w[j]) for j, e in enumerate(ids)]
+    shared_out = []
     if shared is not None:
-        g, u, d = shared
-        y = swiglu_mlp(x, g, u, d)
+        y = swiglu_mlp(x, *shared)
         if shared_gate_w is not None:
             z = (shared_gate_w.reshape(-1) * x).sum()
             y = y * (1.0 / (1.0 + torch.exp(-z)))
-        out = out + y
-    return out
+        shared_out.append(y)
+    return combine_expert_outputs(routed, shared_out, x.shape[0], x.dtype)
 
 
 # --------------------------------------------------------------------------

@@ -1,0 +1,118 @@
+"""The cache manager: no page lost, held twice or freed twice, under random orders of requests."""
+import random
+
+import pytest
+
+from ferrox_amd.cache import CacheManager, PagePool, StateSlots
+
+FULL, WIN = ("full",), ("window", 16)
+
+
+def test_pool_hands_out_and_takes_back():
+    pool = PagePool(4)
+    a = pool.alloc(3)
+    assert a == [0, 1, 2] and pool.n_free == 1
+    assert pool.alloc(2) is None and pool.n_free == 1              # all or nothing, nothing changed
+    pool.free([1])
+    assert pool.alloc(1) == [1]                                    # the page just freed is used again first
+    with pytest.raises(ValueError):
+        pool.free([3])                                             # never handed out
+    pool.free([0])
+    with pytest.raises(ValueError):
+        pool.free([0])                                             # freed twice
+    with pytest.raises(ValueError):
+        pool.free([9])
+
+
+def test_slots():
+    s = StateSlots(2)
+    a, b = s.alloc(), s.alloc()
+    assert {a, b} == {0, 1} and s.alloc() is None
+    s.free(a)
+    assert s.alloc() == a
+    with pytest.raises(ValueError):
+        s.free(5)
+
+
+def test_extend_is_all_or_nothing_across_groups():
+    m = CacheManager({FULL: None, WIN: 16}, {FULL: 4, WIN: 2}, block_size=8, n_slots=2)
+    assert m.admit("a") == 0
+    assert m.extend("a", 16) and m.length("a") == 16               # 2 pages in both groups
+    before = (m.n_free_pages(FULL), m.n_free_pages(WIN), list(m.table("a", FULL)))
+    assert not m.can_extend("a", 17) and not m.extend("a", 17)     # the windowed pool is empty
+    assert (m.n_free_pages(FULL), m.n_free_pages(WIN), list(m.table("a", FULL))) == before and m.length("a") == 16
+    m.check_invariants()
+    m.release("a")
+    m.release("a")                                                 # twice is fine (cache.rs:131-139)
+    assert m.n_free_pages(FULL) == 4 and m.n_free_pages(WIN) == 2 and m.slots.n_free == 2
+    with pytest.raises(ValueError):
+        m.extend("a", 4)
+
+
+def test_window_gives_pages_back_when_they_are_passed():
+    m = CacheManager({FULL: None, WIN: 16}, 16, block_size=8, n_slots=1)
+    m.admit("r")
+    m.extend("r", 40)
+    assert m.trim("r") == 3                   # next query stands at 40 and sees 25..40: blocks 0, 1, 2 are passed
+    assert m.table("r", WIN)[:3] == [-1, -1, -1] and all(p >= 0 for p in m.table("r", WIN)[3:])
+    assert all(p >= 0 for p in m.table("r", FULL))                 # the full group keeps everything
+    assert m.trim("r") == 0
+    m.extend("r", 41)
+    assert m.trim("r") == 0                   # first key still needed is 26, in block 3
+    m.extend("r", 47)
+    assert m.trim("r") == 1                   # 47 - 16 + 1 = 32: block 3 is passed
+    m.check_invariants()
+    m.release("r")
+    assert m.n_free_pages(WIN) == 16 and m.n_free_pages(FULL) == 16
+
+
+def test_pages_of_a_finished_request_are_used_again():
+    m = CacheManager({FULL: None}, 3, block_size=4, n_slots=2)
+    m.admit("a")
+    m.extend("a", 12)
+    pages = list(m.table("a", FULL))
+    m.admit("b")
+    assert not m.extend("b", 1)
+    m.release("a")
+    assert m.extend("b", 12) and sorted(m.table("b", FULL)) == sorted(pages)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_the_invariants(seed):
+    rng = random.Random(seed)
+    m = CacheManager({FULL: None, WIN: 16, ("window", 40): 40}, {FULL: 40, WIN: 12, ("window", 40): 20},
+                     block_size=rng.choice([4, 8, 16]), n_slots=4)
+    live, next_id = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            rid = f"r{next_id}"
+            next_id += 1
+            if m.admit(rid) is not None:
+                live[rid] = 0
+            else:
+                assert len(live) == 4
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 5, 13, 30])
+            had = {k: m.n_free_pages(k) for k in m.groups}
+            if m.extend(rid, live[rid] + n):
+                live[rid] += n
+                m.trim(rid)
+            else:
+                assert {k: m.n_free_pages(k) for k in m.groups} == had
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check_invariants()
+        for rid, n in live.items():
+            assert m.length(rid) == n
+            # every position a later query can see has a page in every group
+            for g in m.groups.values():
+                first = 0 if g.window is None else max(0, n - g.window + 1)
+                assert all(g.tables[rid][b] >= 0 for b in range(first // m.block_size, m.blocks_for(n)))
+    for rid in list(live):
+        m.release(rid)
+    m.check_invariants()
+    assert all(g.pool.n_free == g.pool.num_pages for g in m.groups.values()) and m.slots.n_free == 4
