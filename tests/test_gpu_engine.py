@@ -136,3 +136,149 @@ def test_greedy_generation_through_the_entry_point(model_folders, name):
     got = engine.generate(prompts, max_new_tokens=16, temperature=0.0)
     for p, g in zip(prompts, got):
         assert g == plain.greedy_generate(cfg, w, p, 16)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_windows_and_pages(model_folders, dtype):
+    """a short prompt, then 200 tokens one by one: windowed layers give pages back on the way and the
+    pool holds fewer pages than the sequence is long"""
+    cfg, seed = TINY["B"]
+    reqs = ru.make_requests(cfg["vocab_size"], [230], 77)
+    toks = reqs["r0"]
+    steps = [{"entries": [{"id": "r0", "tokens": toks[:30], "want": list(range(30))}], "end": []}]
+    steps += [{"entries": [{"id": "r0", "tokens": [t], "want": [0]}], "end": []} for t in toks[30:]]
+    steps[-1]["end"] = ["r0"]
+    folder, runner = runner_for(model_folders, "B", dtype, block_size=8, num_pages={("full",): 29, ("window", 16): 7})
+    got = ru.run_trace(runner, steps)
+    ru.compare(got, folder, reqs, *TOL[dtype], f"B {dtype} long decode", MARGIN[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(model_folders, name, dtype):
+    """prompts of one and two tokens, and the first positions decoded from an empty cache"""
+    cfg, seed = TINY[name]
+    reqs = ru.make_requests(cfg["vocab_size"], [1, 2, 5], 9)
+    folder, runner = runner_for(model_folders, name, dtype, block_size=16, num_pages=8)
+    got = ru.run_trace(runner, ru.trace_whole(reqs))
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} first tokens", MARGIN[dtype])
+    got = ru.run_trace(runner, ru.trace_tail_decode(reqs))          # every token alone, from position 0
+    ru.compare(got, folder, reqs, *TOL[dtype], f"{name} {dtype} first tokens one by one", MARGIN[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_stale_pages_are_never_read(model_folders, dtype):
+    """every page is filled with large values before the trace and pages are used again during it"""
+    reqs = requests_for("B")
+    steps = ru.trace_mixed(reqs, seed=11)
+    pages = ru.max_live_tokens(steps, 16) // 16
+    folder, runner = runner_for(model_folders, "B", dtype, block_size=16, num_pages=pages)
+    for c in runner.storage.caches:
+        for t in c.pages.values():
+            t.fill_(3.0e4)
+    got = ru.run_trace(runner, steps)
+    ru.compare(got, folder, reqs, *TOL[dtype], f"B {dtype} mixed over poisoned pages", MARGIN[dtype])
+
+
+def test_far_key_and_window_edge_stand_out(model_folders):
+    """A key hundreds of positions back whose score is made to stand out must be found (decode and
+    prefill kernels, across page edges); with a window, the key at distance W-1 is seen and the
+    one at distance W is not."""
+    import math
+    from ferrox_amd import ops
+    dev = "cuda:0"
+    for dtype in (torch.float32, torch.bfloat16):
+        for bs, window, L in ((16, 0, 700), (64, 0, 700), (8, 0, 300), (16, 100, 700), (64, 257, 700)):
+            nh, nkv, hd = 4, 2, 64
+            g = torch.Generator().manual_seed(L + bs)
+            n_pages = -(-L // bs) + 2
+            perm = torch.randperm(n_pages, generator=g)
+            table = perm[: -(-L // bs)].to(torch.int32)[None].contiguous().to(dev)
+            k = torch.randn(L, nkv, hd, generator=g) * 0.1
+            v = torch.randn(L, nkv, hd, generator=g)
+            last = L - 1
+            targets = [3, last - (333 if L > 400 else 150)] if not window else [last - window + 1, last - window]
+            q = torch.zeros(1, nh, hd)
+            for ti, tpos in enumerate(targets):
+                # head pair (2*ti, 2*ti+1) reads kv head ti: one large coordinate shared by query and target key
+                k[tpos, ti, :] = 0.0
+                k[tpos, ti, 5 + ti] = 30.0
+                q[0, 2 * ti: 2 * ti + 2, 5 + ti] = 30.0
+            k_pages = torch.zeros(n_pages, nkv, bs, hd)
+            v_pages = torch.zeros(n_pages, nkv, hd, bs)
+            for p in range(L):
+                pg = int(table[0, p // bs])
+                k_pages[pg, :, p % bs, :] = k[p]
+                v_pages[pg, :, :, p % bs] = v[p]
+            k_pages, v_pages = k_pages.to(dtype).to(dev), v_pages.to(dtype).to(dev)
+            qd = q.reshape(1, nh * hd).to(dtype).to(dev)
+            pos = torch.tensor([last], dtype=torch.int32, device=dev)
+            zero = torch.zeros(1, dtype=torch.int32, device=dev)
+            one = torch.ones(1, dtype=torch.int32, device=dev)
+            ref = plain_attention_last(q[0].double(), k_pages, v_pages, table, bs, L, nh, nkv, window)
+            for kernel in ("decode", "tiles"):
+                out = torch.zeros(1, nh * hd, dtype=dtype, device=dev)
+                if kernel == "decode":
+                    ops.attention_decode(qd, out, k_pages, v_pages, table, pos, zero, zero, nh, nkv, hd, bs, window,
+                                         1.0 / math.sqrt(hd), max_kv_len=L)
+                else:
+                    ops.attention_tiles(qd, out, k_pages, v_pages, table, pos, zero, zero, one, nh, nkv, hd, bs, window,
+                                        1.0 / math.sqrt(hd))
+                out = out.double().cpu().reshape(nh, hd)
+                tol = 1e-4 if dtype == torch.float32 else 2e-2
+                assert float((out - ref).abs().max()) < tol, (dtype, bs, window, kernel)
+                vv = v_pages.double().cpu()
+                seen = vv[int(table[0, targets[0] // bs]), 0, :, targets[0] % bs]
+                assert float((out[0] - seen).abs().max()) < tol, "the far key was not found"
+                hidden = vv[int(table[0, targets[1] // bs]), 1, :, targets[1] % bs]
+                if window:
+                    assert float((out[2] - hidden).abs().max()) > 0.3, "a key beyond the window was seen"
+                else:
+                    assert float((out[2] - hidden).abs().max()) < tol
+
+
+def plain_attention_last(q, k_pages, v_pages, table, bs, L, nh, nkv, window):
+    """the plain attention of the last position, from what the pages hold"""
+    import plain_qwen2moe as plain
+    kp, vp = k_pages.double().cpu(), v_pages.double().cpu()
+    ks = torch.stack([kp[int(table[0, p // bs]), :, p % bs, :] for p in range(L)])
+    vs = torch.stack([vp[int(table[0, p // bs]), :, :, p % bs] for p in range(L)])
+    qs = torch.zeros(L, nh, q.shape[-1], dtype=torch.float64)
+    qs[-1] = q
+    return plain.causal_attention(qs, ks, vs, nh, nkv, window or None)[-1]
+
+
+def test_preemption_and_seeded_sampling_through_the_entry_point(model_folders):
+    """a pool too small for all requests: the youngest is preempted and recomputed, and every
+    request still produces the tokens it produces alone; temperature sampling is seeded per request"""
+    from ferrox_amd.engine.api import Engine
+    from ferrox_amd.sampling import SamplingParams
+    import plain_qwen2moe as plain
+    folder = model_folders("B", "float32")
+    cfg, w = plain.load_folder(folder)
+    prompts = list(ru.make_requests(cfg["vocab_size"], [3, 17, 40, 64, 90, 120], 6).values())
+    roomy = Engine(folder, dtype="float32", block_size=8, num_pages=200, max_seqs=6, max_tokens_per_step=48, prefill_chunk=24)
+    tight = Engine(folder, dtype="float32", block_size=8, num_pages=34, max_seqs=6, max_tokens_per_step=48, prefill_chunk=24)
+    greedy = roomy.generate(prompts, max_new_tokens=24)
+    assert tight.generate(prompts, max_new_tokens=24) == greedy and tight.last_stats["preemptions"] > 0
+    assert greedy[1] == plain.greedy_generate(cfg, w, prompts[1], 24)
+    params = [SamplingParams(temperature=0.8, seed=100 + i) for i in range(6)]
+    together = [c.token_ids for c in roomy.generate_detailed(prompts, 24, params)]
+    squeezed = [c.token_ids for c in tight.generate_detailed(prompts, 24, params)]
+    alone = [roomy.generate_detailed([p], 24, [sp])[0].token_ids for p, sp in zip(prompts, params)]
+    assert together == alone == squeezed
+    # the plain sampler on the plain model's logits draws the same tokens
+    rng, toks, out = plain.XorShift64(100), list(prompts[0]), []
+    for _ in range(8):
+        t = plain.sample(plain.forward(cfg, w, toks)[-1].tolist(), rng, temperature=0.8)
+        out.append(t)
+        toks.append(t)
+    assert together[0][:8] == out
+    full = [SamplingParams(temperature=0.9, top_k=20, top_p=0.9, repetition_penalty=1.2, seed=5)]
+    rng, toks, out = plain.XorShift64(5), list(prompts[2]), []
+    for _ in range(8):
+        t = plain.sample(plain.forward(cfg, w, toks)[-1].tolist(), rng, temperature=0.9, top_k=20, top_p=0.9,
+                         repetition_penalty=1.2, history=out)
+        out.append(t)
+        toks.append(t)
+    assert roomy.generate_detailed([prompts[2]], 8, full)[0].token_ids == out

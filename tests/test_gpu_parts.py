@@ -1,0 +1,265 @@
+"""Parts alone and put together from data: each built-in part in a model of its own beside
+stand-in parts defined here, a mixer with state of its own registered from outside the package,
+layer orders that name a layer twice or read another layer's cache."""
+import math
+import os
+
+import pytest
+import torch
+
+import plain_qwen2moe as plain
+import replay_util as ru
+from ferrox_amd import ops
+from ferrox_amd.engine.model import Model
+from ferrox_amd.engine.runner import ModelRunner, StepEntry
+from ferrox_amd.parts import (FEED_FORWARDS, MIXERS, FeedForward, LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec,
+                              ScheduleEntry)
+from ferrox_amd.weights import RandomSource
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ---- stand-ins, defined outside the package -----------------------------------------
+@FEED_FORWARDS.register("test_no_ffn")
+class NoFFN(FeedForward):
+    def __init__(self, hidden_size: int = 0):
+        pass
+
+    def forward(self, x, ctx, residual):
+        return None
+
+
+@MIXERS.register("test_no_mixer")
+class NoMixer(Mixer):
+    def __init__(self, hidden_size: int = 0):
+        pass
+
+    def forward(self, x, ctx, cache, residual):
+        return None
+
+
+@MIXERS.register("test_running_mean")
+class RunningMean(Mixer):
+    """y_t = W * mean(x_0 .. x_t): a mixer whose whole memory is a fixed-size state per request
+    (the running sum), kept in a state slot; written with torch operations."""
+
+    def __init__(self, hidden_size: int):
+        self.hidden_size = hidden_size
+        self.weight = None
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec((self.hidden_size, self.hidden_size))}
+
+    def load(self, fetch):
+        self.weight = fetch("mix.weight")
+
+    def state_shapes(self):
+        return {"sum": ((self.hidden_size,), torch.float32)}
+
+    def forward(self, x, ctx, cache, residual):
+        state = cache.state["sum"]
+        for s in range(ctx.n_seqs):
+            b, e = ctx.q_starts[s], ctx.q_starts[s + 1]
+            run = state[ctx.slots[s]] + torch.cumsum(x[b:e].float(), 0)
+            state[ctx.slots[s]] = run[-1]
+            mean = run / (ctx.positions[b:e].float()[:, None] + 1.0)
+            y = mean.to(self.weight.dtype) @ self.weight.T
+            ops.residual_add(residual[b:e], y.contiguous())
+
+
+def norm(H, eps, prefix):
+    return PartSpec("rmsnorm", {"size": H, "eps": eps}, prefix=prefix)
+
+
+def spec_of(H, V, layers, schedule=None, eps=1e-5):
+    return ModelSpec(hidden_size=H, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H}, prefix="emb."),
+                     layers=layers, schedule=schedule or [ScheduleEntry(i) for i in range(len(layers))],
+                     final_norm=norm(H, eps, "norm."), head=PartSpec("linear_head", {"vocab_size": V, "hidden_size": H}, prefix="head."),
+                     max_positions=4096)
+
+
+def layer(i, H, mixer, ffn, eps=1e-5):
+    return LayerSpec("prenorm", f"l{i}.", {"norm1": norm(H, eps, "n1."), "mixer": mixer, "norm2": norm(H, eps, "n2."), "ffn": ffn})
+
+
+def attention_spec(H, nh, nkv, hd, window=None, theta=1e4, bias=True, kind="rope_neox", rotary_dim=None):
+    return PartSpec("paged_attention", {"hidden_size": H, "n_heads": nh, "n_kv_heads": nkv, "head_dim": hd, "bias": bias,
+                                        "window": window, "position": PartSpec(kind, {"head_dim": hd, "theta": theta,
+                                                                                      "rotary_dim": rotary_dim})}, prefix="attn.")
+
+
+def build(spec, dtype, seed=0, std=0.05):
+    model = Model(spec)
+    src = RandomSource(seed, dtype, DEV, std)
+    model.load(src, dtype, DEV)
+    src_cpu = RandomSource(seed, dtype, "cpu", std)
+    src_cpu.expect(model.named_params())
+    weights = {n: src_cpu.tensor(n).double() for n in src_cpu.names()}
+    return model, weights
+
+
+def run_whole_and_cut(model, toks, block_size=8, num_pages=64):
+    """logits of every position, once as one step and once in portions and single tokens"""
+    runner = ModelRunner(model, block_size=block_size, num_pages=num_pages, max_seqs=4)
+    reqs = {"a": toks}
+    whole = ru.run_trace(runner, ru.trace_whole(reqs))
+    cut = ru.run_trace(runner, ru.trace_mixed(reqs, seed=1, decode_tail=9))
+    return (torch.stack([whole[("a", p)] for p in range(len(toks))]).double(),
+            torch.stack([cut[("a", p)] for p in range(len(toks))]).double())
+
+
+def agree(whole, cut, dtype):
+    """float32: the same bits however the tokens were cut; bfloat16: few rows and many rows go
+    through matrix kernels that sum in different orders"""
+    if dtype == torch.float32:
+        return torch.equal(whole, cut)
+    return float((whole - cut).abs().max()) <= 2e-2 * float(whole.abs().max())
+
+
+def head_of(w, h, eps=1e-5):
+    return plain.rms_norm(h, w["norm.weight"], eps) @ w["head.weight"].T
+
+
+TOKS = [(7 * i + 3) % 50 for i in range(45)]
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_embedding_norm_head_alone(dtype, tol):
+    H, V = 40, 50
+    model, w = build(spec_of(H, V, [layer(0, H, PartSpec("test_no_mixer"), PartSpec("test_no_ffn"))]), dtype)
+    whole, cut = run_whole_and_cut(model, TOKS)
+    want = head_of(w, w["emb.weight"][torch.tensor(TOKS)])
+    assert float((whole - want).abs().max()) < tol * float(want.abs().max()) and agree(whole, cut, dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("nh,nkv,hd,window,rot,kind", [(4, 2, 16, None, None, "rope_neox"), (3, 3, 32, 12, 16, "rope_neox"),
+                                                        (2, 1, 48, 20, None, "rope_interleaved")])
+def test_attention_mixer_alone(dtype, tol, nh, nkv, hd, window, rot, kind):
+    """attention with q/k/v bias, full or partial rotary in either pairing, with and without a window"""
+    H, V, theta, T = 40, 50, 5e3, len(TOKS)
+    model, w = build(spec_of(H, V, [layer(0, H, attention_spec(H, nh, nkv, hd, window, theta, True, kind, rot),
+                                          PartSpec("test_no_ffn"))]), dtype)
+    whole, cut = run_whole_and_cut(model, TOKS, block_size=16)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    x = plain.rms_norm(h, w["l0.n1.weight"], 1e-5)
+    proj = lambda n: x @ w[f"l0.attn.{n}_proj.weight"].T + w[f"l0.attn.{n}_proj.bias"]
+    q, k, v = proj("q").reshape(T, nh, hd), proj("k").reshape(T, nkv, hd), proj("v").reshape(T, nkv, hd)
+    r = rot or hd
+
+    def rotate(t):
+        out = t.clone()
+        for p in range(T):
+            if kind == "rope_neox":
+                out[p, :, :r] = plain.rope_neox(t[p, :, :r], p, theta)
+            else:
+                for i in range(r // 2):
+                    ang = p / (theta ** (2 * i / r))
+                    a, b = t[p, :, 2 * i], t[p, :, 2 * i + 1]
+                    out[p, :, 2 * i], out[p, :, 2 * i + 1] = a * math.cos(ang) - b * math.sin(ang), a * math.sin(ang) + b * math.cos(ang)
+        return out
+
+    att = plain.causal_attention(rotate(q), rotate(k), v, nh, nkv, window)
+    want = head_of(w, h + att.reshape(T, nh * hd) @ w["l0.attn.o_proj.weight"].T)
+    scale = float(want.abs().max())
+    assert float((whole - want).abs().max()) < tol * scale
+    assert float((cut - want).abs().max()) < tol * scale
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_feed_forwards_alone(dtype, tol):
+    H, V = 40, 50
+    dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 56}, prefix="mlp.")
+    moe = PartSpec("sparse_moe", {"hidden_size": H, "n_experts": 5, "top_k": 2, "expert_intermediate_size": 24,
+                                  "norm_topk_prob": True, "shared_intermediate_size": 32}, prefix="moe.")
+    model, w = build(spec_of(H, V, [layer(0, H, PartSpec("test_no_mixer"), dense), layer(1, H, PartSpec("test_no_mixer"), moe)]),
+                     dtype, std=0.2)
+    whole, cut = run_whole_and_cut(model, TOKS)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    x = plain.rms_norm(h, w["l0.n2.weight"], 1e-5)
+    h = h + plain.swiglu_mlp(x, w["l0.mlp.gate_proj.weight"], w["l0.mlp.up_proj.weight"], w["l0.mlp.down_proj.weight"])
+    x = plain.rms_norm(h, w["l1.n2.weight"], 1e-5)
+    ex = [tuple(w[f"l1.moe.experts.{e}.{n}_proj.weight"] for n in ("gate", "up", "down")) for e in range(5)]
+    sh = tuple(w[f"l1.moe.shared_expert.{n}_proj.weight"] for n in ("gate", "up", "down"))
+    margins = []
+    f = torch.stack([plain.moe_ffn_token(x[t], w["l1.moe.gate.weight"], ex, 2, True, sh, w["l1.moe.shared_expert_gate.weight"],
+                                         margins) for t in range(len(TOKS))])
+    want = head_of(w, h + f)
+    keep = [t for t in range(len(TOKS)) if dtype == torch.float32 or margins[t] > 0.01]
+    assert len(keep) > 0.8 * len(TOKS)
+    assert float((whole - want)[keep].abs().max()) < tol * float(want.abs().max()) and agree(whole[keep], cut[keep], dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_a_mixer_with_state_of_its_own(dtype, tol):
+    """registered above, built from a spec and stepped; nothing in the package knows it"""
+    H, V = 32, 50
+    layers = [layer(0, H, PartSpec("test_running_mean", {"hidden_size": H}, prefix="rm."), PartSpec("test_no_ffn")),
+              layer(1, H, attention_spec(H, 2, 2, 16), PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 48}, prefix="mlp."))]
+    model, w = build(spec_of(H, V, layers), dtype)
+    assert model.cache_groups() == {("full",): None}
+    runner = ModelRunner(model, block_size=8, num_pages=32, max_seqs=3)
+    assert runner.storage.caches[0].state["sum"].shape == (3, H) and not runner.storage.caches[0].pages
+    reqs = {"a": TOKS, "b": TOKS[5:30], "c": TOKS[::-1]}
+    whole = ru.run_trace(runner, ru.trace_whole(reqs))
+    mixed = ru.run_trace(runner, ru.trace_mixed(reqs, seed=4, max_live=3))       # slots are taken again, state starts at zero
+    for key in whole:
+        assert float((whole[key] - mixed[key]).abs().max()) <= tol * float(whole[key].abs().max())
+    # against a plain computation of the first layer followed by the rest
+    toks = reqs["a"]
+    T = len(toks)
+    h = w["emb.weight"][torch.tensor(toks)]
+    x = plain.rms_norm(h, w["l0.n1.weight"], 1e-5)
+    mean = torch.cumsum(x, 0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None]
+    h = h + mean @ w["l0.rm.mix.weight"].T
+    x = plain.rms_norm(h, w["l1.n1.weight"], 1e-5)
+    proj = lambda n: x @ w[f"l1.attn.{n}_proj.weight"].T + w[f"l1.attn.{n}_proj.bias"]
+    q, k, v = (plain.rope_neox_rows(proj("q").reshape(T, 2, 16), range(T), 1e4),
+               plain.rope_neox_rows(proj("k").reshape(T, 2, 16), range(T), 1e4), proj("v").reshape(T, 2, 16))
+    h = h + plain.causal_attention(q, k, v, 2, 2, None).reshape(T, 32) @ w["l1.attn.o_proj.weight"].T
+    x = plain.rms_norm(h, w["l1.n2.weight"], 1e-5)
+    h = h + plain.swiglu_mlp(x, w["l1.mlp.gate_proj.weight"], w["l1.mlp.up_proj.weight"], w["l1.mlp.down_proj.weight"])
+    want = head_of(w, h)
+    got = torch.stack([whole[("a", p)] for p in range(T)]).double()
+    assert float((got - want).abs().max()) < tol * float(want.abs().max())
+
+
+def test_layer_order_is_data():
+    """one layer run twice (with a cache of its own each time) and a layer that reads another's cache"""
+    H, V, T = 32, 50, len(TOKS)
+    att = lambda: attention_spec(H, 2, 1, 16, bias=False)
+    layers = [layer(0, H, att(), PartSpec("test_no_ffn")), layer(1, H, att(), PartSpec("test_no_ffn"))]
+    w_of = lambda w, l, n: w[f"l{l}.attn.{n}_proj.weight"]
+
+    def attend(w, l, h, kv_from=None):
+        x = plain.rms_norm(h, w[f"l{l}.n1.weight"], 1e-5)
+        q = plain.rope_neox_rows((x @ w_of(w, l, "q").T).reshape(T, 2, 16), range(T), 1e4)
+        if kv_from is None:
+            k = plain.rope_neox_rows((x @ w_of(w, l, "k").T).reshape(T, 1, 16), range(T), 1e4)
+            v = (x @ w_of(w, l, "v").T).reshape(T, 1, 16)
+        else:
+            k, v = kv_from
+        return h + plain.causal_attention(q, k, v, 2, 1, None).reshape(T, 32) @ w_of(w, l, "o").T, (k, v)
+
+    # layer 0 twice, then layer 1
+    model, w = build(spec_of(H, V, layers, [ScheduleEntry(0), ScheduleEntry(0), ScheduleEntry(1)]), torch.float32)
+    whole, cut = run_whole_and_cut(model, TOKS)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    for l in (0, 0, 1):
+        h, _ = attend(w, l, h)
+    want = head_of(w, h)
+    assert float((whole - want).abs().max()) < 2e-5 * float(want.abs().max()) and torch.equal(whole, cut)
+    # layer 1 reads the keys and values that layer 0 wrote
+    model, w = build(spec_of(H, V, layers, [ScheduleEntry(0), ScheduleEntry(1, cache=0)]), torch.float32)
+    whole, cut = run_whole_and_cut(model, TOKS)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    h, kv = attend(w, 0, h)
+    h, _ = attend(w, 1, h, kv_from=kv)
+    want = head_of(w, h)
+    assert float((whole - want).abs().max()) < 2e-5 * float(want.abs().max()) and torch.equal(whole, cut)
+    with pytest.raises(ValueError):
+        Model(spec_of(H, V, layers, [ScheduleEntry(0, cache=1), ScheduleEntry(1)]))      # only an earlier entry's cache
+    with pytest.raises(KeyError):
+        Model(spec_of(H, V, [layer(0, H, PartSpec("no_such_mixer"), PartSpec("test_no_ffn"))]))
