@@ -77,9 +77,8 @@ def _writable_dir() -> str:
     for d in _lib_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".probe_{os.getpid()}")
-            with open(probe, "w"):
-                pass
+            fd, probe = tempfile.mkstemp(prefix=".probe_", dir=d)      # a name of its own for every caller
+            os.close(fd)
             os.remove(probe)
             return d
         except OSError:
@@ -96,7 +95,7 @@ def compile_library(name: str, verbose: bool = True) -> str:
         raise KernelBuildError(f"kernel library '{name}' is not built and hipcc was not found")
     out_dir = _writable_dir()
     so = os.path.join(out_dir, name + ".so")
-    tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.so")
+    tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
     cmd = [hipcc] + FLAGS + [os.path.join(HERE, name + ".hip"), "-o", tmp]
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)   # hipcc wants a home for its temporary files
