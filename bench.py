@@ -149,7 +149,9 @@ class Bench:
         dt = (time.perf_counter() - t0) / steps
         # one more, untimed, step that records which experts the router chose
         SparseMoE.record = []
+        graphs, self.runner.use_graphs = self.runner.use_graphs, False      # the hook needs the eager path
         one_step(cur)
+        self.runner.use_graphs = graphs
         torch.cuda.synchronize()
         per_layer = [len(set(t.flatten().tolist())) for t in SparseMoE.record]
         SparseMoE.record = None
@@ -171,6 +173,7 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode runs")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-graphs", action="store_true", help="launch every decode kernel from the host instead of replaying a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -180,6 +183,8 @@ def main() -> int:
     max_batch = max(args.batch, 1 if args.no_points else 64)
     b = Bench(args.layers, args.dtype, args.block_size, max_batch, args.ctx, max(new_tokens, 64))
     c = b.cfg
+    if args.no_graphs:
+        b.runner.use_graphs = False
 
     dt, distinct = b.decode(args.batch, args.ctx, args.steps, args.warmup)
     tok_s = args.batch / dt

@@ -28,8 +28,76 @@ class StepEntry:
     want: list = field(default_factory=list)     # places among `tokens` whose logits are asked for
 
 
+class DecodeGraph:
+    """One decode step (every sequence brings one token) recorded as a HIP graph.
+
+    What changes from step to step — tokens, positions, slots, block tables — lives in one
+    int32 device buffer at a fixed address that is refreshed before each replay; everything a
+    kernel launch depends on beside that (number of sequences, width of the block tables, the
+    bound on the sequence lengths that sets the number of attention splits) is fixed per graph.
+    """
+
+    def __init__(self, runner, n_seqs: int, kv_bound: int):
+        self.runner, self.n, self.kv_bound = runner, n_seqs, kv_bound
+        mgr = runner.manager
+        self.max_blocks = max(1, mgr.blocks_for(kv_bound))
+        self.keys = list(mgr.groups)
+        total = 3 * n_seqs + len(self.keys) * n_seqs * self.max_blocks
+        dev = runner.device
+        self.meta = torch.zeros(total, dtype=torch.int32, device=dev)
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        self.arange = torch.arange(n_seqs, dtype=torch.int32, device=dev)
+        self.graph = None
+        self.logits = None
+
+    def _context(self) -> StepContext:
+        n, mb = self.n, self.max_blocks
+        tables, o = {}, 3 * n
+        for key in self.keys:
+            tables[key] = self.meta[o:o + n * mb].view(n, mb)
+            o += n * mb
+        ctx = StepContext(n_tokens=n, n_seqs=n, act_dtype=self.runner.act_dtype, device=self.runner.device,
+                          token_ids=self.meta[0:n], positions=self.meta[n:2 * n], token_seq=self.arange,
+                          q_starts=list(range(n + 1)), kv_lens=[self.kv_bound] * n, slot_ids=self.meta[2 * n:3 * n],
+                          slots=None, block_tables=tables, block_size=self.runner.block_size, logit_rows=self.arange)
+        ctx._memo["attention_items"] = {"n_decode": n, "n_tiles": 0, "max_kv": self.kv_bound,
+                                        "dec_seq": self.arange, "dec_tok": self.arange}
+        return ctx
+
+    def run(self, tokens, positions, slots, table_rows) -> torch.Tensor:
+        n, mb = self.n, self.max_blocks
+        self.copied.synchronize()                  # the last upload has left the staging buffer
+        h = self.host
+        h[0:n] = torch.tensor(tokens, dtype=torch.int32)
+        h[n:2 * n] = torch.tensor(positions, dtype=torch.int32)
+        h[2 * n:3 * n] = torch.tensor(slots, dtype=torch.int32)
+        o = 3 * n
+        for rows in table_rows:                    # one list of rows per group, in the order of self.keys
+            flat = []
+            for r in rows:
+                flat.extend(max(p, 0) for p in r[:mb])
+                flat.extend([0] * (mb - min(len(r), mb)))
+            h[o:o + n * mb] = torch.tensor(flat, dtype=torch.int32)
+            o += n * mb
+        self.meta.copy_(h, non_blocking=True)
+        self.copied.record()
+        model, caches = self.runner.model, self.runner.storage.caches
+        if self.graph is None:
+            model.forward(self._context(), caches)              # once eagerly: loads the kernels
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = model.forward(self._context(), caches)
+            self.graph = graph
+        self.graph.replay()
+        return self.logits
+
+
 class ModelRunner:
-    def __init__(self, model, *, block_size: int = 64, num_pages: int = 64, max_seqs: int = 8):
+    def __init__(self, model, *, block_size: int = 64, num_pages: int = 64, max_seqs: int = 8,
+                 use_graphs: bool = True, graph_kv_step: int = 512):
         if model.device is None:
             raise RuntimeError("load the model's weights before making a runner")
         if model.device.type != "cuda":
@@ -41,6 +109,10 @@ class ModelRunner:
         self.manager = CacheManager(model.cache_groups(), num_pages, block_size, max_seqs)
         self.storage = CacheStorage(model, self.manager, self.act_dtype, self.device)
         self.vocab_size = model.spec.vocab_size
+        # decode steps are replayed from HIP graphs if every mixer can be recorded
+        self.use_graphs = use_graphs and all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
+        self.graph_kv_step = graph_kv_step
+        self._graphs: dict = {}
 
     # ---- requests ----------------------------------------------------------
     def admit(self, req) -> bool:
@@ -91,6 +163,19 @@ class ModelRunner:
         if len({e.req for e in entries}) != len(entries):
             raise ValueError("a request appears twice in one step")
         n_seqs, T = len(entries), len(tokens)
+        if self.use_graphs and T == n_seqs and len(rows) == n_seqs:
+            # every sequence brings one token and wants its logits: a recorded decode step
+            bound = -(-max(kv_lens) // self.graph_kv_step) * self.graph_kv_step
+            key = (n_seqs, bound)
+            if key not in self._graphs:
+                if len(self._graphs) >= 16:
+                    self._graphs.pop(next(iter(self._graphs)))
+                self._graphs[key] = DecodeGraph(self, n_seqs, bound)
+            logits = self._graphs[key].run(tokens, positions, slots,
+                                           [[mgr.table(e.req, k) for e in entries] for k in mgr.groups])
+            for e in entries:
+                mgr.trim(e.req)
+            return logits
         max_blocks = max(1, max(mgr.blocks_for(L) for L in kv_lens))
         tables = {}
         flat = tokens + positions + token_seq + slots + rows

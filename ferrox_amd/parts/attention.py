@@ -51,6 +51,7 @@ def attention_items(ctx):
 @MIXERS.register("paged_attention")
 class PagedAttention(Mixer):
     kernel_libraries = ("elementwise", "gemm", "attention")
+    graph_safe = True      # its launches depend on device data and on sizes that are fixed per graph
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, bias: bool,
                  position: PartSpec, window: int | None = None, scale: float | None = None):
