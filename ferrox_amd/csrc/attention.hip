@@ -210,22 +210,39 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
     }
 }
 
+// Merges the chunks' partial results in ascending order.  One block per (token, head): first
+// the weights exp(m_s - m) / sum of all chunks (kept in LDS), then every thread sums its head
+// dimensions over the chunks with several loads in flight.
 template <typename T>
-__global__ __launch_bounds__(64) void attn_decode_merge_kernel(AttnArgs a) {
-    const int item = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
+    extern __shared__ float wsm[];   // splits weights
+    __shared__ float red[2];
+    const int item = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int tok = a.item_tok[item];
-    const int hd = a.hd;
-    const float* po = a.part_o + ((size_t)item * a.nh + h) * a.splits * hd;
-    const float* pml = a.part_ml + ((size_t)item * a.nh + h) * a.splits * 2;
+    const int hd = a.hd, S = a.splits;
+    const float* po = a.part_o + ((size_t)item * a.nh + h) * S * hd;
+    const float* pml = a.part_ml + ((size_t)item * a.nh + h) * S * 2;
     float m = NEG_INF;
-    for (int s = 0; s < a.splits; ++s) m = fmaxf(m, pml[2 * s]);
+    for (int s = tid; s < S; s += 128) m = fmaxf(m, pml[2 * s]);
+    m = wave_max(m);
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(red[0], red[1]);
+    for (int s = tid; s < S; s += 128) {
+        const float ms = pml[2 * s];
+        wsm[s] = (ms == NEG_INF) ? 0.f : expf(ms - m);
+    }
+    __syncthreads();
     float l = 0.f;
-    for (int s = 0; s < a.splits; ++s)
-        if (pml[2 * s] != NEG_INF) l += pml[2 * s + 1] * expf(pml[2 * s] - m);
-    for (int d = lane; d < hd; d += 64) {
+    for (int s = 0; s < S; ++s) l += wsm[s] * ((wsm[s] > 0.f) ? pml[2 * s + 1] : 0.f);   // ascending, the same in every thread
+    for (int d = tid; d < hd; d += 128) {
         float acc = 0.f;
-        for (int s = 0; s < a.splits; ++s)
-            if (pml[2 * s] != NEG_INF) acc += po[(size_t)s * hd + d] * expf(pml[2 * s] - m);
+#pragma unroll 8
+        for (int s = 0; s < S; ++s) {
+            const float w = wsm[s];
+            const float v = (w > 0.f) ? po[(size_t)s * hd + d] : 0.f;   // an empty chunk wrote nothing
+            acc = fmaf(w, v, acc);
+        }
         from_float((T*)a.out + (size_t)tok * a.ldo + (size_t)h * hd + d, acc / l);
     }
 }
@@ -511,6 +528,7 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           float* part_o, float* part_ml, int splits, int chunk) {
     if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window)) return 1;
     FX_REQUIRE(splits > 0 && chunk > 0 && chunk % 64 == 0, "attn_decode: chunk %d must be a positive multiple of 64", chunk);
+    FX_REQUIRE(splits <= 8192, "attn_decode: %d chunks are more than the merge kernel takes (8192)", splits);
     if (n_items <= 0) return 0;
     AttnArgs a = {};
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
@@ -522,7 +540,7 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FX_F32) {
         attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
-        attn_decode_merge_kernel<float><<<grid2, 64, 0, s>>>(a);
+        attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
     } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
         const int group = nh / nkv;
         dim3 gridm(n_items, nkv * ((group + 15) / 16), splits);
@@ -530,10 +548,10 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
         else if (hd <= 64) attn_mfma_decode_kernel<64><<<gridm, 64, 0, s>>>(a);
         else if (hd <= 128) attn_mfma_decode_kernel<128><<<gridm, 64, 0, s>>>(a);
         else attn_mfma_decode_kernel<256><<<gridm, 64, 0, s>>>(a);
-        attn_decode_merge_kernel<bf16><<<grid2, 64, 0, s>>>(a);
+        attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);
     } else {
         attn_decode_kernel<bf16><<<grid, 64, 0, s>>>(a);
-        attn_decode_merge_kernel<bf16><<<grid2, 64, 0, s>>>(a);
+        attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);
     }
     FX_CHECK_LAUNCH("attn_decode");
     return 0;

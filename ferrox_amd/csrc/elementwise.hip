@@ -51,6 +51,26 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     __shared__ float red[4];
     const int r = blockIdx.x;
     const float* x = h + (size_t)(rows ? rows[r] : r) * H;
+    if (H <= 256 * 16) {   // the row stays in registers: one pass over memory, the weights fetched meanwhile
+        float xv[16], wv[16];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * 256;
+            xv[i] = c < H ? x[c] : 0.f;
+            wv[i] = c < H ? load_as_float(w, w_dtype, c) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ss += xv[i] * xv[i];
+        ss = block_sum<4>(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < H) from_float(out + (size_t)r * H + c, xv[i] * scale * wv[i]);
+        }
+        return;
+    }
     float ss = 0.f;
     for (int c = threadIdx.x; c < H; c += 256) {
         float v = x[c];
@@ -226,9 +246,9 @@ FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, 
 
 // ---------------------------------------------------------------------------
 // Weighted sum of the routed experts' outputs into the residual stream:
-//   h[t, :] += sum_j w[t, j] * y[inv[t*k + j], :]
+//   h[t, :] += sum_j w[t, j] * y[inv[t*k + j], :]      (inv null: y[t*k + j, :])
 // in ascending j, the selection order (ferrox-moe/src/lib.rs:735-745).
-// y is float32 [n_sorted, H].
+// y is float32 [T*k, H].
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
@@ -236,7 +256,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h,
     const int t = blockIdx.x;
     for (int c = threadIdx.x; c < H; c += 256) {
         float acc = 0.f;
-        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)inv[t * k + j] * H + c];
+        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
         h[(size_t)t * H + c] += acc;
     }
 }

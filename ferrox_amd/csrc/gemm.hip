@@ -31,6 +31,7 @@ struct GemmArgs {
     long ldc;
     const float* row_scale;  // [M] or null, multiplies the product before it is added (EPI_RESID)
     const int* a_rows;       // [M] or null: row of A to read for logical row m
+    const int* c_rows;       // [M] or null: row of C to write for logical row m
     const int* expert_offsets;  // [E+1] or null
     int E;
     int M, N, K;
@@ -192,8 +193,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int m = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
-            if (m >= r_end) continue;
+            const int ml = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
+            if (ml >= r_end) continue;
+            const int m = g.c_rows ? g.c_rows[ml] : ml;
             if (DUAL) {
 #pragma unroll
                 for (int j = 0; j < NT; j += 2) {
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                     } else if (EPI == EPI_STORE_F32) {
                         ((float*)g.C)[(size_t)m * g.ldc + n] = v;
                     } else {
-                        if (g.row_scale) v *= g.row_scale[m];
+                        if (g.row_scale) v *= g.row_scale[ml];
                         ((float*)g.C)[(size_t)m * g.ldc + n] += v;
                     }
                 }
@@ -262,30 +264,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     const int n_super = (g.K + 127) / 128;
     const int per = (n_super + WAVES - 1) / WAVES;
     const int s_end = min(n_super, (wave + 1) * per);
-    for (int s = wave * per; s < s_end; ++s) {
-        const int kb = s * 128 + grp * 32;
-        uint4 w[4], wu[4];
+    constexpr int UN = (MT <= 2) ? 2 : 1;     // pieces whose loads are issued together
+    for (int s = wave * per; s < s_end; s += UN) {
+        uint4 w[UN][4], wu[UN][4], x[UN][MT][4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            w[u] = load16(wrow, kb + 8 * u, g.K);
-            if (DUAL) wu[u] = load16(wrow ? wrow + g.up_offset : nullptr, kb + 8 * u, g.K);
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            uint4 x[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) x[u] = load16(xrow[mt], kb + 8 * u, g.K);
+        for (int p = 0; p < UN; ++p) {
+            const int kb = (s + p) * 128 + grp * 32;
+            const bool live = s + p < s_end;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[u]);
-                if (DUAL) {
-                    acc[2 * mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[u]), xb, acc[2 * mt], 0, 0, 0);
-                    acc[2 * mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wu[u]), xb, acc[2 * mt + 1], 0, 0, 0);
-                } else {
-                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[u]), xb, acc[mt], 0, 0, 0);
-                }
+                w[p][u] = load16(live ? wrow : nullptr, kb + 8 * u, g.K);
+                if (DUAL) wu[p][u] = load16(live && wrow ? wrow + g.up_offset : nullptr, kb + 8 * u, g.K);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 8 * u, g.K);
             }
         }
+#pragma unroll
+        for (int p = 0; p < UN; ++p)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[p][mt][u]);
+                    if (DUAL) {
+                        acc[2 * mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][u]), xb, acc[2 * mt], 0, 0, 0);
+                        acc[2 * mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wu[p][u]), xb, acc[2 * mt + 1], 0, 0, 0);
+                    } else {
+                        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][u]), xb, acc[mt], 0, 0, 0);
+                    }
+                }
     }
 #pragma unroll
     for (int a = 0; a < NACC; ++a) red[wave][a][lane] = acc[a];
@@ -302,8 +309,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
                 v += red[w][mt][L];
             }
         }
-        const int m = r0 + mt * 16 + (L & 15);
-        if (m >= r_end) continue;
+        const int ml = r0 + mt * 16 + (L & 15);
+        if (ml >= r_end) continue;
+        const int m = g.c_rows ? g.c_rows[ml] : ml;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n0 + (L >> 4) * 4 + r;
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             } else if (EPI == EPI_STORE_F32) {
                 ((float*)g.C)[(size_t)m * g.ldc + n] = o;
             } else {
-                if (g.row_scale) o *= g.row_scale[m];
+                if (g.row_scale) o *= g.row_scale[ml];
                 ((float*)g.C)[(size_t)m * g.ldc + n] += o;
             }
         }
@@ -393,8 +401,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int m = r0 + ty * 4 + i;
-        if (m >= r_end) continue;
+        const int ml = r0 + ty * 4 + i;
+        if (ml >= r_end) continue;
+        const int m = g.c_rows ? g.c_rows[ml] : ml;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
@@ -406,7 +415,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             } else {
                 if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
                 if (EPI == EPI_RESID) {
-                    if (g.row_scale) v *= g.row_scale[m];
+                    if (g.row_scale) v *= g.row_scale[ml];
                     *out += v;
                 } else {
                     *out = v;
@@ -459,8 +468,8 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int m_
 // rows_hint: in grouped mode, the expected number of rows per expert (chooses the tile).
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
-                   const float* row_scale, const int* a_rows, const int* expert_offsets, int E,
-                   int M, int N, int K) {
+                   const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
+                   int E, int M, int N, int K) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -472,7 +481,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     GemmArgs g;
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
-    g.a_rows = a_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
+    g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
     hipStream_t s = (hipStream_t)stream;
     const int nonempty = expert_offsets ? (E < M ? E : M) : 0;
     if (dtype == FX_F32) {

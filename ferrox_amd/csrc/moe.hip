@@ -105,6 +105,7 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, i
 // Stable counting sort of n = T*k (token, slot) pairs by expert, one block.
 //   expert_offsets[E+1] : rows of expert e are [off[e], off[e+1])
 //   sorted_token[i]     : token of sorted row i
+//   sorted_pair[i]      : pair t*k + j of sorted row i
 //   inv[t*k + j]        : sorted row of pair (t, j)
 // Thread th owns the contiguous pairs [th*c, (th+1)*c) and counts them per
 // expert in its own row cnt[th][.]; thread e then turns column e into running
@@ -114,7 +115,8 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, i
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E,
                                                         int* __restrict__ expert_offsets,
-                                                        int* __restrict__ sorted_token, int* __restrict__ inv) {
+                                                        int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
+                                                        int* __restrict__ inv) {
     extern __shared__ int lds[];
     int* offs = lds;                              // E + 1
     uint16_t* cnt = (uint16_t*)(lds + E + 1);     // [rows][E]
@@ -155,13 +157,14 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ 
             const int dst = offs[e] + cnt[th * E + e];
             cnt[th * E + e] += 1;
             sorted_token[dst] = i / k;
-            inv[i] = dst;
+            if (sorted_pair) sorted_pair[dst] = i;
+            if (inv) inv[i] = dst;
         }
     }
 }
 
 FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
-                        int* sorted_token, int* inv) {
+                        int* sorted_token, int* sorted_pair, int* inv) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
     FX_REQUIRE(E >= 1, "moe_align: E=%d", E);
     int nt = 256;
@@ -169,7 +172,7 @@ FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* 
     const size_t shm = (size_t)nt * E * 2 + (E + 1) * 4;
     FX_REQUIRE(shm <= 48 * 1024, "moe_align: %d experts exceed this kernel's limit of about 380", E);
     FX_REQUIRE((n + nt - 1) / nt < 65536, "moe_align: %d pairs are too many for one block", n);
-    moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, expert_offsets, sorted_token, inv);
+    moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, expert_offsets, sorted_token, sorted_pair, inv);
     FX_CHECK_LAUNCH("moe_align");
     return 0;
 }

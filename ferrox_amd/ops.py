@@ -54,7 +54,7 @@ _sigs = {
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
-                          c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
+                          c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -64,7 +64,7 @@ _sigs = {
                                       c_void_p, c_void_p, c_int, c_int],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p],
-    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
 _fns: dict = {}
@@ -166,7 +166,7 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
 
 
 def moe_combine(h, y_sorted, inv, weights, top_k) -> None:
-    """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]]."""
+    """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]]  (inv None: y is in pair order t*k + j)."""
     T, H = h.shape
     if y_sorted.dtype != torch.float32 or h.dtype != torch.float32:
         raise KernelError("moe_combine works on float32")
@@ -175,7 +175,8 @@ def moe_combine(h, y_sorted, inv, weights, top_k) -> None:
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: torch.Tensor | None = None,
          bias: torch.Tensor | None = None, row_scale: torch.Tensor | None = None,
-         a_rows: torch.Tensor | None = None, expert_offsets: torch.Tensor | None = None,
+         a_rows: torch.Tensor | None = None, c_rows: torch.Tensor | None = None,
+         expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
@@ -183,7 +184,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     EPI_STORE stores in a's dtype (+bias); EPI_STORE_F32 stores float32; EPI_RESID adds the
     product (times row_scale[m]) into the float32 `out`; EPI_SILU_MUL multiplies two
     matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores silu(gate)*up.
-    `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.
+    `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.  `c_rows`
+    scatters the rows of the output (row_scale stays indexed by the logical row).
     """
     if a.dtype != w.dtype:
         raise KernelError(f"gemm: activations are {a.dtype}, weights {w.dtype}")
@@ -224,7 +226,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
         raise KernelError(f"gemm: bias has {bias.numel()} elements for {N} columns")
     _call("gemm", "fx_gemm", _stream(), dtype_code(a.dtype), epilogue, _p(a), a.stride(0), _p(w), w_stride, up_offset,
           _p(bias), dtype_code(bias.dtype) if bias is not None else 0, _p(out), out.stride(0),
-          _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K)
+          _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
+          _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K)
     return out
 
 
@@ -278,15 +281,16 @@ def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gat
 
 
 def moe_align(ids: torch.Tensor, n_experts: int):
-    """Returns (expert_offsets [E+1], sorted_token [n], inv [n]) for ids [T, k]."""
+    """For ids [T, k]: (expert_offsets [E+1], sorted_token [n], sorted_pair [n], inv [n]): sorted row i
+    belongs to pair sorted_pair[i] = t*k + j of token sorted_token[i]; inv is the inverse map."""
     T, k = ids.shape
     n = T * k
     dev = ids.device
     offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
-    sorted_token = torch.empty((n,), dtype=torch.int32, device=dev)
-    inv = torch.empty((n,), dtype=torch.int32, device=dev)
-    _call("moe", "fx_moe_align", _stream(), _p(_i32(ids, "ids")), n, k, n_experts, _p(offsets), _p(sorted_token), _p(inv))
-    return offsets, sorted_token, inv
+    buf = torch.empty((3, n), dtype=torch.int32, device=dev)
+    _call("moe", "fx_moe_align", _stream(), _p(_i32(ids, "ids")), n, k, n_experts, _p(offsets), _p(buf[0]), _p(buf[1]),
+          _p(buf[2]))
+    return offsets, buf[0], buf[1], buf[2]
 
 
 def sample(logits: torch.Tensor, *, temperature=None, draw=None, top_k=None, top_p=None, rep_penalty=None,

@@ -72,10 +72,11 @@ class SparseMoE(FeedForward):
                                                self.has_shared_gate)
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
-        offsets, sorted_token, inv = ops.moe_align(ids, self.n_experts)
+        offsets, sorted_token, sorted_pair, _ = ops.moe_align(ids, self.n_experts)
         act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
                      expert_offsets=offsets, n_rows=T * self.top_k)
-        y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets)
-        ops.moe_combine(residual, y, inv, weights, self.top_k)
+        # each expert's rows go back to the place of their (token, slot) pair
+        y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+        ops.moe_combine(residual, y, None, weights, self.top_k)
         if self.shared is not None:
             self.shared.forward(x, ctx, residual, row_scale=gate)

@@ -63,7 +63,7 @@ def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     g = torch.Generator().manual_seed(5)
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
     wts = torch.rand(T, k, generator=g).to(DEV)
-    offsets, sorted_token, inv = ops.moe_align(ids, E)
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
     # the sort: offsets are the counts' prefix sums; every pair sits in its expert's range; order is stable
     counts = torch.bincount(ids.flatten().long().cpu(), minlength=E)
     assert offsets.cpu().tolist() == [0] + torch.cumsum(counts, 0).tolist()
@@ -71,7 +71,7 @@ def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     assert sorted(inv_c.tolist()) == list(range(T * k))
     for i in range(T * k):
         e = int(ids_c.flatten()[i])
-        assert offsets[e] <= inv_c[i] < offsets[e + 1] and st_c[inv_c[i]] == i // k
+        assert offsets[e] <= inv_c[i] < offsets[e + 1] and st_c[inv_c[i]] == i // k and sorted_pair[inv_c[i]] == i
     for e in range(E):
         seg = [i for i in range(T * k) if int(ids_c.flatten()[i]) == e]
         assert [int(inv_c[i]) for i in seg] == list(range(int(offsets[e]), int(offsets[e + 1])))
@@ -79,6 +79,11 @@ def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets)
     h = torch.zeros(T, H, device=DEV)
     ops.moe_combine(h, y, inv, wts, k)
+    # the same with the second product scattering its rows back into pair order
+    y2 = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+    h2 = torch.zeros(T, H, device=DEV)
+    ops.moe_combine(h2, y2, None, wts, k)
+    assert torch.equal(h, h2)
     ref = torch.zeros(T, H, dtype=torch.float64)
     xd, gud, dnd = x.double().cpu(), w_gu.double().cpu(), w_dn.double().cpu()
     for t in range(T):
