@@ -228,10 +228,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 // Few rows (decode): the weights are streamed once from memory straight into
 // MFMA operands, no LDS staging.  A block owns 16 output columns (16 rows of W)
 // and up to 16*MT logical rows; its WAVES waves split K between them in pieces
-// of 128 and their partial sums are added in wave order through LDS.  Lane
-// (i = lane%16, g = lane/16) reads 64 contiguous bytes of W row n0+i per piece,
-// so the four g-lanes of a row cover 256 contiguous bytes; the activations use
-// the same k -> lane assignment, which is all the MFMA needs to be right.
+// of 128 and their partial sums are added in wave order through LDS.  In each
+// of the four loads of a piece the lanes (i = lane%16, g = lane/16) of a row
+// read 64 contiguous bytes of W row n0+i; the activations use the same
+// k -> lane assignment, which is all the MFMA needs to be right.
 // W is the A operand: the accumulator of lane (m = lane%16, g) holds
 // C[m][n0 + 4g + r], r = 0..3.
 // ---------------------------------------------------------------------------
@@ -239,44 +239,53 @@ __device__ __forceinline__ uint4 load16(const bf16* row, int k, int K) {
     return (row && k < K) ? *(const uint4*)(row + k) : make_uint4(0, 0, 0, 0);
 }
 
-template <int MT, int WAVES, bool DUAL, int EPI>
+template <int MT, int WAVES, int NW, bool DUAL, int EPI>   // NW: sets of 16 weight rows per wave (dual: gate and up)
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
-    constexpr int NACC = MT * (DUAL ? 2 : 1);
+    static_assert(!DUAL || NW == 2, "dual mode multiplies two matrices");
+    constexpr int NACC = MT * NW;
+    constexpr int COLS = DUAL ? 16 : 16 * NW;   // output columns of a block
     __shared__ f32x4_t red[WAVES][NACC][64];
     int r0, r_end, expert;
     locate_rows<16 * MT>(g, blockIdx.y, r0, r_end, expert);
     if (r0 < 0) return;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * COLS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, grp = lane >> 4;
     const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
-    const bf16* wrow = (n0 + li < g.N) ? Wbase + (size_t)(n0 + li) * g.K : nullptr;
+    const bf16* wrow[NW];
+#pragma unroll
+    for (int a = 0; a < NW; ++a) {
+        const int n = DUAL ? n0 + li : n0 + a * 16 + li;
+        wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + ((DUAL && a) ? g.up_offset : 0) : nullptr;
+    }
     const bf16* xrow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = r0 + mt * 16 + li;
         xrow[mt] = (m < r_end) ? (const bf16*)g.A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : nullptr;
     }
-    f32x4_t acc[NACC];
+    f32x4_t acc[MT][NW];
 #pragma unroll
-    for (int a = 0; a < NACC; ++a) acc[a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int a = 0; a < NW; ++a) acc[mt][a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     const int n_super = (g.K + 127) / 128;
     const int per = (n_super + WAVES - 1) / WAVES;
     const int s_end = min(n_super, (wave + 1) * per);
-    constexpr int UN = (MT <= 2) ? 2 : 1;     // pieces whose loads are issued together
+    constexpr int UN = (MT * NW <= 4) ? 2 : 1;     // pieces whose loads are issued together
     for (int s = wave * per; s < s_end; s += UN) {
-        uint4 w[UN][4], wu[UN][4], x[UN][MT][4];
+        uint4 w[UN][NW][4], x[UN][MT][4];
 #pragma unroll
         for (int p = 0; p < UN; ++p) {
-            const int kb = (s + p) * 128 + grp * 32;
+            const int kb = (s + p) * 128 + grp * 8;     // load u of this lane: k = kb + 32u .. +7
             const bool live = s + p < s_end;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                w[p][u] = load16(live ? wrow : nullptr, kb + 8 * u, g.K);
-                if (DUAL) wu[p][u] = load16(live && wrow ? wrow + g.up_offset : nullptr, kb + 8 * u, g.K);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 8 * u, g.K);
+                for (int a = 0; a < NW; ++a) w[p][a][u] = load16(live ? wrow[a] : nullptr, kb + 32 * u, g.K);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 32 * u, g.K);
             }
         }
 #pragma unroll
@@ -286,35 +295,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[p][mt][u]);
-                    if (DUAL) {
-                        acc[2 * mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][u]), xb, acc[2 * mt], 0, 0, 0);
-                        acc[2 * mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wu[p][u]), xb, acc[2 * mt + 1], 0, 0, 0);
-                    } else {
-                        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][u]), xb, acc[mt], 0, 0, 0);
-                    }
+#pragma unroll
+                    for (int a = 0; a < NW; ++a)
+                        acc[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][a][u]), xb,
+                                                                            acc[mt][a], 0, 0, 0);
                 }
     }
 #pragma unroll
-    for (int a = 0; a < NACC; ++a) red[wave][a][lane] = acc[a];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int a = 0; a < NW; ++a) red[wave][mt * NW + a][lane] = acc[mt][a];
     __syncthreads();
-    for (int idx = tid; idx < MT * 64; idx += WAVES * 64) {
-        const int mt = idx >> 6, L = idx & 63;
+    constexpr int OUTS = DUAL ? MT : MT * NW;     // accumulator tiles that become output tiles
+    for (int idx = tid; idx < OUTS * 64; idx += WAVES * 64) {
+        const int t = idx >> 6, L = idx & 63;
+        const int mt = DUAL ? t : t / NW, a = DUAL ? 0 : t % NW;
         f32x4_t v = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v2 = v;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            if (DUAL) {
-                v += red[w][2 * mt][L];
-                v2 += red[w][2 * mt + 1][L];
-            } else {
-                v += red[w][mt][L];
-            }
+            v += red[w][mt * NW + a][L];
+            if (DUAL) v2 += red[w][mt * NW + 1][L];
         }
         const int ml = r0 + mt * 16 + (L & 15);
         if (ml >= r_end) continue;
         const int m = g.c_rows ? g.c_rows[ml] : ml;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int n = n0 + (L >> 4) * 4 + r;
+            const int n = n0 + a * 16 + (L >> 4) * 4 + r;
             if (n >= g.N) continue;
             float o = v[r];
             if (DUAL) {
@@ -440,28 +447,34 @@ static void launch_bf16(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) 
     }
 }
 
-template <int MT, int WAVES>
+template <int MT, int WAVES, int NW>
 static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
-    dim3 grid(ceil_div(g.N, 16), m_tiles);
-    switch (epi) {
-        case EPI_STORE: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_STORE><<<grid, WAVES * 64, 0, s>>>(g); break;
-        case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
-        case EPI_RESID: gemm_bf16_skinny_kernel<MT, WAVES, false, EPI_RESID><<<grid, WAVES * 64, 0, s>>>(g); break;
-        default:
-            if constexpr (MT * 2 * WAVES <= 32)
-                gemm_bf16_skinny_kernel<MT, WAVES, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
-            break;
+    dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 16 : 16 * NW), m_tiles);
+    if constexpr (MT * NW * WAVES <= 32) {       // the partial sums of all waves fit in LDS
+        switch (epi) {
+            case EPI_STORE: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE><<<grid, WAVES * 64, 0, s>>>(g); break;
+            case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
+            case EPI_RESID: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_RESID><<<grid, WAVES * 64, 0, s>>>(g); break;
+            default:
+                if constexpr (NW == 2) gemm_bf16_skinny_kernel<MT, WAVES, 2, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
+                break;
+        }
     }
 }
 
-static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int m_tiles, hipStream_t s) {
-    if (mt == 1) {
-        if (eight) launch_skinny_cfg<1, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<1, 4>(g, epi, m_tiles, s);
-    } else if (mt == 2) {
-        if (eight) launch_skinny_cfg<2, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<2, 4>(g, epi, m_tiles, s);
+// mt: row tiles per block (1, 2, 4); eight: 8 waves split K instead of 4; nw: 16-row weight sets per wave
+static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int nw, int m_tiles, hipStream_t s) {
+#define FX_SK(MT_, W_, NW_) launch_skinny_cfg<MT_, W_, NW_>(g, epi, m_tiles, s)
+    if (nw == 2) {
+        if (mt == 1) { if (eight) FX_SK(1, 8, 2); else FX_SK(1, 4, 2); }
+        else if (mt == 2) { if (eight) FX_SK(2, 8, 2); else FX_SK(2, 4, 2); }
+        else FX_SK(4, 4, 2);
     } else {
-        if (eight) launch_skinny_cfg<4, 8>(g, epi, m_tiles, s); else launch_skinny_cfg<4, 4>(g, epi, m_tiles, s);
+        if (mt == 1) { if (eight) FX_SK(1, 8, 1); else FX_SK(1, 4, 1); }
+        else if (mt == 2) { if (eight) FX_SK(2, 8, 1); else FX_SK(2, 4, 1); }
+        else { if (eight) FX_SK(4, 8, 1); else FX_SK(4, 4, 1); }
     }
+#undef FX_SK
 }
 
 // dtype: type of A and W.  C is: T for EPI_STORE and EPI_SILU_MUL, float32 otherwise.
@@ -503,10 +516,13 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     if (g.vec_ok && per_group <= 64) {
         const int mt = per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4);
         const int m_tiles = M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
-        const long blocks = (long)ceil_div(N, 16) * m_tiles;
         const bool dual = epi == EPI_SILU_MUL;
-        const bool eight = blocks < 1024 && mt * (dual ? 2 : 1) <= 4 && K >= 2048;
-        launch_skinny(g, epi, mt, eight, m_tiles, s);
+        // two sets of weight rows per wave share the activations they multiply: worth it when
+        // there are blocks enough either way
+        const int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 2048) ? 2 : 1;
+        const long blocks = (long)ceil_div(N, dual ? 16 : 16 * nw) * m_tiles;
+        const bool eight = blocks < 1024 && mt * nw <= 4 && K >= 2048;
+        launch_skinny(g, epi, mt, eight, nw, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }
