@@ -108,62 +108,49 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // [page][kv_head][head_dim][slot], which is what the attention kernels read.
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+__global__ __launch_bounds__(128) void rope_kv_write_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
-    const int t = blockIdx.x;
+    // one block per (token, head): query heads first, then the kv heads
+    const int t = blockIdx.x, head = blockIdx.y;
     const int pos = positions[t];
     const int half = rot >> 1;
-    T* k_dst = nullptr;
-    T* v_dst = nullptr;
-    int slot = 0;
-    if (k_pages) {
-        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
-        slot = pos % bs;
-        k_dst = k_pages + (size_t)page * nkv * bs * hd;
-        v_dst = v_pages + (size_t)page * nkv * hd * bs;
-    }
-    // one (cos, sin) per rotated pair of this token, shared by all heads
-    __shared__ float cs_s[512], sn_s[512];
-    for (int p = threadIdx.x; p < half; p += 256) {
-        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
-        sincosf((float)pos * freq, &sn_s[p], &cs_s[p]);
-    }
-    __syncthreads();
-    // rotated pairs of q (in place) and k (into the page)
-    const int n_pairs = (nh + nkv) * half;
-    for (int i = threadIdx.x; i < n_pairs; i += 256) {
-        const int head = i / half, p = i % half;
-        const float cs = cs_s[p], sn = sn_s[p];
-        const int ia = interleaved ? 2 * p : p;
-        const int ib = interleaved ? 2 * p + 1 : p + half;
-        if (head < nh) {
-            T* row = q + (size_t)t * ldq + (size_t)head * hd;
+    if (head < nh) {
+        T* row = q + (size_t)t * ldq + (size_t)head * hd;
+        for (int p = threadIdx.x; p < half; p += 128) {
+            const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
+            float sn, cs;
+            sincosf((float)pos * freq, &sn, &cs);
+            const int ia = interleaved ? 2 * p : p;
+            const int ib = interleaved ? 2 * p + 1 : p + half;
             const float a = to_float(row[ia]), b = to_float(row[ib]);
             from_float(row + ia, a * cs - b * sn);
             from_float(row + ib, a * sn + b * cs);
-        } else if (k_dst) {
-            const int kh = head - nh;
-            const T* row = k + (size_t)t * ldk + (size_t)kh * hd;
-            const float a = to_float(row[ia]), b = to_float(row[ib]);
-            T* dst = k_dst + ((size_t)kh * bs + slot) * hd;
-            from_float(dst + ia, a * cs - b * sn);
-            from_float(dst + ib, a * sn + b * cs);
         }
+        return;
     }
-    if (!k_dst) return;
-    // the part of k beyond the rotated dimensions, and v
-    const int tail = hd - rot;
-    for (int i = threadIdx.x; i < nkv * tail; i += 256) {
-        const int kh = i / tail, d = rot + i % tail;
-        k_dst[((size_t)kh * bs + slot) * hd + d] = k[(size_t)t * ldk + (size_t)kh * hd + d];
+    if (!k_pages) return;
+    const int kh = head - nh;
+    const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+    const int slot = pos % bs;
+    T* k_dst = k_pages + (((size_t)page * nkv + kh) * bs + slot) * hd;
+    T* v_dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + slot;
+    const T* krow = k + (size_t)t * ldk + (size_t)kh * hd;
+    const T* vrow = v + (size_t)t * ldv + (size_t)kh * hd;
+    for (int p = threadIdx.x; p < half; p += 128) {
+        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
+        float sn, cs;
+        sincosf((float)pos * freq, &sn, &cs);
+        const int ia = interleaved ? 2 * p : p;
+        const int ib = interleaved ? 2 * p + 1 : p + half;
+        const float a = to_float(krow[ia]), b = to_float(krow[ib]);
+        from_float(k_dst + ia, a * cs - b * sn);
+        from_float(k_dst + ib, a * sn + b * cs);
     }
-    for (int i = threadIdx.x; i < nkv * hd; i += 256) {
-        const int kh = i / hd, d = i % hd;
-        v_dst[((size_t)kh * hd + d) * bs + slot] = v[(size_t)t * ldv + i];
-    }
+    for (int d = rot + threadIdx.x; d < hd; d += 128) k_dst[d] = krow[d];     // beyond the rotated dimensions
+    for (int d = threadIdx.x; d < hd; d += 128) v_dst[(size_t)d * bs] = vrow[d];
 }
 
 FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const void* k, int ldk,
@@ -171,17 +158,18 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
                             const int* block_table, int max_blocks, void* k_pages, void* v_pages,
                             int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
     FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
-    FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0 && rot <= 1024, "rope_kv_write: rotary dim %d must be even, <= head_dim %d and <= 1024", rot, hd);
+    FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
+    FX_REQUIRE(nh + nkv <= 65535, "rope_kv_write: too many heads");
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FX_F32)
-        rope_kv_write_kernel<float><<<T, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
+        rope_kv_write_kernel<float><<<dim3(T, nh + nkv), 128, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
                                                       positions, token_seq, block_table, max_blocks,
                                                       (float*)k_pages, (float*)v_pages, nh, nkv, hd, bs, rot,
                                                       interleaved, theta);
     else if (dtype == FX_BF16)
-        rope_kv_write_kernel<bf16><<<T, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
+        rope_kv_write_kernel<bf16><<<dim3(T, nh + nkv), 128, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
                                                      positions, token_seq, block_table, max_blocks,
                                                      (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, bs, rot,
                                                      interleaved, theta);
@@ -254,18 +242,18 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
                                                           int H, int k) {
     const int t = blockIdx.x;
-    for (int c = threadIdx.x; c < H; c += 256) {
-        float acc = 0.f;
-        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
-        h[(size_t)t * H + c] += acc;
-    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= H) return;
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
+    h[(size_t)t * H + c] += acc;
 }
 
 FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv, const float* w,
                           int T, int H, int k) {
     FX_REQUIRE(T >= 0 && H > 0 && k > 0, "moe_combine: bad sizes");
     if (T == 0) return 0;
-    moe_combine_kernel<<<T, 256, 0, (hipStream_t)stream>>>(h, y, inv, w, H, k);
+    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, H, k);
     FX_CHECK_LAUNCH("moe_combine");
     return 0;
 }

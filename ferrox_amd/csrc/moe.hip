@@ -27,15 +27,11 @@ enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
 //   GATE_SIGMOID scores each expert with 1/(1+exp(-logit)) instead
 //   (ferrox-moe/src/lib.rs:100-121).
 //   gate_out[t] = sigmoid(logits[t, E])  (decoder.rs:2670-2672).
-__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, int T, int E,
-                                                            int k, int renorm, int gating, int* __restrict__ ids,
-                                                            float* __restrict__ weights, float* __restrict__ gate_out) {
-    __shared__ float score_all[4][E_MAX];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * 4 + wave;
-    if (t >= T) return;
-    float* score = score_all[wave];
-    const float* row = logits + (size_t)t * ld;
+// selection for one token by one wave; `score` is E floats of LDS owned by the wave
+__device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm,
+                                             int gating, int* __restrict__ ids, float* __restrict__ weights,
+                                             float* __restrict__ gate_out, int* ids_copy) {
+    const int lane = threadIdx.x & 63;
     if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E]));
     if (gating == GATE_SOFTMAX) {
         float mx = NEG_INFINITY_F;
@@ -78,6 +74,7 @@ __global__ __launch_bounds__(256) void router_select_kernel(const float* __restr
         if (lane == j) my_w = best;
         if (lane == 0) {
             ids[t * k + j] = bi;
+            if (ids_copy) ids_copy[t * k + j] = bi;
             score[bi] = -2.f;  // scores are >= 0; taken out of the race
         }
         wsum += best;
@@ -85,6 +82,16 @@ __global__ __launch_bounds__(256) void router_select_kernel(const float* __restr
         __threadfence_block();
     }
     if (lane < k) weights[t * k + lane] = renorm ? my_w / wsum : my_w;
+}
+
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, int T, int E,
+                                                            int k, int renorm, int gating, int* __restrict__ ids,
+                                                            float* __restrict__ weights, float* __restrict__ gate_out) {
+    extern __shared__ float score_all[];   // 4 x E
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;
+    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr);
 }
 
 FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, int E, int k, int renorm,
@@ -95,8 +102,8 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, i
     FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     if (T == 0) return 0;
-    router_select_kernel<<<(T + 3) / 4, 256, 0, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
-                                                                     gate_out);
+    router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating,
+                                                                                         ids, weights, gate_out);
     FX_CHECK_LAUNCH("router_select");
     return 0;
 }
@@ -113,14 +120,11 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, i
 // walks its pairs again and places them.  The order inside an expert is the
 // order of the pairs, whatever the number of threads.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E,
-                                                        int* __restrict__ expert_offsets,
-                                                        int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
-                                                        int* __restrict__ inv) {
-    extern __shared__ int lds[];
-    int* offs = lds;                              // E + 1
-    uint16_t* cnt = (uint16_t*)(lds + E + 1);     // [rows][E]
-    const int nt = blockDim.x, th = threadIdx.x;
+// the sort itself, by one block; `offs` (E+1 ints) and `cnt` (rows*E uint16) are LDS
+__device__ __forceinline__ void align_block(const int* ids, int n, int k, int E, int* offs, uint16_t* cnt,
+                                            int* __restrict__ expert_offsets, int* __restrict__ sorted_token,
+                                            int* __restrict__ sorted_pair, int* __restrict__ inv) {
+    const int nt = blockDim.x, th = threadIdx.x, lane = th & 63;
     const int c = max(1, (n + nt - 1) / nt);
     const int rows = min(nt, (n + c - 1) / c);    // threads that own at least one pair
     const int b = min(n, th * c), b_end = min(n, (th + 1) * c);
@@ -141,12 +145,19 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ 
         offs[e + 1] = run;  // total of expert e, scanned below
     }
     __syncthreads();
-    if (th == 0) {
-        int run = 0;
-        offs[0] = 0;
-        for (int e = 0; e < E; ++e) {
-            run += offs[e + 1];
-            offs[e + 1] = run;
+    if (th < 64) {   // inclusive scan of the totals by the first wave, 64 experts at a time
+        int carry = 0;
+        if (lane == 0) offs[0] = 0;
+        for (int base = 0; base < E; base += 64) {
+            const int e = base + lane;
+            int v = e < E ? offs[e + 1] : 0;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int u = __shfl_up(v, o, 64);
+                if (lane >= o) v += u;
+            }
+            if (e < E) offs[e + 1] = carry + v;
+            carry += __shfl(v, 63, 64);
         }
     }
     __syncthreads();
@@ -163,6 +174,33 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ 
     }
 }
 
+__global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E,
+                                                        int* __restrict__ expert_offsets,
+                                                        int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
+                                                        int* __restrict__ inv) {
+    extern __shared__ int lds[];
+    align_block(ids, n, k, E, lds, (uint16_t*)(lds + E + 1), expert_offsets, sorted_token, sorted_pair, inv);
+}
+
+// few tokens: selection (a wave per token, in turns) and the sort in one block
+__global__ __launch_bounds__(256) void router_select_align_kernel(const float* __restrict__ logits, long ld, int T, int E,
+                                                                  int k, int renorm, int gating, int* __restrict__ ids,
+                                                                  float* __restrict__ weights, float* __restrict__ gate_out,
+                                                                  int* __restrict__ expert_offsets,
+                                                                  int* __restrict__ sorted_token,
+                                                                  int* __restrict__ sorted_pair, int* __restrict__ inv) {
+    extern __shared__ int lds[];
+    float* score = (float*)lds;                 // 4 x E
+    int* ids_s = lds + 4 * E;                   // T * k
+    int* offs = ids_s + T * k;                  // E + 1
+    uint16_t* cnt = (uint16_t*)(offs + E + 1);  // rows x E
+    const int wave = threadIdx.x >> 6;
+    for (int t = wave; t < T; t += 4)
+        select_token(logits + (size_t)t * ld, score + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, ids_s);
+    __syncthreads();
+    align_block(ids_s, T * k, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
+}
+
 FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
                         int* sorted_token, int* sorted_pair, int* inv) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
@@ -174,5 +212,26 @@ FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* 
     FX_REQUIRE((n + nt - 1) / nt < 65536, "moe_align: %d pairs are too many for one block", n);
     moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, expert_offsets, sorted_token, sorted_pair, inv);
     FX_CHECK_LAUNCH("moe_align");
+    return 0;
+}
+
+// Both steps in one launch when the batch is small enough for one block; returns 2 (and
+// launches nothing) when it is not, so that the caller runs the two kernels.
+FX_API int fx_router_select_align(void* stream, const float* logits, long ld, int T, int E, int k, int renorm,
+                                  int gating, int* ids, float* weights, float* gate_out, int* expert_offsets,
+                                  int* sorted_token, int* sorted_pair, int* inv) {
+    FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
+    FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
+    FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
+    FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
+    FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
+    const long n = (long)T * k;
+    const long rows = n < 256 ? n : 256;
+    const size_t shm = (size_t)(4 * E + n + E + 1) * 4 + (size_t)rows * E * 2;
+    if (T > 64 || n > 2048 || shm > 48 * 1024) return 2;
+    if (T == 0) return 0;
+    router_select_align_kernel<<<1, 256, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
+                                                                     gate_out, expert_offsets, sorted_token, sorted_pair, inv);
+    FX_CHECK_LAUNCH("router_select_align");
     return 0;
 }

@@ -64,6 +64,8 @@ _sigs = {
                                       c_void_p, c_void_p, c_int, c_int],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
@@ -278,6 +280,31 @@ def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gat
     _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), T, n_experts, top_k,
           1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
     return ids, weights, gate
+
+
+def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+    """router_select followed by moe_align; one launch when the batch is small.
+    Returns (ids, weights, gate, expert_offsets, sorted_token, sorted_pair, inv)."""
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("route: logits must be float32 [T, E] with unit inner stride")
+    T = logits.shape[0]
+    dev = logits.device
+    if T <= 64 and logits.shape[1] >= n_experts + (1 if has_gate else 0):
+        n = T * top_k
+        ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+        weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
+        gate = torch.empty((T,), dtype=torch.float32, device=dev) if has_gate else None
+        offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
+        buf = torch.empty((3, n), dtype=torch.int32, device=dev)
+        f, handle = _fn("moe", "fx_router_select_align")
+        rc = f(_stream(), _p(logits), logits.stride(0), T, n_experts, top_k, 1 if renorm else 0, gating, _p(ids),
+               _p(weights), _p(gate), _p(offsets), _p(buf[0]), _p(buf[1]), _p(buf[2]))
+        if rc == 0:
+            return ids, weights, gate, offsets, buf[0], buf[1], buf[2]
+        if rc != 2:
+            raise KernelError(handle.fx_last_error().decode())
+    ids, weights, gate = router_select(logits, n_experts, top_k, renorm, gating, has_gate)
+    return (ids, weights, gate) + moe_align(ids, n_experts)
 
 
 def moe_align(ids: torch.Tensor, n_experts: int):

@@ -68,11 +68,10 @@ class SparseMoE(FeedForward):
     def forward(self, x, ctx, residual) -> None:
         T = x.shape[0]
         logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
-        ids, weights, gate = ops.router_select(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
-                                               self.has_shared_gate)
+        ids, weights, gate, offsets, sorted_token, sorted_pair, _ = ops.route(
+            logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating, self.has_shared_gate)
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
-        offsets, sorted_token, sorted_pair, _ = ops.moe_align(ids, self.n_experts)
         act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
                      expert_offsets=offsets, n_rows=T * self.top_k)
         # each expert's rows go back to the place of their (token, slot) pair

@@ -256,3 +256,15 @@ def test_sampling_kernel():
                              hist=torch.tensor(hist, dtype=torch.int32, device=DEV),
                              hist_start=torch.tensor([0, len(hist)], dtype=torch.int32, device=DEV)).tolist()[0]
             assert got == want, f"{case} trial {trial}: kernel {got}, plain {want}"
+
+
+@pytest.mark.parametrize("T,E,k", [(1, 8, 2), (8, 60, 4), (64, 60, 4), (33, 130, 8), (65, 6, 3), (300, 60, 4)])
+def test_route_in_one_launch_equals_two(T, E, k):
+    """selection and sort fused for small batches give what the two kernels give"""
+    from ferrox_amd import ops
+    logits = rnd(T, E + 1, scale=2.0)
+    fused = ops.route(logits, E, k, True, has_gate=True)
+    ids, w, gate = ops.router_select(logits, E, k, True, has_gate=True)
+    two = (ids, w, gate) + ops.moe_align(ids, E)
+    for a, b in zip(fused, two):
+        assert torch.equal(a, b)
