@@ -235,25 +235,28 @@ FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, 
 // ---------------------------------------------------------------------------
 // Weighted sum of the routed experts' outputs into the residual stream:
 //   h[t, :] += sum_j w[t, j] * y[inv[t*k + j], :]      (inv null: y[t*k + j, :])
+//              + gate[t] * shared[t, :]                  (if a shared expert's output is given)
 // in ascending j, the selection order (ferrox-moe/src/lib.rs:735-745).
 // y is float32 [T*k, H].
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
+                                                          const float* __restrict__ shared, const float* __restrict__ gate,
                                                           int H, int k) {
     const int t = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= H) return;
     float acc = 0.f;
     for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
+    if (shared) acc += (gate ? gate[t] : 1.f) * shared[(size_t)t * H + c];     // routed first, then shared (lib.rs:746-750)
     h[(size_t)t * H + c] += acc;
 }
 
 FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv, const float* w,
-                          int T, int H, int k) {
+                          const float* shared, const float* gate, int T, int H, int k) {
     FX_REQUIRE(T >= 0 && H > 0 && k > 0, "moe_combine: bad sizes");
     if (T == 0) return 0;
-    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, H, k);
+    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, shared, gate, H, k);
     FX_CHECK_LAUNCH("moe_combine");
     return 0;
 }

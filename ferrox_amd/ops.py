@@ -51,7 +51,8 @@ _sigs = {
                                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
-    ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
+    ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_int, c_int],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
@@ -167,12 +168,16 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
     _call("elementwise", "fx_fill_u32", _stream(), _p(t), value, t.element_size() * t.numel() // 4)
 
 
-def moe_combine(h, y_sorted, inv, weights, top_k) -> None:
-    """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]]  (inv None: y is in pair order t*k + j)."""
+def moe_combine(h, y_sorted, inv, weights, top_k, shared=None, gate=None) -> None:
+    """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]] (inv None: y is in pair order t*k + j)
+    + gate[t] * shared[t] if the float32 output of a shared expert is given."""
     T, H = h.shape
     if y_sorted.dtype != torch.float32 or h.dtype != torch.float32:
         raise KernelError("moe_combine works on float32")
-    _call("elementwise", "fx_moe_combine", _stream(), _p(h), _p(y_sorted), _p(_i32(inv, "inv")), _p(weights), T, H, top_k)
+    if shared is not None and (shared.dtype != torch.float32 or shared.shape != h.shape or not shared.is_contiguous()):
+        raise KernelError("moe_combine: the shared expert's output must be float32 of h's shape")
+    _call("elementwise", "fx_moe_combine", _stream(), _p(h), _p(y_sorted), _p(_i32(inv, "inv")), _p(weights),
+          _p(shared), _p(gate), T, H, top_k)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: torch.Tensor | None = None,

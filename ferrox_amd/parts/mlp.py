@@ -26,6 +26,10 @@ class SwiGLU(FeedForward):
         self.gate_up = Linear(torch.cat(same_dtype([fetch("gate_proj.weight"), fetch("up_proj.weight")]), dim=0))
         self.down = Linear(fetch("down_proj.weight"))
 
+    def output(self, x):
+        """The feed-forward's output as float32 [T, H], added to nothing."""
+        return self.down(self.gate_up(x, epilogue=ops.EPI_SILU_MUL), epilogue=ops.EPI_STORE_F32)
+
     def forward(self, x, ctx, residual, row_scale=None) -> None:
         act = self.gate_up(x, epilogue=ops.EPI_SILU_MUL)
         self.down(act, epilogue=ops.EPI_RESID, out=residual, row_scale=row_scale)

@@ -17,6 +17,16 @@ from .linear import matmul, same_dtype
 from .mlp import SwiGLU
 
 GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
+OVERLAP_MAX_TOKENS = 256     # up to here the shared expert runs beside the routed ones on a second stream
+_side_streams: dict = {}
+
+
+def side_stream(device) -> torch.cuda.Stream:
+    """One extra stream per device, of the default priority."""
+    key = torch.device(device)
+    if key not in _side_streams:
+        _side_streams[key] = torch.cuda.Stream(device=key)
+    return _side_streams[key]
 
 
 @FEED_FORWARDS.register("sparse_moe")
@@ -67,6 +77,17 @@ class SparseMoE(FeedForward):
 
     def forward(self, x, ctx, residual) -> None:
         T = x.shape[0]
+        overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
+        if overlap:
+            # few tokens: both halves are bound by reading weights, so the shared expert streams its
+            # weights on a second stream while the routed experts run; its output joins in the combine
+            main, side = torch.cuda.current_stream(), side_stream(x.device)
+            fork, join = torch.cuda.Event(), torch.cuda.Event()
+            fork.record(main)
+            side.wait_event(fork)
+            with torch.cuda.stream(side):
+                shared_out = self.shared.output(x)
+                join.record(side)
         logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = ops.route(
             logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating, self.has_shared_gate)
@@ -76,6 +97,11 @@ class SparseMoE(FeedForward):
                      expert_offsets=offsets, n_rows=T * self.top_k)
         # each expert's rows go back to the place of their (token, slot) pair
         y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
-        ops.moe_combine(residual, y, None, weights, self.top_k)
-        if self.shared is not None:
-            self.shared.forward(x, ctx, residual, row_scale=gate)
+        if overlap:
+            main.wait_event(join)
+            shared_out.record_stream(main)
+            ops.moe_combine(residual, y, None, weights, self.top_k, shared=shared_out, gate=gate)
+        else:
+            ops.moe_combine(residual, y, None, weights, self.top_k)
+            if self.shared is not None:
+                self.shared.forward(x, ctx, residual, row_scale=gate)
