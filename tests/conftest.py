@@ -42,7 +42,28 @@ TINY_C = {
     "rms_norm_eps": 3e-6, "max_position_embeddings": 512, "use_sliding_window": True, "sliding_window": 40,
     "max_window_layers": 0, "tie_word_embeddings": False,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# layer sizes of the models the engine is built for (one layer, small vocabulary), so that the
+# kernels take the code paths they take in production: head_dim 128, K = 2048 and more, 60 experts
+WIDE_D = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 1, "hidden_size": 2048, "num_attention_heads": 16, "num_key_value_heads": 16,
+    "num_experts": 60, "num_experts_per_tok": 4, "norm_topk_prob": False, "moe_intermediate_size": 1408,
+    "shared_expert_intermediate_size": 5632, "intermediate_size": 5632, "decoder_sparse_step": 1,
+    "mlp_only_layers": [], "vocab_size": 1000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 8192, "use_sliding_window": False, "sliding_window": 4096,
+    "max_window_layers": 1, "tie_word_embeddings": False,
+}
+# few experts with many rows each, grouped-query attention with 7 query heads per kv head, a window
+WIDE_E = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 2, "hidden_size": 1792, "num_attention_heads": 14, "num_key_value_heads": 2,
+    "num_experts": 4, "num_experts_per_tok": 2, "norm_topk_prob": True, "moe_intermediate_size": 640,
+    "shared_expert_intermediate_size": 1280, "intermediate_size": 2368, "decoder_sparse_step": 1,
+    "mlp_only_layers": [1], "vocab_size": 777, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 8192, "use_sliding_window": True, "sliding_window": 100,
+    "max_window_layers": 1, "tie_word_embeddings": True,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4)}
 
 
 @pytest.fixture(scope="session")

@@ -139,7 +139,8 @@ def combine_expert_outputs(routed, shared, hidden_dim: int, dtype=torch.float64)
     return out
 
 
-def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w, margins=None):
+def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w, margins=None, forced_ids=None,
+                  chosen=None):
     """One token through the sparse block.
 
     Router logits r = router . x with no bias (ferrox-models/src/decoder.rs:2915),
@@ -147,9 +148,19 @@ def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w
     shared expert scaled by sigmoid(shared_gate . x)
     (ferrox-models/src/decoder.rs:2660-2679).
     `experts` is a list of (gate, up, down); `shared` one such triple or None.
+    `forced_ids` replaces the router's choice of experts (their weights are still the router's
+    probabilities); `chosen`, a list, receives the ids used.
     """
     logits = router_w @ x
     ids, w = route_top_k(logits, k, norm_topk_prob)
+    if forced_ids is not None and list(forced_ids) != ids:
+        ids = [int(e) for e in forced_ids]
+        e_ = torch.exp(logits - logits.max())
+        w = torch.stack([(e_ / e_.sum())[i] for i in ids])
+        if norm_topk_prob:
+            w = w / w.sum()
+    if chosen is not None:
+        chosen.append(list(ids))
     if margins is not None:
         margins.append(router_margin(logits, k))
     routed = [(swiglu_mlp(x, *experts[e]), w[j]) for j, e in enumerate(ids)]
@@ -199,15 +210,20 @@ def load_folder(folder: str, dtype=torch.float64):
     return cfg, weights
 
 
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0, margins=None) -> torch.Tensor:
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0, margins=None, routing=None,
+            chosen=None) -> torch.Tensor:
     """Logits[T, V] of one whole sequence (ferrox-models/src/decoder.rs:3014-3678
     followed by the head on every row, decoder.rs:2952-2973).
 
     `start_pos` shifts every position (used by the shift-invariance test only).
     `margins`, a list of T floats if given, receives for every position the smallest
-    `router_margin` over the sparse layers.
+    `router_margin` over the sparse layers.  `routing[t][j]` forces the experts of position t in the
+    j-th sparse layer; `chosen`, a list, receives the experts used in the same shape.
     """
     T = len(tokens)
+    n_sparse = 0
+    if chosen is not None:
+        chosen[:] = [[] for _ in range(T)]
     if margins is not None:
         margins[:] = [1.0] * T
     nh = cfg["num_attention_heads"]
@@ -247,11 +263,17 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
                           w[p + "mlp.shared_expert.down_proj.weight"])
                 gate_w = w[p + "mlp.shared_expert_gate.weight"]
             layer_margins = [] if margins is not None else None
+            layer_chosen = []
             f = torch.stack([
                 moe_ffn_token(x2[t], w[p + "mlp.gate.weight"], experts,
                               cfg["num_experts_per_tok"], cfg.get("norm_topk_prob", False),
-                              shared, gate_w, layer_margins)
+                              shared, gate_w, layer_margins,
+                              routing[t][n_sparse] if routing is not None else None, layer_chosen)
                 for t in range(T)])
+            if chosen is not None:
+                for t in range(T):
+                    chosen[t].append(layer_chosen[t])
+            n_sparse += 1
             if margins is not None:
                 for t in range(T):
                     margins[t] = min(margins[t], layer_margins[t])
