@@ -182,21 +182,21 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ 
     align_block(ids, n, k, E, lds, (uint16_t*)(lds + E + 1), expert_offsets, sorted_token, sorted_pair, inv);
 }
 
-// few tokens: selection (a wave per token, in turns) and the sort in one block
-__global__ __launch_bounds__(256) void router_select_align_kernel(const float* __restrict__ logits, long ld, int T, int E,
+// few tokens: selection (a wave per token) and the sort in one block of 16 waves
+__global__ __launch_bounds__(1024) void router_select_align_kernel(const float* __restrict__ logits, long ld, int T, int E,
                                                                   int k, int renorm, int gating, int* __restrict__ ids,
                                                                   float* __restrict__ weights, float* __restrict__ gate_out,
                                                                   int* __restrict__ expert_offsets,
                                                                   int* __restrict__ sorted_token,
                                                                   int* __restrict__ sorted_pair, int* __restrict__ inv) {
     extern __shared__ int lds[];
-    float* score = (float*)lds;                 // 4 x E
-    int* ids_s = lds + 4 * E;                   // T * k
+    float* score = (float*)lds;                 // 16 x E
+    int* ids_s = lds + 16 * E;                  // T * k
     int* offs = ids_s + T * k;                  // E + 1
     uint16_t* cnt = (uint16_t*)(offs + E + 1);  // rows x E
     const int wave = threadIdx.x >> 6;
-    for (int t = wave; t < T; t += 4)
-        select_token(logits + (size_t)t * ld, score + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, ids_s);
+    if (wave < T)
+        select_token(logits + (size_t)wave * ld, score + wave * E, wave, E, k, renorm, gating, ids, weights, gate_out, ids_s);
     __syncthreads();
     align_block(ids_s, T * k, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
 }
@@ -226,11 +226,11 @@ FX_API int fx_router_select_align(void* stream, const float* logits, long ld, in
     FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     const long n = (long)T * k;
-    const long rows = n < 256 ? n : 256;
-    const size_t shm = (size_t)(4 * E + n + E + 1) * 4 + (size_t)rows * E * 2;
-    if (T > 64 || n > 2048 || shm > 48 * 1024) return 2;
+    const long rows = n < 1024 ? n : 1024;
+    const size_t shm = (size_t)(16 * E + n + E + 1) * 4 + (size_t)rows * E * 2;
+    if (T > 16 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
-    router_select_align_kernel<<<1, 256, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
+    router_select_align_kernel<<<1, 1024, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
                                                                      gate_out, expert_offsets, sorted_token, sorted_pair, inv);
     FX_CHECK_LAUNCH("router_select_align");
     return 0;

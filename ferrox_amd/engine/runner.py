@@ -171,11 +171,21 @@ class ModelRunner:
                 if len(self._graphs) >= 16:
                     self._graphs.pop(next(iter(self._graphs)))
                 self._graphs[key] = DecodeGraph(self, n_seqs, bound)
-            logits = self._graphs[key].run(tokens, positions, slots,
-                                           [[mgr.table(e.req, k) for e in entries] for k in mgr.groups])
-            for e in entries:
-                mgr.trim(e.req)
-            return logits
+            try:
+                logits = self._graphs[key].run(tokens, positions, slots,
+                                               [[mgr.table(e.req, k) for e in entries] for k in mgr.groups])
+            except RuntimeError as err:
+                # recording is an optimisation of how kernels are launched, not another code path:
+                # if the runtime refuses it, the same kernels are launched one by one from here on
+                import warnings
+                warnings.warn(f"recording decode steps as HIP graphs failed ({err}); launching kernels directly")
+                self.use_graphs = False
+                self._graphs.clear()
+                logits = None
+            if logits is not None:
+                for e in entries:
+                    mgr.trim(e.req)
+                return logits
         max_blocks = max(1, max(mgr.blocks_for(L) for L in kv_lens))
         tables = {}
         flat = tokens + positions + token_seq + slots + rows

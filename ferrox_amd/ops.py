@@ -294,7 +294,7 @@ def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False)
         raise KernelError("route: logits must be float32 [T, E] with unit inner stride")
     T = logits.shape[0]
     dev = logits.device
-    if T <= 64 and logits.shape[1] >= n_experts + (1 if has_gate else 0):
+    if T <= 16 and logits.shape[1] >= n_experts + (1 if has_gate else 0):
         n = T * top_k
         ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
         weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
