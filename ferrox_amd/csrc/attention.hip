@@ -49,17 +49,18 @@ __device__ __forceinline__ const T* value_col(const AttnArgs& a, const int* bt, 
 }
 
 // ---------------------------------------------------------------------------
-// Any number of queries: one wave per (tile of up to 16 queries of one
-// sequence, head); lanes are keys for the scores and head dimensions for the
-// output.
+// Any number of queries.  A work item is a block of up to 64 consecutive
+// queries of one sequence; one wave per (quarter of an item = up to 16 queries,
+// head); lanes are keys for the scores and head dimensions for the output.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
     __shared__ float Qs[TQ][HD_MAX];
     __shared__ float Ps[TQ][64];
-    const int item = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int item = blockIdx.x >> 2, sub = blockIdx.x & 3, h = blockIdx.y, lane = threadIdx.x;
     const int kvh = h / (a.nh / a.nkv);
-    const int tok0 = a.item_tok[item], n = a.item_n[item];
+    const int tok0 = a.item_tok[item] + TQ * sub, n = min(TQ, a.item_n[item] - TQ * sub);
+    if (n <= 0) return;
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
 
@@ -403,9 +404,10 @@ struct WaveAttn {
 // prefill: item = up to 16 consecutive queries of one sequence; block = one wave = (item, head)
 template <int HD>
 __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
-    const int item = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+    const int item = blockIdx.x >> 2, sub = blockIdx.x & 3, h = blockIdx.y, lane = threadIdx.x, li = lane & 15, g = lane >> 4;
     const int kvh = h / (a.nh / a.nkv);
-    const int tok0 = a.item_tok[item], n = a.item_n[item];
+    const int tok0 = a.item_tok[item] + 16 * sub, n = min(16, a.item_n[item] - 16 * sub);
+    if (n <= 0) return;
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int pmin = a.positions[tok0], pmax = a.positions[tok0 + n - 1];
@@ -477,6 +479,182 @@ __global__ __launch_bounds__(64) void attn_mfma_decode_kernel(AttnArgs a) {
     }
 }
 
+// Prefill with the keys and values of a tile shared through LDS: a block of four waves owns up
+// to 64 consecutive queries of one head (16 each); per tile of 64 keys the block stages K
+// (rows permuted so that the 16 keys an MFMA operand needs lie in consecutive rows) and the
+// transposed V once, and every wave takes its operands from there.  While a tile is multiplied
+// the next one is already on its way from memory into registers.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
+    constexpr int KS = HD / 32, CB = HD / 16;
+    constexpr int KROW = HD + 8;          // bf16 elements per staged key row (16 bytes of padding)
+    constexpr int VROW = 64 + 8;          // bf16 elements per staged value row
+    constexpr int KCH = 64 * (HD / 8), VCH = HD * 8;      // 16-byte chunks per tile
+    constexpr int NK = (KCH + 255) / 256, NV = (VCH + 255) / 256;
+    __shared__ __attribute__((aligned(16))) bf16 Ks[64 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 Vs[HD * VROW];
+    const int item = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, g = lane >> 4;
+    const int kvh = h / (a.nh / a.nkv);
+    const int tok_first = a.item_tok[item], n_all = a.item_n[item];
+    const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
+    const int hd = a.hd, bs = a.bs;
+    const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
+    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_end = pmax + 1;
+    // this wave's 16 rows
+    const int tok0 = tok_first + 16 * wave, n = min(16, n_all - 16 * wave);
+    int lo = 1, hi = 0;
+    const bf16* qrow = nullptr;
+    if (li < n) {
+        hi = a.positions[tok0 + li];
+        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * hd;
+    }
+    int w_lo = 0x7fffffff, w_hi = -1;     // keys any row of this wave can see
+    if (n > 0) {
+        w_hi = a.positions[tok0 + n - 1];
+        w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
+    }
+    float m = NEG_INF, l = 0.f;
+    f32x4_t o[CB];
+    bf16x8_t qf[KS];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) o[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < KS; ++u) {
+        const int d = 32 * u + 8 * g;
+        uint4 v = (qrow && d < hd) ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
+        qf[u] = __builtin_bit_cast(bf16x8_t, v);
+    }
+
+    uint4 kreg[NK], vreg[NV];
+    auto fetch = [&](int kt0) {
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int c = tid + i * 256;
+            kreg[i] = make_uint4(0, 0, 0, 0);
+            if (c < KCH) {
+                const int r = c / (HD / 8), d = (c % (HD / 8)) * 8;
+                const int key = kt0 + r;
+                if (key >= kv_begin && key < kv_end && d < hd)
+                    kreg[i] = *(const uint4*)((const bf16*)a.k_pages +
+                                              (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd + d);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = tid + i * 256;
+            vreg[i] = make_uint4(0, 0, 0, 0);
+            if (c < VCH) {
+                const int d = c >> 3, k8 = (c & 7) * 8;
+                const int kg = kt0 + (k8 & ~15);          // pages are read in groups of 16 keys
+                if (d < hd && kg < kv_end && kg + 16 > kv_begin)
+                    vreg[i] = *(const uint4*)((const bf16*)a.v_pages + (((size_t)bt[kg / bs] * a.nkv + kvh) * hd + d) * bs +
+                                              (kt0 + k8) % bs);
+            }
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int c = tid + i * 256;
+            if (c < KCH) {
+                const int r = c / (HD / 8), d = (c % (HD / 8)) * 8;
+                const int row = ((r >> 2) & 3) * 16 + (r >> 4) * 4 + (r & 3);     // key 16a + 4kb + b -> row 16kb + 4a + b
+                *(uint4*)(Ks + row * KROW + d) = kreg[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = tid + i * 256;
+            if (c < VCH) *(uint4*)(Vs + (c >> 3) * VROW + (c & 7) * 8) = vreg[i];
+        }
+    };
+
+    const int kt_first = (kv_begin / 64) * 64;
+    fetch(kt_first);
+    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64) {
+        __syncthreads();          // the previous tile has been read by every wave
+        stage();
+        __syncthreads();
+        if (kt0 + 64 < kv_end) fetch(kt0 + 64);
+        if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;      // nothing in this tile for this wave's rows
+        f32x4_t sc[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < KS; ++u) {
+                const bf16x8_t kf = *(const bf16x8_t*)(Ks + (kb * 16 + li) * KROW + 32 * u + 8 * g);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u], sc[kb], 0, 0, 0);
+            }
+        }
+        float mt = NEG_INF;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kt0 + 16 * g + 4 * kb + r;
+                const float v = (key >= lo && key <= hi) ? sc[kb][r] * a.scale : NEG_INF;
+                sc[kb][r] = v;
+                mt = fmaxf(mt, v);
+            }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
+        float ps = 0.f;
+        uint2 pk[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[r] = (sc[kb][r] == NEG_INF) ? 0.f : expf(sc[kb][r] - m_new);
+                ps += p[r];
+            }
+            pk[kb] = make_uint2(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]));
+        }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * alpha + ps;
+        m = m_new;
+        float al[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const bf16* vr = Vs + (16 * cb + li) * VROW + 16 * g;
+            const uint4 v0 = *(const uint4*)vr, v1 = *(const uint4*)(vr + 8);
+            f32x4_t acc = o[cb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] *= al[r];
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[0]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.x, v0.y)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[1]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.z, v0.w)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[2]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.x, v1.y)), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[3]),
+                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.z, v1.w)), acc, 0, 0, 0);
+            o[cb] = acc;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        const float lr = __shfl(l, row, 64);
+        if (row < n) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int d = 16 * cb + li;
+                if (d < hd) from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * hd + d, o[cb][r] / lr);
+            }
+        }
+    }
+}
+
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
     return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
@@ -492,7 +670,7 @@ static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int
     return 0;
 }
 
-// Queries in tiles: item i covers item_n[i] <= 16 consecutive tokens of one sequence.
+// Queries in blocks: item i covers item_n[i] <= 64 consecutive tokens of one sequence.
 FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
@@ -504,15 +682,15 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
-    dim3 grid(n_items, nh);
+    dim3 grid(n_items * 4, nh), grid_blocks(n_items, nh);     // a wave per 16 queries / a block per item
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
-    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages) && hd % 16 == 0) {
-        if (hd <= 32) attn_mfma_tile_kernel<32><<<grid, 64, 0, s>>>(a);
-        else if (hd <= 64) attn_mfma_tile_kernel<64><<<grid, 64, 0, s>>>(a);
-        else if (hd <= 128) attn_mfma_tile_kernel<128><<<grid, 64, 0, s>>>(a);
-        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
+        if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
+        else if (hd <= 64) attn_mfma_block_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
+        else if (hd <= 128) attn_mfma_block_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
+        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);       // too large to stage in LDS
     } else
         attn_tile_kernel<bf16><<<grid, 64, 0, s>>>(a);
     FX_CHECK_LAUNCH("attn_tiles");

@@ -16,12 +16,12 @@ from .. import ops
 from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec
 from .linear import Linear, same_dtype
 
-TILE_Q = 16   # queries per work item of the tiled kernel
+TILE_Q = 64   # queries per work item of the prefill kernels
 
 
 def attention_items(ctx):
     """Work items of a step, shared by all attention layers: sequences with one
-    new token go to the split decode kernel, the others are cut into tiles of
+    new token go to the split decode kernel, the others are cut into blocks of
     TILE_Q consecutive queries."""
     dec_seq, dec_tok, t_seq, t_tok, t_n = [], [], [], [], []
     max_kv = 1

@@ -175,11 +175,11 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
         qs = q_rot[starts[s]:starts[s + 1]].double().cpu().reshape(L, nh, hd)
         ref[starts[s]:starts[s + 1]] = plain.causal_attention(qs, ks, vs, nh, nkv, window or None)
     ref = ref.reshape(T, nh * hd)
-    # tiles of up to 16 queries
+    # blocks of up to 64 queries
     t_seq, t_tok, t_n = [], [], []
     for s, L in enumerate(seq_lens):
-        for t0 in range(0, L, 16):
-            t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(16, L - t0))
+        for t0 in range(0, L, 64):
+            t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(64, L - t0))
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     out = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
     ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale)
