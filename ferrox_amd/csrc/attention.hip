@@ -30,6 +30,7 @@ struct AttnArgs {
     const int* item_tok;   // per work item: first token
     const int* item_n;     // per work item: number of queries (prefill tiles only)
     int nh, nkv, hd, bs, window;
+    int n_items;
     float scale;
     // decode only
     float* part_o;   // [items, nh, splits, hd]
@@ -256,17 +257,75 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
 // (decode).  For a tile of 64 keys it computes S^T = K Q^T with K as the A
 // operand, so that the accumulator of lane (row = lane%16, g = lane/16) holds 16
 // scores of its own row; the softmax runs on those registers, and the same
-// registers, rounded to bfloat16, are the A operand of O += P V (16x16x16 MFMA,
-// whose lane (row, g) supplies k = 4g..4g+3).  To make that work, A-row i of key
-// block kb reads key 16*(i/4) + 4*kb + i%4 of the tile, and the B operand reads
-// 16 consecutive keys 16g..16g+15 of a transposed value row.
+// registers, rounded to bfloat16, are the A operand of O += P V: two 16x16x32
+// MFMAs per 16 output columns, in which lane (row, g) supplies the probabilities
+// of keys 16g..16g+7 and 16g+8..16g+15.  To make that work, A-row i of key block
+// kb reads key 16*(i/4) + 4*kb + i%4 of the tile, and the B operand reads 16
+// consecutive keys 16g..16g+15 of a transposed value row.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
+#define LOG2E 1.4426950408889634f
+#define LN2 0.6931471805599453f
+
+// One step of the one-pass softmax on a lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r
+// (key0 = tile start + 16g), in base 2: t = score * c with c = scale * log2(e), m and l are the
+// running maximum (of t) and sum of this lane's row, shared by the row's four lanes.  MASKED: only
+// keys in [lo, hi] count.  Returns the factor for what was accumulated so far, and the
+// probabilities rounded to bfloat16: p_lo for keys key0 .. key0+7, p_hi for key0+8 .. key0+15.
+template <bool MASKED>
+__device__ __forceinline__ float softmax_step(f32x4_t (&sc)[4], int key0, int lo, int hi, float c, float& m, float& l,
+                                              uint4& p_lo, uint4& p_hi) {
+    float mt = NEG_INF;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = sc[kb][r] * c;
+            if (MASKED) {
+                const int key = key0 + 4 * kb + r;
+                v = (key >= lo && key <= hi) ? v : NEG_INF;
+            }
+            sc[kb][r] = v;
+            mt = fmaxf(mt, v);
+        }
+    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float m_use = (m_new == NEG_INF) ? 0.f : m_new;      // a row that has seen nothing yet
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);      // exp2(-inf) = 0
+    float ps = 0.f;
+    float p[16];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[4 * kb + r] = __builtin_amdgcn_exp2f(sc[kb][r] - m_use);
+            ps += p[4 * kb + r];
+        }
+    p_lo = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+    p_hi = make_uint4(pack_bf16(p[8], p[9]), pack_bf16(p[10], p[11]), pack_bf16(p[12], p[13]), pack_bf16(p[14], p[15]));
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * ((m_new == NEG_INF) ? 1.f : alpha) + ps;
+    m = m_new;
+    return (m_new == NEG_INF) ? 1.f : alpha;
+}
+
+// O = O * factor(row) + P V for one block of 16 output columns.  The accumulator holds rows
+// 4g+r, so the factors come from the lanes that own those rows; `rescale` is false when every
+// row's factor is 1.
+__device__ __forceinline__ f32x4_t pv_step(f32x4_t acc, bool rescale, const float (&al)[4], uint4 p_lo, uint4 p_hi,
+                                           uint4 v0, uint4 v1) {
+    if (rescale) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] *= al[r];
+    }
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, p_lo), __builtin_bit_cast(bf16x8_t, v0), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, p_hi), __builtin_bit_cast(bf16x8_t, v1), acc, 0, 0, 0);
+    return acc;
 }
 
 template <int HD>   // compile-time bound of head_dim (a.hd <= HD)
@@ -297,36 +356,40 @@ struct WaveAttn {
                                          int lo, int hi) {
         const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
         const int hd = a.hd, bs = a.bs;
+        // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
+        // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
+        const int safe_group = (kv_end - 1) & ~15;
         // values first, so that they arrive while the scores are computed: 16 consecutive keys
         // kt0 + 16g .. of transposed row d = 16*cb + li
         const int kg = kt0 + 16 * g;
-        const bf16* vbase = nullptr;
-        if (kg < kv_end && kg + 16 > kv_begin)
-            vbase = (const bf16*)a.v_pages + ((size_t)bt[kg / bs] * a.nkv + kvh) * hd * bs + kg % bs;
+        const bool vlive = kg < kv_end && kg + 16 > kv_begin;
+        const int vkey = vlive ? kg : safe_group;
+        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)bt[vkey / bs] * a.nkv + kvh) * hd * bs + vkey % bs;
         uint4 vv[EARLY_V ? CB : 1][2];
         if (EARLY_V) {
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const int d = 16 * cb + li;
-                vv[cb][0] = vv[cb][1] = make_uint4(0, 0, 0, 0);
-                if (vbase && d < hd) {
-                    vv[cb][0] = *(const uint4*)(vbase + (size_t)d * bs);
-                    vv[cb][1] = *(const uint4*)(vbase + (size_t)d * bs + 8);
-                }
+                const bf16* vr = vbase + (size_t)(d < hd ? d : 0) * bs;
+                const uint4 x0 = *(const uint4*)vr, x1 = *(const uint4*)(vr + 8);
+                const bool ok = vlive && d < hd;
+                vv[cb][0] = ok ? x0 : make_uint4(0, 0, 0, 0);
+                vv[cb][1] = ok ? x1 : make_uint4(0, 0, 0, 0);
             }
         }
         f32x4_t sc[4];
         uint4 kf[4][KS];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-            const int key = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
-            const bf16* kr = nullptr;
-            if (key >= kv_begin && key < kv_end)
-                kr = (const bf16*)a.k_pages + (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd;
+            const int key0 = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
+            const bool klive = key0 >= kv_begin && key0 < kv_end;
+            const int key = klive ? key0 : safe_group;
+            const bf16* kr = (const bf16*)a.k_pages + (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd;
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
                 const int d = 32 * u + 8 * g;
-                kf[kb][u] = (kr && d < hd) ? *(const uint4*)(kr + d) : make_uint4(0, 0, 0, 0);
+                const uint4 x = *(const uint4*)(kr + (d < hd ? d : 0));
+                kf[kb][u] = (klive && d < hd) ? x : make_uint4(0, 0, 0, 0);
             }
         }
 #pragma unroll
@@ -337,40 +400,14 @@ struct WaveAttn {
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[kb][u]), qf[u], sc[kb], 0, 0, 0);
         }
         // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
-        float mt = NEG_INF;
+        uint4 p_lo, p_hi;
+        const float alpha = softmax_step<true>(sc, kt0 + 16 * g, lo, hi, a.scale * LOG2E, m, l, p_lo, p_hi);
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+        float al[4] = {1.f, 1.f, 1.f, 1.f};
+        if (rescale) {
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = kt0 + 16 * g + 4 * kb + r;
-                const float v = (key >= lo && key <= hi) ? sc[kb][r] * a.scale : NEG_INF;
-                sc[kb][r] = v;
-                mt = fmaxf(mt, v);
-            }
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
-        float ps = 0.f;
-        uint2 pk[4];
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
-            float p[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                p[r] = (sc[kb][r] == NEG_INF) ? 0.f : expf(sc[kb][r] - m_new);
-                ps += p[r];
-            }
-            pk[kb] = make_uint2(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]));
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
         }
-        ps += __shfl_xor(ps, 16, 64);
-        ps += __shfl_xor(ps, 32, 64);
-        l = l * alpha + ps;
-        m = m_new;
-        // the accumulators hold rows 4g+r: fetch their factors from the lanes that own those rows
-        float al[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             uint4 v0, v1;
@@ -379,24 +416,13 @@ struct WaveAttn {
                 v1 = vv[cb][1];
             } else {
                 const int d = 16 * cb + li;
-                v0 = v1 = make_uint4(0, 0, 0, 0);
-                if (vbase && d < hd) {
-                    v0 = *(const uint4*)(vbase + (size_t)d * bs);
-                    v1 = *(const uint4*)(vbase + (size_t)d * bs + 8);
-                }
+                const bf16* vr = vbase + (size_t)(d < hd ? d : 0) * bs;
+                const uint4 x0 = *(const uint4*)vr, x1 = *(const uint4*)(vr + 8);
+                const bool ok = vlive && d < hd;
+                v0 = ok ? x0 : make_uint4(0, 0, 0, 0);
+                v1 = ok ? x1 : make_uint4(0, 0, 0, 0);
             }
-            f32x4_t acc = o[cb];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] *= al[r];
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[0]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.x, v0.y)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[1]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.z, v0.w)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[2]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.x, v1.y)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[3]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.z, v1.w)), acc, 0, 0, 0);
-            o[cb] = acc;
+            o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, v0, v1);
         }
     }
 };
@@ -461,7 +487,7 @@ __global__ __launch_bounds__(64) void attn_mfma_decode_kernel(AttnArgs a) {
     }
     if (li < n && g == 0) {
         float* pml = a.part_ml + (((size_t)item * a.nh + h0 + li) * a.splits + split) * 2;
-        pml[0] = empty ? NEG_INF : w.m;
+        pml[0] = empty ? NEG_INF : w.m * LN2;        // the running maximum is kept in base 2
         pml[1] = empty ? 0.f : w.l;
     }
     if (empty) return;
@@ -493,7 +519,14 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     constexpr int NK = (KCH + 255) / 256, NV = (VCH + 255) / 256;
     __shared__ __attribute__((aligned(16))) bf16 Ks[64 * KROW];
     __shared__ __attribute__((aligned(16))) bf16 Vs[HD * VROW];
-    const int item = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Blocks go to the 8 XCDs in turn, each with an L2 of its own: block b runs on XCD b % 8.  The
+    // (head, item) pairs are dealt out so that an XCD works through whole heads, whose keys and
+    // values then stay in its L2, and the items with the longest key range start first.
+    const int per_xcd = (a.n_items * a.nh + 7) / 8;
+    const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (logical >= a.n_items * a.nh) return;
+    const int h = logical / a.n_items, item = a.n_items - 1 - logical % a.n_items;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, g = lane >> 4;
     const int kvh = h / (a.nh / a.nkv);
     const int tok_first = a.item_tok[item], n_all = a.item_n[item];
@@ -512,10 +545,16 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * hd;
     }
     int w_lo = 0x7fffffff, w_hi = -1;     // keys any row of this wave can see
+    int w_lo_max = 0x7fffffff, w_hi_min = -1;   // keys every row of this wave sees: [w_lo_max, w_hi_min]
     if (n > 0) {
         w_hi = a.positions[tok0 + n - 1];
         w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
+        if (n == 16) {                    // a wave with idle rows masks always
+            w_hi_min = a.positions[tok0];
+            w_lo_max = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
+        }
     }
+    const float c2 = a.scale * LOG2E;
     float m = NEG_INF, l = 0.f;
     f32x4_t o[CB];
     bf16x8_t qf[KS];
@@ -528,34 +567,45 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         qf[u] = __builtin_bit_cast(bf16x8_t, v);
     }
 
-    uint4 kreg[NK], vreg[NV];
-    auto fetch = [&](int kt0) {
+    uint4 kreg_a[NK], vreg_a[NV], kreg_b[NK], vreg_b[NV];     // two tiles on their way from memory
+    // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
+    // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
+    const int safe_group = (kv_end - 1) & ~15;
+    auto fetch = [&](uint4* kreg, uint4* vreg, int kt0) {
+        size_t kbase[4], vbase[4];     // page and slot of each group of 16 keys of the tile (the same for all threads)
+        bool live[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int key0 = kt0 + 16 * j;
+            live[j] = key0 < kv_end && key0 + 16 > kv_begin;
+            const int key = live[j] ? key0 : safe_group;
+            const size_t page = bt[key / bs];
+            kbase[j] = ((page * a.nkv + kvh) * bs + key % bs) * hd;
+            vbase[j] = (page * a.nkv + kvh) * hd * bs + key % bs;
+        }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
             const int c = tid + i * 256;
-            kreg[i] = make_uint4(0, 0, 0, 0);
             if (c < KCH) {
                 const int r = c / (HD / 8), d = (c % (HD / 8)) * 8;
                 const int key = kt0 + r;
-                if (key >= kv_begin && key < kv_end && d < hd)
-                    kreg[i] = *(const uint4*)((const bf16*)a.k_pages +
-                                              (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd + d);
+                const bool ok = key >= kv_begin && key < kv_end && d < hd;
+                const uint4 v = *(const uint4*)((const bf16*)a.k_pages + kbase[r >> 4] + (size_t)(r & 15) * hd + (d < hd ? d : 0));
+                kreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = tid + i * 256;
-            vreg[i] = make_uint4(0, 0, 0, 0);
             if (c < VCH) {
                 const int d = c >> 3, k8 = (c & 7) * 8;
-                const int kg = kt0 + (k8 & ~15);          // pages are read in groups of 16 keys
-                if (d < hd && kg < kv_end && kg + 16 > kv_begin)
-                    vreg[i] = *(const uint4*)((const bf16*)a.v_pages + (((size_t)bt[kg / bs] * a.nkv + kvh) * hd + d) * bs +
-                                              (kt0 + k8) % bs);
+                const bool ok = d < hd && live[k8 >> 4];
+                const uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < hd ? d : 0) * bs + (k8 & 15));
+                vreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](const uint4* kreg, const uint4* vreg) {
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
             const int c = tid + i * 256;
@@ -573,12 +623,16 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     };
 
     const int kt_first = (kv_begin / 64) * 64;
-    fetch(kt_first);
-    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64) {
-        __syncthreads();          // the previous tile has been read by every wave
-        stage();
-        __syncthreads();
-        if (kt0 + 64 < kv_end) fetch(kt0 + 64);
+    fetch(kreg_a, vreg_a, kt_first);
+    if (kt_first + 64 < kv_end) fetch(kreg_b, vreg_b, kt_first + 64);
+    int parity = 0;
+    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, parity ^= 1) {
+        lds_barrier();            // the previous tile has been read by every wave
+        if (parity == 0) stage(kreg_a, vreg_a); else stage(kreg_b, vreg_b);
+        lds_barrier();
+        if (kt0 + 128 < kv_end) {  // the registers just emptied take the tile after the next
+            if (parity == 0) fetch(kreg_a, vreg_a, kt0 + 128); else fetch(kreg_b, vreg_b, kt0 + 128);
+        }
         if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;      // nothing in this tile for this wave's rows
         f32x4_t sc[4];
 #pragma unroll
@@ -590,55 +644,21 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u], sc[kb], 0, 0, 0);
             }
         }
-        float mt = NEG_INF;
+        // tiles that every row of this wave sees whole need no mask
+        const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
+        uint4 p_lo, p_hi;
+        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi);
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+        float al[4] = {1.f, 1.f, 1.f, 1.f};
+        if (rescale) {
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = kt0 + 16 * g + 4 * kb + r;
-                const float v = (key >= lo && key <= hi) ? sc[kb][r] * a.scale : NEG_INF;
-                sc[kb][r] = v;
-                mt = fmaxf(mt, v);
-            }
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
-        float ps = 0.f;
-        uint2 pk[4];
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
-            float p[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                p[r] = (sc[kb][r] == NEG_INF) ? 0.f : expf(sc[kb][r] - m_new);
-                ps += p[r];
-            }
-            pk[kb] = make_uint2(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]));
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
         }
-        ps += __shfl_xor(ps, 16, 64);
-        ps += __shfl_xor(ps, 32, 64);
-        l = l * alpha + ps;
-        m = m_new;
-        float al[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             const bf16* vr = Vs + (16 * cb + li) * VROW + 16 * g;
-            const uint4 v0 = *(const uint4*)vr, v1 = *(const uint4*)(vr + 8);
-            f32x4_t acc = o[cb];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] *= al[r];
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[0]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.x, v0.y)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[1]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v0.z, v0.w)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[2]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.x, v1.y)), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, pk[3]),
-                                                           __builtin_bit_cast(s16x4_t, make_uint2(v1.z, v1.w)), acc, 0, 0, 0);
-            o[cb] = acc;
+            o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, *(const uint4*)vr, *(const uint4*)(vr + 8));
         }
     }
 #pragma unroll
@@ -682,7 +702,8 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
-    dim3 grid(n_items * 4, nh), grid_blocks(n_items, nh);     // a wave per 16 queries / a block per item
+    a.n_items = n_items;
+    dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);

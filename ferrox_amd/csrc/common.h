@@ -47,17 +47,21 @@ struct bf16 {
 
 __device__ __forceinline__ float bf16_to_float(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN (the hardware conversion of gfx950)
 __device__ __forceinline__ bf16 float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
+    const __bf16 b = (__bf16)f;
     bf16 r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = (uint16_t)((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = (uint16_t)(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, b);
     return r;
+}
+
+// two floats to two packed bfloat16 (first in the low half)
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    bf16x2_t v;
+    v[0] = (__bf16)a;
+    v[1] = (__bf16)b;
+    return __builtin_bit_cast(uint32_t, v);
 }
 
 __device__ __forceinline__ float to_float(float v) { return v; }
@@ -94,6 +98,13 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) s += red[i];
     return s;
+}
+
+// A block barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for
+// every global load in flight, which would stall a pipeline that fetches tiles ahead of their
+// use; the compiler still waits for a load where its registers are consumed.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
