@@ -36,6 +36,7 @@ struct GemmArgs {
     int E;
     int M, N, K;
     int vec_ok;  // 16-byte loads are legal for A and W
+    int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
 
 // block -> (first logical row, end of rows, expert).  Plain: tiles of TM rows.
@@ -77,10 +78,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define BK 64
 #define LDS_STRIDE (BK + 8)  // bf16 elements; keeps 16-byte reads of 16 rows on distinct banks
 
-__device__ __forceinline__ uint4 load_chunk(const bf16* row, int k, int K, int vec_ok) {
+template <bool VEC>   // VEC: K is a multiple of 8 and rows are 16-byte aligned
+__device__ __forceinline__ uint4 load_chunk(const bf16* row, int k, int K) {
     uint4 v = make_uint4(0, 0, 0, 0);
     if (!row || k >= K) return v;
-    if (vec_ok && k + 8 <= K) return *(const uint4*)(row + k);
+    if (VEC) return *(const uint4*)(row + k);
     uint16_t tmp[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) tmp[i] = (k + i < K) ? row[k + i].bits : (uint16_t)0;
@@ -93,7 +95,7 @@ __device__ __forceinline__ uint4 load_chunk(const bf16* row, int k, int K, int v
 
 // TM x TN block tile (TN counts weight rows: in dual mode half of them are gate
 // rows and half up rows, interleaved in groups of 16), 4 waves of WM x WN.
-template <int TM, int TN, int WM, int WN, bool DUAL, int EPI>
+template <int TM, int TN, int WM, int WN, bool DUAL, int EPI, bool VEC>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
     constexpr int WAVES_N = TN / WN;
     static_assert((TM / WM) * WAVES_N == 4, "four waves per block");
@@ -103,10 +105,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) bf16 As[TM * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) bf16 Bs[TN * LDS_STRIDE];
 
+    // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), each with an L2 of its own: the
+    // tiles are dealt out so that an XCD works through a contiguous range of column tiles, rows
+    // fastest, and the weights of those columns stay in its L2.
+    const int per_xcd = (g.n_col_tiles * g.n_row_tiles + 7) / 8;
+    const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (logical >= g.n_col_tiles * g.n_row_tiles) return;
     int r0, r_end, expert;
-    locate_rows<TM>(g, blockIdx.y, r0, r_end, expert);
+    locate_rows<TM>(g, logical % g.n_row_tiles, r0, r_end, expert);
     if (r0 < 0) return;
-    const int n0 = blockIdx.x * OUT_TN;
+    const int n0 = (logical / g.n_row_tiles) * OUT_TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const bf16* Abase = (const bf16*)g.A;
@@ -144,49 +152,54 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-    uint4 a_reg[NA], b_reg[NB];
+    // Two tiles are on their way from memory into registers while a third is multiplied out of LDS.
+    uint4 a0[NA], b0[NB], a1[NA], b1[NB];
     const int kc = (tid & 7) * 8;
-#pragma unroll
-    for (int i = 0; i < NA; ++i) a_reg[i] = load_chunk(a_src[i], kc, g.K, g.vec_ok);
-#pragma unroll
-    for (int i = 0; i < NB; ++i) b_reg[i] = load_chunk(b_src[i], kc, g.K, g.vec_ok);
-
-    for (int k0 = 0; k0 < g.K; k0 += BK) {
-        __syncthreads();  // the previous tile has been read
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            const int c = tid + i * 256;
-            if (c < TM * 8) *(uint4*)(As + (c >> 3) * LDS_STRIDE + kc) = a_reg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            const int c = tid + i * 256;
-            if (c < TN * 8) *(uint4*)(Bs + (c >> 3) * LDS_STRIDE + kc) = b_reg[i];
-        }
-        __syncthreads();
-        if (k0 + BK < g.K) {  // fetch the next tile while this one is multiplied
-#pragma unroll
-            for (int i = 0; i < NA; ++i) a_reg[i] = load_chunk(a_src[i], k0 + BK + kc, g.K, g.vec_ok);
-#pragma unroll
-            for (int i = 0; i < NB; ++i) b_reg[i] = load_chunk(b_src[i], k0 + BK + kc, g.K, g.vec_ok);
-        }
-#pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-            const int koff = ks * 32 + (lane >> 4) * 8;
-            bf16x8_t af[MT], bfr[NT];
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-                af[i] = *(const bf16x8_t*)(As + (wm * WM + i * 16 + (lane & 15)) * LDS_STRIDE + koff);
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-                bfr[j] = *(const bf16x8_t*)(Bs + (wn * WN + j * 16 + (lane & 15)) * LDS_STRIDE + koff);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int j = 0; j < NT; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
+#define FX_FETCH(AR, BR, K0)                                                                  \
+    {                                                                                         \
+        _Pragma("unroll") for (int i = 0; i < NA; ++i) AR[i] = load_chunk<VEC>(a_src[i], (K0) + kc, g.K); \
+        _Pragma("unroll") for (int i = 0; i < NB; ++i) BR[i] = load_chunk<VEC>(b_src[i], (K0) + kc, g.K); \
     }
+#define FX_STAGE(AR, BR)                                                                      \
+    {                                                                                         \
+        _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                      \
+            const int c = tid + i * 256;                                                      \
+            if (c < TM * 8) *(uint4*)(As + (c >> 3) * LDS_STRIDE + kc) = AR[i];               \
+        }                                                                                     \
+        _Pragma("unroll") for (int i = 0; i < NB; ++i) {                                      \
+            const int c = tid + i * 256;                                                      \
+            if (c < TN * 8) *(uint4*)(Bs + (c >> 3) * LDS_STRIDE + kc) = BR[i];               \
+        }                                                                                     \
+    }
+#define FX_MULTIPLY()                                                                         \
+    _Pragma("unroll") for (int ks = 0; ks < BK / 32; ++ks) {                                  \
+        const int koff = ks * 32 + (lane >> 4) * 8;                                           \
+        bf16x8_t af[MT], bfr[NT];                                                             \
+        _Pragma("unroll") for (int i = 0; i < MT; ++i)                                        \
+            af[i] = *(const bf16x8_t*)(As + (wm * WM + i * 16 + (lane & 15)) * LDS_STRIDE + koff); \
+        _Pragma("unroll") for (int j = 0; j < NT; ++j)                                        \
+            bfr[j] = *(const bf16x8_t*)(Bs + (wn * WN + j * 16 + (lane & 15)) * LDS_STRIDE + koff); \
+        _Pragma("unroll") for (int i = 0; i < MT; ++i)                                        \
+            _Pragma("unroll") for (int j = 0; j < NT; ++j)                                    \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0); \
+    }
+    FX_FETCH(a0, b0, 0);
+    FX_FETCH(a1, b1, BK);          // beyond K this loads zeros
+    for (int k0 = 0; k0 < g.K; k0 += 2 * BK) {
+        lds_barrier();  // the previous tile has been read
+        FX_STAGE(a0, b0);
+        lds_barrier();
+        FX_FETCH(a0, b0, k0 + 2 * BK);
+        FX_MULTIPLY();
+        lds_barrier();
+        FX_STAGE(a1, b1);           // a tile of zeros if K ends before it
+        lds_barrier();
+        FX_FETCH(a1, b1, k0 + 3 * BK);
+        FX_MULTIPLY();
+    }
+#undef FX_FETCH
+#undef FX_STAGE
+#undef FX_MULTIPLY
 
     // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
 #pragma unroll
@@ -383,7 +396,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             const bool kin = k0 + kk < g.K;
             As[kk][row] = (a_src[i] && kin) ? a_src[i][k0 + kk] : 0.f;
             Bs[0][kk][row] = (b_src[i] && kin) ? b_src[i][k0 + kk] : 0.f;
-            if (DUAL) Bs[1][kk][row] = (b_src[i] && kin) ? b_src[i][g.up_offset + k0 + kk] : 0.f;
+            if (DUAL) Bs[DUAL ? 1 : 0][kk][row] = (b_src[i] && kin) ? b_src[i][g.up_offset + k0 + kk] : 0.f;
         }
         __syncthreads();
 #pragma unroll
@@ -395,7 +408,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             for (int j = 0; j < 4; ++j) b[j] = Bs[0][k][tx * 4 + j];
             if (DUAL) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) b2[j] = Bs[1][k][tx * 4 + j];
+                for (int j = 0; j < 4; ++j) b2[j] = Bs[DUAL ? 1 : 0][k][tx * 4 + j];
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -436,15 +449,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
 // host side
 // ===========================================================================
 template <int TM, int TN, int WM, int WN>
-static void launch_bf16(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
+static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
     const bool dual = epi == EPI_SILU_MUL;
-    dim3 grid(ceil_div(g.N, dual ? TN / 2 : TN), m_tiles);
+    g.n_col_tiles = ceil_div(g.N, dual ? TN / 2 : TN);
+    g.n_row_tiles = m_tiles;
+    dim3 grid(8 * ceil_div((long)g.n_col_tiles * g.n_row_tiles, 8));
+#define FX_TILED(DUAL_, EPI_)                                                                       \
+    if (g.vec_ok) gemm_bf16_kernel<TM, TN, WM, WN, DUAL_, EPI_, true><<<grid, 256, 0, s>>>(g);     \
+    else gemm_bf16_kernel<TM, TN, WM, WN, DUAL_, EPI_, false><<<grid, 256, 0, s>>>(g)
     switch (epi) {
-        case EPI_STORE: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_STORE><<<grid, 256, 0, s>>>(g); break;
-        case EPI_STORE_F32: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_STORE_F32><<<grid, 256, 0, s>>>(g); break;
-        case EPI_RESID: gemm_bf16_kernel<TM, TN, WM, WN, false, EPI_RESID><<<grid, 256, 0, s>>>(g); break;
-        default: gemm_bf16_kernel<TM, TN, WM, WN, true, EPI_SILU_MUL><<<grid, 256, 0, s>>>(g); break;
+        case EPI_STORE: FX_TILED(false, EPI_STORE); break;
+        case EPI_STORE_F32: FX_TILED(false, EPI_STORE_F32); break;
+        case EPI_RESID: FX_TILED(false, EPI_RESID); break;
+        default: FX_TILED(true, EPI_SILU_MUL); break;
     }
+#undef FX_TILED
 }
 
 template <int MT, int WAVES, int NW>
@@ -531,7 +550,12 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else {
         const int m_tiles = M / 128 + (expert_offsets ? nonempty : (M % 128 != 0));
-        launch_bf16<128, 128, 64, 64>(g, epi, m_tiles, s);
+        const bool dual = epi == EPI_SILU_MUL;
+        // narrow outputs: tiles of 64 columns give the 256 CUs at least two blocks each
+        if (!dual && (long)ceil_div(N, 128) * m_tiles < 512)
+            launch_bf16<128, 64, 64, 32>(g, epi, m_tiles, s);
+        else
+            launch_bf16<128, 128, 64, 64>(g, epi, m_tiles, s);
     }
     FX_CHECK_LAUNCH("gemm_bf16");
     return 0;
