@@ -1,6 +1,10 @@
 """Book-keeping of the cache: pages, block tables, state slots.  Host side only;
 the device memory the ids point into is owned by `CacheStorage`.
 
+The book-keeping itself is native code (`csrc/host_runtime.cpp`, loaded through
+ctypes); this module is its Python face: it maps request names to handles and
+group keys to indexes, and turns error codes into exceptions.
+
 Layers with the same need share a *group*: one pool of page ids and one block
 table per request (a page id indexes a slab of every layer of the group).  A
 group is either "all keys" (window None) or "the last W keys".  The reference
@@ -17,177 +21,296 @@ Freed pages go to the top of a LIFO list and are handed out again first.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes
+
+import numpy as np
+
+from ..csrc.build import load_library
+
+_I32P = ctypes.POINTER(ctypes.c_int)
+_I64P = ctypes.POINTER(ctypes.c_int64)
+_lib = None
+
+
+def _native():
+    global _lib
+    if _lib is None:
+        lib = load_library("host_runtime")
+        lib.fxc_create.restype = ctypes.c_void_p
+        lib.fxc_create.argtypes = [ctypes.c_int, _I32P, _I32P, ctypes.c_int, ctypes.c_int]
+        lib.fxc_destroy.argtypes = [ctypes.c_void_p]
+        lib.fxc_destroy.restype = None
+        lib.fxc_last_error.restype = ctypes.c_char_p
+        lib.fxc_last_error.argtypes = [ctypes.c_void_p]
+        for name, extra in (("admit", []), ("contains", []), ("length", []), ("slot", []), ("trim", []),
+                            ("pages_needed", [ctypes.c_int, ctypes.c_int]), ("extend", [ctypes.c_int, ctypes.c_int]),
+                            ("table", [ctypes.c_int, _I32P, ctypes.c_int])):
+            fn = getattr(lib, "fxc_" + name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.c_void_p, ctypes.c_int64] + extra
+        lib.fxc_release.restype = None
+        lib.fxc_release.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+        for name, extra in (("n_free_pages", [ctypes.c_int]), ("num_pages", [ctypes.c_int]), ("n_free_slots", []),
+                            ("n_requests", []), ("check", []), ("pool_take", [ctypes.c_int, ctypes.c_int, _I32P]),
+                            ("pool_give", [ctypes.c_int, ctypes.c_int]), ("slot_take", []), ("slot_give", [ctypes.c_int])):
+            fn = getattr(lib, "fxc_" + name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.c_void_p] + extra
+        lib.fxc_pack_step.restype = ctypes.c_long
+        lib.fxc_pack_step.argtypes = [ctypes.c_void_p, ctypes.c_int, _I64P, _I32P, _I32P, _I32P, _I32P, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_void_p, ctypes.c_long, _I32P, _I32P, _I32P]
+        _lib = lib
+    return _lib
+
+
+class _Core:
+    """Owns one native manager."""
+
+    def __init__(self, windows: list, num_pages: list, block_size: int, n_slots: int):
+        for n in num_pages:
+            if n < 0:
+                raise ValueError("num_pages must be >= 0")
+        if block_size < 1:
+            raise ValueError("block_size must be >= 1")
+        self.lib = _native()
+        n = len(windows)
+        w = (ctypes.c_int * max(n, 1))(*[-1 if x is None else int(x) for x in windows])
+        p = (ctypes.c_int * max(n, 1))(*[int(x) for x in num_pages])
+        self.h = self.lib.fxc_create(n, w, p, block_size, n_slots)
+        if not self.h:
+            raise ValueError("the cache manager refused its sizes")
+
+    def __del__(self):
+        h, self.h = getattr(self, "h", None), None
+        if h:
+            self.lib.fxc_destroy(h)
+
+    def error(self) -> str:
+        return self.lib.fxc_last_error(self.h).decode()
 
 
 class PagePool:
+    """One pool of page ids on its own."""
+
     def __init__(self, num_pages: int):
-        if num_pages < 0:
-            raise ValueError("num_pages must be >= 0")
+        self._core = _Core([None], [num_pages], 1, 0)
         self.num_pages = num_pages
-        self._free = list(range(num_pages - 1, -1, -1))      # pop() hands out 0, 1, 2, ... at first
-        self._is_free = [True] * num_pages
 
     @property
     def n_free(self) -> int:
-        return len(self._free)
+        return self._core.lib.fxc_n_free_pages(self._core.h, 0)
 
     def alloc(self, n: int):
         """n page ids, or None (and no change) if fewer are free."""
-        if n > len(self._free):
+        out = (ctypes.c_int * max(n, 1))()
+        if not self._core.lib.fxc_pool_take(self._core.h, 0, n, out):
             return None
-        out = [self._free.pop() for _ in range(n)]
-        for p in out:
-            self._is_free[p] = False
-        return out
+        return list(out[:n])
 
     def free(self, pages) -> None:
         for p in pages:
-            if not 0 <= p < self.num_pages:
-                raise ValueError(f"page {p} does not belong to this pool")
-            if self._is_free[p]:
-                raise ValueError(f"page {p} freed twice")
-            self._is_free[p] = True
-            self._free.append(p)
+            if not self._core.lib.fxc_pool_give(self._core.h, 0, int(p)):
+                raise ValueError(f"page {p} does not belong to this pool or is freed twice")
 
 
 class StateSlots:
     """Slots for per-request state of fixed size (sampler state, a recurrent mixer's state)."""
 
     def __init__(self, n_slots: int):
+        self._core = _Core([], [], 1, n_slots)
         self.n_slots = n_slots
-        self._free = list(range(n_slots - 1, -1, -1))
-        self._used: set[int] = set()
 
     @property
     def n_free(self) -> int:
-        return len(self._free)
+        return self._core.lib.fxc_n_free_slots(self._core.h)
 
     def alloc(self):
-        if not self._free:
-            return None
-        s = self._free.pop()
-        self._used.add(s)
-        return s
+        s = self._core.lib.fxc_slot_take(self._core.h)
+        return None if s < 0 else s
 
     def free(self, slot: int) -> None:
-        if slot not in self._used:
+        if not self._core.lib.fxc_slot_give(self._core.h, int(slot)):
             raise ValueError(f"slot {slot} is not in use")
-        self._used.remove(slot)
-        self._free.append(slot)
 
 
-@dataclass
+class _PoolView:
+    def __init__(self, mgr, index):
+        self._m, self._g = mgr, index
+
+    @property
+    def n_free(self) -> int:
+        return self._m._lib.fxc_n_free_pages(self._m._h, self._g)
+
+    @property
+    def num_pages(self) -> int:
+        return self._m._lib.fxc_num_pages(self._m._h, self._g)
+
+
+class _TablesView:
+    def __init__(self, mgr, key):
+        self._m, self._key = mgr, key
+
+    def __getitem__(self, req) -> list:
+        return self._m.table(req, self._key)
+
+
 class Group:
-    key: object
-    window: int | None
-    pool: PagePool
-    tables: dict = field(default_factory=dict)     # request -> list of page ids, -1 where given back
+    """What one group shows: its key, its window, its pool's counts and the block tables."""
+
+    def __init__(self, mgr, key, window, index):
+        self.key, self.window, self.index = key, window, index
+        self.pool = _PoolView(mgr, index)
+        self.tables = _TablesView(mgr, key)
 
 
-@dataclass
-class Sequence:
-    slot: int
-    length: int = 0
+class _SlotsView:
+    def __init__(self, mgr, n_slots):
+        self._m, self.n_slots = mgr, n_slots
+
+    @property
+    def n_free(self) -> int:
+        return self._m._lib.fxc_n_free_slots(self._m._h)
+
+
+class PackedStep:
+    """A step's batch as the native packer laid it out in a host int32 buffer:
+    tokens[T] | positions[T] | token_seq[T] | slots[n] | rows[R] | tables[groups][n][max_blocks]."""
+    __slots__ = ("total", "n_tokens", "n_rows", "max_blocks", "starts", "lens")
+
+    def __init__(self, total, n_tokens, n_rows, max_blocks, starts, lens):
+        self.total, self.n_tokens, self.n_rows, self.max_blocks = total, n_tokens, n_rows, max_blocks
+        self.starts, self.lens = starts, lens
 
 
 class CacheManager:
     def __init__(self, groups: dict, num_pages, block_size: int, n_slots: int):
         """`groups`: key -> window (None = all keys).  `num_pages`: an int for every group, or key -> int."""
-        if block_size < 1:
-            raise ValueError("block_size must be >= 1")
+        keys = list(groups)
+        pages = [num_pages[k] if isinstance(num_pages, dict) else num_pages for k in keys]
+        self._core = _Core([groups[k] for k in keys], pages, block_size, n_slots)
+        self._lib, self._h = self._core.lib, self._core.h
         self.block_size = block_size
-        self.groups: dict = {}
-        for key, window in groups.items():
-            n = num_pages[key] if isinstance(num_pages, dict) else num_pages
-            self.groups[key] = Group(key, window, PagePool(n))
-        self.slots = StateSlots(n_slots)
-        self.seqs: dict = {}
+        self.groups = {k: Group(self, k, groups[k], i) for i, k in enumerate(keys)}
+        self.slots = _SlotsView(self, n_slots)
+        self._handles: dict = {}        # request name -> handle
+        self._next = 0
 
     # ---- requests --------------------------------------------------------
+    def _handle(self, req) -> int:
+        h = self._handles.get(req)
+        if h is None:
+            raise ValueError(f"request {req!r} is not admitted")
+        return h
+
+    def _checked(self, code: int) -> int:
+        if code == -2:
+            raise ValueError(self._core.error())
+        return code
+
     def admit(self, req) -> int | None:
         """A state slot and empty block tables; None if no slot is free."""
-        if req in self.seqs:
+        if req in self._handles:
             raise ValueError(f"request {req!r} is already admitted")
-        slot = self.slots.alloc()
-        if slot is None:
+        slot = self._checked(self._lib.fxc_admit(self._h, self._next))
+        if slot < 0:
             return None
-        self.seqs[req] = Sequence(slot)
-        for g in self.groups.values():
-            g.tables[req] = []
+        self._handles[req] = self._next
+        self._next += 1
         return slot
 
     def __contains__(self, req) -> bool:
-        return req in self.seqs
+        return req in self._handles
 
-    def _seq(self, req) -> Sequence:
-        seq = self.seqs.get(req)
-        if seq is None:
-            raise ValueError(f"request {req!r} is not admitted")
-        return seq
+    @property
+    def seqs(self) -> dict:
+        """request -> length, for inspection"""
+        return {r: self.length(r) for r in self._handles}
 
     def length(self, req) -> int:
-        return self._seq(req).length
+        return self._checked(self._lib.fxc_length(self._h, self._handle(req)))
 
     def slot(self, req) -> int:
-        return self._seq(req).slot
+        return self._checked(self._lib.fxc_slot(self._h, self._handle(req)))
 
     def table(self, req, key) -> list:
-        return self.groups[key].tables[req]
+        h, g = self._handle(req), self.groups[key].index
+        n = self._checked(self._lib.fxc_table(self._h, h, g, None, 0))
+        out = (ctypes.c_int * max(n, 1))()
+        self._lib.fxc_table(self._h, h, g, out, n)
+        return list(out[:n])
 
     def blocks_for(self, length: int) -> int:
         return -(-length // self.block_size)
 
     def pages_needed(self, req, new_len: int) -> dict:
         """key -> number of pages `extend(req, new_len)` would take."""
-        return {k: max(0, self.blocks_for(new_len) - len(g.tables[req])) for k, g in self.groups.items()}
+        h = self._handle(req)
+        return {k: self._checked(self._lib.fxc_pages_needed(self._h, h, new_len, g.index))
+                for k, g in self.groups.items()}
 
     def can_extend(self, req, new_len: int) -> bool:
-        need = self.pages_needed(req, new_len)
-        return all(self.groups[k].pool.n_free >= n for k, n in need.items())
+        return self._checked(self._lib.fxc_extend(self._h, self._handle(req), new_len, 1)) == 1
 
     def extend(self, req, new_len: int) -> bool:
         """Pages for positions [length, new_len) in every group, all or nothing; sets the length."""
-        seq = self._seq(req)
-        if new_len < seq.length:
-            raise ValueError("a sequence cannot shrink")
-        need = self.pages_needed(req, new_len)
-        if any(self.groups[k].pool.n_free < n for k, n in need.items()):
-            return False
-        for k, n in need.items():
-            g = self.groups[k]
-            g.tables[req].extend(g.pool.alloc(n))
-        seq.length = new_len
-        return True
+        return self._checked(self._lib.fxc_extend(self._h, self._handle(req), new_len, 0)) == 1
 
     def trim(self, req) -> int:
         """Give back pages that a window has passed: every query from now on stands at
         position >= length and sees keys t with position - t < W, so t >= length - W + 1.
         Returns the number of pages freed."""
-        seq = self._seq(req)
-        freed = 0
-        for g in self.groups.values():
-            if g.window is None:
-                continue
-            first_needed = seq.length - g.window + 1
-            if first_needed <= 0:
-                continue
-            table = g.tables[req]
-            for b in range(min(first_needed // self.block_size, len(table))):
-                if table[b] >= 0:
-                    g.pool.free([table[b]])
-                    table[b] = -1
-                    freed += 1
-        return freed
+        return self._checked(self._lib.fxc_trim(self._h, self._handle(req)))
 
     def release(self, req) -> None:
         """Everything the request holds goes back; a second call does nothing."""
-        seq = self.seqs.pop(req, None)
-        if seq is None:
-            return
-        for g in self.groups.values():
-            g.pool.free([p for p in g.tables.pop(req) if p >= 0])
-        self.slots.free(seq.slot)
+        h = self._handles.pop(req, None)
+        if h is not None:
+            self._lib.fxc_release(self._h, h)
+
+    # ---- the step's batch ----------------------------------------------------
+    def pack_step(self, reqs: list, token_lists: list, wants: list, vocab: int, out_ptr: int, capacity: int,
+                  force_blocks: int = 0) -> PackedStep:
+        """Lay the batch out in the host buffer at `out_ptr` (room for `capacity` int32).
+        Checks every id and place; raises ValueError naming the request at fault."""
+        n = len(reqs)
+        handles = np.empty(n, dtype=np.int64)
+        for i, r in enumerate(reqs):
+            h = self._handles.get(r)
+            if h is None:
+                raise ValueError(f"request {r!r} was not admitted")
+            handles[i] = h
+        n_tok = np.fromiter((len(t) for t in token_lists), dtype=np.int32, count=n)
+        try:
+            tokens = np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for t in token_lists]) if n else \
+                np.empty(0, dtype=np.int64)
+            flat_want = np.concatenate([np.asarray(w, dtype=np.int64).reshape(-1) for w in wants]) if n else \
+                np.empty(0, dtype=np.int64)
+        except (OverflowError, TypeError, ValueError) as e:
+            raise ValueError(f"token ids and wanted places must be integers: {e}") from None
+        if tokens.size and (tokens.min() < 0 or tokens.max() >= vocab):
+            bad = int(tokens[(tokens < 0) | (tokens >= vocab)][0])
+            raise ValueError(f"token id {bad} is outside the vocabulary of {vocab}")     # ferrox-cli/src/run.rs:598-601
+        if flat_want.size and (flat_want.min() < -(2 ** 31) or flat_want.max() >= 2 ** 31):
+            raise ValueError("a wanted place is outside its request's tokens")
+        tokens, flat_want = tokens.astype(np.int32), flat_want.astype(np.int32)
+        want_start = np.zeros(n + 1, dtype=np.int32)
+        np.cumsum([len(w) for w in wants], out=want_start[1:])
+        sizes = np.zeros(3, dtype=np.int32)
+        starts, lens = np.zeros(max(n, 1), dtype=np.int32), np.zeros(max(n, 1), dtype=np.int32)
+        ip = lambda a: a.ctypes.data_as(_I32P)
+        total = self._lib.fxc_pack_step(self._h, n, handles.ctypes.data_as(_I64P), ip(n_tok), ip(tokens), ip(want_start),
+                                        ip(flat_want), vocab, force_blocks, out_ptr, capacity, ip(sizes), ip(starts),
+                                        ip(lens))
+        if total < 0:
+            msg = self._core.error()
+            by_handle = {h: r for r, h in self._handles.items()}
+            for h, r in by_handle.items():              # name the request as the caller knows it
+                msg = msg.replace(f"request {h} ", f"request {r!r} ").replace(f"request {h}:", f"request {r!r}:")
+            raise ValueError(msg)
+        return PackedStep(int(total), int(sizes[0]), int(sizes[1]), int(sizes[2]), starts[:n].tolist(), lens[:n].tolist())
+
+    def step_words(self, n_tokens: int, n_seqs: int, n_rows: int, max_blocks: int) -> int:
+        return 3 * n_tokens + n_seqs + n_rows + len(self.groups) * n_seqs * max_blocks
 
     # ---- accounting --------------------------------------------------------
     def n_free_pages(self, key=None) -> int:
@@ -196,24 +319,7 @@ class CacheManager:
         return min(g.pool.n_free for g in self.groups.values()) if self.groups else 0
 
     def check_invariants(self) -> None:
-        for g in self.groups.values():
-            held = [p for t in g.tables.values() for p in t if p >= 0]
-            if len(held) != len(set(held)):
-                raise AssertionError(f"group {g.key!r}: a page is held twice")
-            free = list(g.pool._free)
-            if len(free) != len(set(free)):
-                raise AssertionError(f"group {g.key!r}: a page is in the free list twice")
-            if set(free) & set(held):
-                raise AssertionError(f"group {g.key!r}: a page is both free and held")
-            if len(free) + len(held) != g.pool.num_pages:
-                raise AssertionError(f"group {g.key!r}: {g.pool.num_pages - len(free) - len(held)} pages lost")
-            if set(g.tables) != set(self.seqs):
-                raise AssertionError(f"group {g.key!r}: tables and sequences differ")
-            for req, t in g.tables.items():
-                if len(t) < self.blocks_for(self.seqs[req].length):
-                    raise AssertionError(f"group {g.key!r}: request {req!r} has too few blocks")
-        slots = [s.slot for s in self.seqs.values()]
-        if len(slots) != len(set(slots)):
-            raise AssertionError("a state slot is held twice")
-        if len(slots) + self.slots.n_free != self.slots.n_slots:
-            raise AssertionError("state slots lost")
+        if self._lib.fxc_check(self._h) != 0:
+            raise AssertionError(self._core.error())
+        if self._lib.fxc_n_requests(self._h) != len(self._handles):
+            raise AssertionError("requests known to the manager and to its core differ")

@@ -1,7 +1,8 @@
-"""Compiles and loads the HIP kernel libraries.
+"""Compiles and loads the native libraries: HIP kernels and the host runtime.
 
 Every `<name>.hip` beside this file becomes one shared object `_lib/<name>.so`,
-built with hipcc for gfx950 and loaded through ctypes.  A library is compiled
+built with hipcc for gfx950 and loaded through ctypes; `host_runtime.cpp` (cache
+book-keeping and step packing, no GPU code) is built with the host compiler.  A library is compiled
 when it is first asked for and no object built from the same sources and flags
 is there (a hash of both is kept beside the object), so a model compiles what
 its parts need and nothing else.  While hipcc runs, a line is printed every few
@@ -24,7 +25,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling")
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
+HOST_LIBRARIES = ("host_runtime",)
+LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling") + HOST_LIBRARIES
 HEADERS = ("common.h",)
 
 _loaded: dict[str, ctypes.CDLL] = {}
@@ -42,10 +45,22 @@ def _hipcc() -> str | None:
     return None
 
 
+def _host_compiler() -> str | None:
+    for cand in (os.environ.get("CXX"), "g++", "c++", "clang++"):
+        path = shutil.which(cand) if cand else None
+        if path:
+            return path
+    return _hipcc()          # hipcc compiles plain C++ for the host as well
+
+
+def _sources(name: str) -> tuple:
+    return (name + ".cpp",) if name in HOST_LIBRARIES else (name + ".hip",) + HEADERS
+
+
 def _source_hash(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
-    for f in (name + ".hip",) + HEADERS:
+    h.update(" ".join(HOST_FLAGS if name in HOST_LIBRARIES else FLAGS).encode())
+    for f in _sources(name):
         with open(os.path.join(HERE, f), "rb") as fh:
             h.update(fh.read())
     return h.hexdigest()
@@ -90,18 +105,19 @@ def compile_library(name: str, verbose: bool = True) -> str:
     """Run hipcc for one library, whatever is already built; returns the path of the object."""
     if name not in LIBRARIES:
         raise KernelBuildError(f"unknown kernel library '{name}'")
-    hipcc = _hipcc()
-    if hipcc is None:
-        raise KernelBuildError(f"kernel library '{name}' is not built and hipcc was not found")
+    host = name in HOST_LIBRARIES
+    compiler = _host_compiler() if host else _hipcc()
+    if compiler is None:
+        raise KernelBuildError(f"library '{name}' is not built and no {'C++ compiler' if host else 'hipcc'} was found")
     out_dir = _writable_dir()
     so = os.path.join(out_dir, name + ".so")
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [hipcc] + FLAGS + [os.path.join(HERE, name + ".hip"), "-o", tmp]
+    cmd = [compiler] + (HOST_FLAGS if host else FLAGS) + [os.path.join(HERE, _sources(name)[0]), "-o", tmp]
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)   # hipcc wants a home for its temporary files
     t0 = time.time()
     if verbose:
-        print(f"[ferrox_amd] compiling kernel library '{name}' for {ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[ferrox_amd] compiling library '{name}' for {'the host' if host else ARCH} ...", file=sys.stderr, flush=True)
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=out_dir)
     result: dict = {}
 
@@ -120,7 +136,7 @@ def compile_library(name: str, verbose: bool = True) -> str:
             os.remove(tmp)
         except OSError:
             pass
-        raise KernelBuildError(f"hipcc failed for '{name}' (exit {proc.returncode}):\n{text}")
+        raise KernelBuildError(f"{os.path.basename(compiler)} failed for '{name}' (exit {proc.returncode}):\n{text}")
     os.replace(tmp, so)
     with open(os.path.join(out_dir, name + ".hash"), "w") as f:
         f.write(_source_hash(name))
@@ -165,6 +181,7 @@ def load_library(name: str) -> ctypes.CDLL:
         if so is None:
             so = compile_library(name)
         lib = ctypes.CDLL(so)
-        lib.fx_last_error.restype = ctypes.c_char_p
+        if name not in HOST_LIBRARIES:
+            lib.fx_last_error.restype = ctypes.c_char_p
         _loaded[name] = lib
         return lib

@@ -42,46 +42,36 @@ class DecodeGraph:
         mgr = runner.manager
         self.max_blocks = max(1, mgr.blocks_for(kv_bound))
         self.keys = list(mgr.groups)
-        total = 3 * n_seqs + len(self.keys) * n_seqs * self.max_blocks
+        total = mgr.step_words(n_seqs, n_seqs, n_seqs, self.max_blocks)
         dev = runner.device
         self.meta = torch.zeros(total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
-        self.arange = torch.arange(n_seqs, dtype=torch.int32, device=dev)
         self.graph = None
         self.logits = None
 
     def _context(self) -> StepContext:
-        n, mb = self.n, self.max_blocks
-        tables, o = {}, 3 * n
+        n, mb, m = self.n, self.max_blocks, self.meta
+        tables, o = {}, 5 * n
         for key in self.keys:
-            tables[key] = self.meta[o:o + n * mb].view(n, mb)
+            tables[key] = m[o:o + n * mb].view(n, mb)
             o += n * mb
         ctx = StepContext(n_tokens=n, n_seqs=n, act_dtype=self.runner.act_dtype, device=self.runner.device,
-                          token_ids=self.meta[0:n], positions=self.meta[n:2 * n], token_seq=self.arange,
-                          q_starts=list(range(n + 1)), kv_lens=[self.kv_bound] * n, slot_ids=self.meta[2 * n:3 * n],
-                          slots=None, block_tables=tables, block_size=self.runner.block_size, logit_rows=self.arange)
+                          token_ids=m[0:n], positions=m[n:2 * n], token_seq=m[2 * n:3 * n],
+                          q_starts=list(range(n + 1)), kv_lens=[self.kv_bound] * n, slot_ids=m[3 * n:4 * n],
+                          slots=None, block_tables=tables, block_size=self.runner.block_size,
+                          logit_rows=m[4 * n:5 * n])
         ctx._memo["attention_items"] = {"n_decode": n, "n_tiles": 0, "max_kv": self.kv_bound,
-                                        "dec_seq": self.arange, "dec_tok": self.arange}
+                                        "dec_seq": m[2 * n:3 * n], "dec_tok": m[4 * n:5 * n]}
         return ctx
 
-    def run(self, tokens, positions, slots, table_rows) -> torch.Tensor:
-        n, mb = self.n, self.max_blocks
+    def run(self, entries) -> torch.Tensor:
         self.copied.synchronize()                  # the last upload has left the staging buffer
-        h = self.host
-        h[0:n] = torch.tensor(tokens, dtype=torch.int32)
-        h[n:2 * n] = torch.tensor(positions, dtype=torch.int32)
-        h[2 * n:3 * n] = torch.tensor(slots, dtype=torch.int32)
-        o = 3 * n
-        for rows in table_rows:                    # one list of rows per group, in the order of self.keys
-            flat = []
-            for r in rows:
-                flat.extend(max(p, 0) for p in r[:mb])
-                flat.extend([0] * (mb - min(len(r), mb)))
-            h[o:o + n * mb] = torch.tensor(flat, dtype=torch.int32)
-            o += n * mb
-        self.meta.copy_(h, non_blocking=True)
+        self.runner.manager.pack_step([e.req for e in entries], [e.tokens for e in entries],
+                                      [e.want for e in entries], self.runner.vocab_size, self.host.data_ptr(),
+                                      self.host.numel(), force_blocks=self.max_blocks)
+        self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
         model, caches = self.runner.model, self.runner.storage.caches
         if self.graph is None:
@@ -102,7 +92,7 @@ class ModelRunner:
             raise RuntimeError("load the model's weights before making a runner")
         if model.device.type != "cuda":
             raise RuntimeError("the engine runs on the GPU only; there is no CPU path")
-        ensure_built(model.kernel_libraries())
+        ensure_built(list(model.kernel_libraries()) + ["host_runtime"])
         self.model = model
         self.act_dtype, self.device = model.act_dtype, model.device
         self.block_size = block_size
@@ -113,6 +103,8 @@ class ModelRunner:
         self.use_graphs = use_graphs and all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
         self.graph_kv_step = graph_kv_step
         self._graphs: dict = {}
+        self._host = None                      # pinned staging buffer of the step's int32 data
+        self._uploaded = torch.cuda.Event()
 
     # ---- requests ----------------------------------------------------------
     def admit(self, req) -> bool:
@@ -130,50 +122,34 @@ class ModelRunner:
         self.manager.release(req)
 
     # ---- the step ----------------------------------------------------------
+    def _staging(self, words: int) -> torch.Tensor:
+        """A pinned host buffer of at least `words` int32 that no upload is still reading."""
+        if self._host is None or self._host.numel() < words:
+            self._host = torch.zeros(max(4096, 2 * words), dtype=torch.int32, pin_memory=True)
+        else:
+            self._uploaded.synchronize()
+        return self._host
+
     def step(self, entries: list) -> torch.Tensor | None:
         """Logits [number of wanted places, vocab] in the order of the entries and of each
         entry's `want`, or None if nothing is wanted.  Every entry's request must hold pages
         for its tokens already (`reserve`)."""
-        mgr, bs = self.manager, self.block_size
-        tokens, positions, token_seq, q_starts, kv_lens, slots, rows = [], [], [], [0], [], [], []
-        for s, e in enumerate(entries):
-            n = len(e.tokens)
-            if n == 0:
-                raise ValueError(f"request {e.req!r} brings no tokens to this step")
-            if e.req not in mgr:
-                raise ValueError(f"request {e.req!r} was not admitted")
-            end = mgr.length(e.req)
-            start = end - n
-            if start < 0:
-                raise ValueError(f"request {e.req!r}: {n} tokens but only {end} positions are reserved")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise ValueError(f"request {e.req!r}: token id {t} is outside the vocabulary "
-                                     f"of {self.vocab_size}")     # ferrox-cli/src/run.rs:598-601
-            for w in e.want:
-                if not 0 <= int(w) < n:
-                    raise ValueError(f"request {e.req!r}: wanted place {w} is outside its {n} tokens")
-                rows.append(len(tokens) + int(w))
-            tokens.extend(int(t) for t in e.tokens)
-            positions.extend(range(start, end))
-            token_seq.extend([s] * n)
-            q_starts.append(len(tokens))
-            kv_lens.append(end)
-            slots.append(mgr.slot(e.req))
-        if len({e.req for e in entries}) != len(entries):
-            raise ValueError("a request appears twice in one step")
-        n_seqs, T = len(entries), len(tokens)
-        if self.use_graphs and T == n_seqs and len(rows) == n_seqs:
+        mgr = self.manager
+        n_seqs = len(entries)
+        reqs = [e.req for e in entries]
+        token_lists, wants = [e.tokens for e in entries], [e.want for e in entries]
+        T, R = sum(len(t) for t in token_lists), sum(len(w) for w in wants)
+        if self.use_graphs and n_seqs and all(len(t) == 1 for t in token_lists) and all(len(w) == 1 for w in wants):
             # every sequence brings one token and wants its logits: a recorded decode step
-            bound = -(-max(kv_lens) // self.graph_kv_step) * self.graph_kv_step
+            longest = max(mgr.length(r) for r in reqs)
+            bound = -(-longest // self.graph_kv_step) * self.graph_kv_step
             key = (n_seqs, bound)
             if key not in self._graphs:
                 if len(self._graphs) >= 16:
                     self._graphs.pop(next(iter(self._graphs)))
                 self._graphs[key] = DecodeGraph(self, n_seqs, bound)
             try:
-                logits = self._graphs[key].run(tokens, positions, slots,
-                                               [[mgr.table(e.req, k) for e in entries] for k in mgr.groups])
+                logits = self._graphs[key].run(entries)
             except RuntimeError as err:
                 # recording is an optimisation of how kernels are launched, not another code path:
                 # if the runtime refuses it, the same kernels are launched one by one from here on
@@ -183,18 +159,16 @@ class ModelRunner:
                 self._graphs.clear()
                 logits = None
             if logits is not None:
-                for e in entries:
-                    mgr.trim(e.req)
+                for r in reqs:
+                    mgr.trim(r)
                 return logits
-        max_blocks = max(1, max(mgr.blocks_for(L) for L in kv_lens))
-        tables = {}
-        flat = tokens + positions + token_seq + slots + rows
-        for key in mgr.groups:
-            for e in entries:
-                t = mgr.table(e.req, key)
-                flat.extend(max(p, 0) for p in t[:max_blocks])
-                flat.extend([0] * (max_blocks - min(len(t), max_blocks)))
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
+        longest = max((mgr.length(r) for r in reqs if r in mgr), default=0)
+        max_blocks = max(1, mgr.blocks_for(longest))
+        host = self._staging(mgr.step_words(T, n_seqs, R, max_blocks))
+        packed = mgr.pack_step(reqs, token_lists, wants, self.vocab_size, host.data_ptr(), host.numel())
+        dev = torch.empty(packed.total, dtype=torch.int32, device=self.device)
+        dev.copy_(host[:packed.total], non_blocking=True)
+        self._uploaded.record()
         o = 0
 
         def take(n):
@@ -203,14 +177,17 @@ class ModelRunner:
             o += n
             return v
 
-        d_tokens, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(n_seqs), take(len(rows))
-        for key in mgr.groups:
-            tables[key] = take(n_seqs * max_blocks).view(n_seqs, max_blocks)
+        mb = packed.max_blocks
+        d_tokens, d_pos, d_seq, d_slots, d_rows = take(T), take(T), take(T), take(n_seqs), take(R)
+        tables = {key: take(n_seqs * mb).view(n_seqs, mb) for key in mgr.groups}
+        q_starts = [0]
+        for t in token_lists:
+            q_starts.append(q_starts[-1] + len(t))
         ctx = StepContext(n_tokens=T, n_seqs=n_seqs, act_dtype=self.act_dtype, device=self.device,
                           token_ids=d_tokens, positions=d_pos, token_seq=d_seq, q_starts=q_starts,
-                          kv_lens=kv_lens, slot_ids=d_slots, slots=slots, block_tables=tables,
-                          block_size=bs, logit_rows=d_rows if rows else None)
+                          kv_lens=packed.lens, slot_ids=d_slots, slots=host[3 * T:3 * T + n_seqs].tolist(),
+                          block_tables=tables, block_size=self.block_size, logit_rows=d_rows if R else None)
         logits = self.model.forward(ctx, self.storage.caches)
-        for e in entries:
-            mgr.trim(e.req)
+        for r in reqs:
+            mgr.trim(r)
         return logits

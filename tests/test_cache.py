@@ -116,3 +116,57 @@ def test_random_orders_keep_the_invariants(seed):
         m.release(rid)
     m.check_invariants()
     assert all(g.pool.n_free == g.pool.num_pages for g in m.groups.values()) and m.slots.n_free == 4
+
+
+def _pack(m, reqs, toks, wants, vocab=100, force=0, cap=4096):
+    import numpy as np
+    buf = np.full(cap, -7, dtype=np.int32)
+    p = m.pack_step(reqs, toks, wants, vocab, buf.ctypes.data, cap, force_blocks=force)
+    return p, buf
+
+
+def test_pack_step_layout():
+    m = CacheManager({FULL: None, WIN: 16}, 16, block_size=8, n_slots=4)
+    for r, n in (("a", 21), ("b", 40)):
+        m.admit(r)
+        m.extend(r, n)
+    m.trim("b")                                                    # b's first windowed blocks are given back
+    p, buf = _pack(m, ["b", "a"], [[7], [1, 2, 3]], [[0], [0, 2]])
+    T, n, R, mb = 4, 2, 3, 5
+    assert (p.n_tokens, p.n_rows, p.max_blocks, p.total) == (T, R, mb, 3 * T + n + R + 2 * n * mb)
+    assert p.starts == [39, 18] and p.lens == [40, 21]
+    assert buf[:T].tolist() == [7, 1, 2, 3]
+    assert buf[T:2 * T].tolist() == [39, 18, 19, 20]               # positions go on where the cache ends
+    assert buf[2 * T:3 * T].tolist() == [0, 1, 1, 1]
+    assert buf[3 * T:3 * T + n].tolist() == [m.slot("b"), m.slot("a")]
+    assert buf[3 * T + n:3 * T + n + R].tolist() == [0, 1, 3]      # rows of the flat batch
+    o = 3 * T + n + R
+    full_b, full_a = m.table("b", FULL), m.table("a", FULL)
+    assert buf[o:o + mb].tolist() == full_b and buf[o + mb:o + 2 * mb].tolist() == full_a + [0, 0]
+    win_b = [max(x, 0) for x in m.table("b", WIN)]                 # freed entries are written as 0, never read
+    assert buf[o + 2 * mb:o + 3 * mb].tolist() == win_b and m.table("b", WIN)[:3] == [-1, -1, -1]
+    assert buf[p.total] == -7                                      # nothing written past the end
+    p2, buf2 = _pack(m, ["b", "a"], [[7], [1, 2, 3]], [[0], [0, 2]], force=9)
+    assert p2.max_blocks == 9 and buf2[o:o + 9].tolist() == full_b + [0] * 4
+
+
+def test_pack_step_refuses_what_does_not_fit():
+    m = CacheManager({FULL: None}, 8, block_size=8, n_slots=4)
+    m.admit("a")
+    m.extend("a", 3)
+    for reqs, toks, wants, word in (
+            (["zz"], [[1]], [[0]], "not admitted"),
+            (["a"], [[]], [[]], "no tokens"),
+            (["a"], [[1, 2, 3, 4]], [[]], "reserved"),
+            (["a"], [[1, 100]], [[]], "vocabulary"),
+            (["a"], [[1, -1]], [[]], "vocabulary"),
+            (["a"], [[1, 2]], [[2]], "wanted place"),
+            (["a", "a"], [[1], [2]], [[], []], "twice")):
+        with pytest.raises(ValueError, match=word):
+            _pack(m, reqs, toks, wants)
+    with pytest.raises(ValueError, match="too small"):
+        _pack(m, ["a"], [[1, 2]], [[1]], cap=4)
+    with pytest.raises(ValueError, match="cannot hold"):
+        m.extend("a", 20)
+        _pack(m, ["a"], [[1, 2]], [[1]], force=2)
+    m.check_invariants()
