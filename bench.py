@@ -173,6 +173,7 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode runs")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling); prints its own line")
     ap.add_argument("--no-graphs", action="store_true", help="launch every decode kernel from the host instead of replaying a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -180,11 +181,17 @@ def main() -> int:
         return 2
 
     new_tokens = args.steps + args.warmup + 2
-    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
     b = Bench(args.layers, args.dtype, args.block_size, max_batch, args.ctx, max(new_tokens, 64))
     c = b.cfg
     if args.no_graphs:
         b.runner.use_graphs = False
+
+    if args.only_prefill:
+        t = b.prefill(2048, reps=max(1, args.steps))
+        print(json.dumps({"prefill_tokens": 2048, "ms": round(t * 1e3, 3), "tokens_per_s": round(2048 / t, 1),
+                          "frac": round(b.prefill_flops(2048) / t / PEAK_FLOPS[args.dtype], 4)}), flush=True)
+        return 0
 
     dt, distinct = b.decode(args.batch, args.ctx, args.steps, args.warmup)
     tok_s = args.batch / dt

@@ -107,4 +107,39 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// ---- results that blocks of one launch hand to each other ----------------------
+// The eight XCDs have an L2 each, so a plain store of one block need not be seen by a block on
+// another XCD before the kernel ends.  Values that the launch's last block gathers are therefore
+// written and read at device scope (they go past the caches that are not shared), which costs
+// nothing like a fence: a fence would write a whole L2 back.
+__device__ __forceinline__ void store_shared(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_shared(int* p, int v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int load_shared(const int* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// True, in every thread, in the block that is the last of `total` blocks to get here.  What the
+// other blocks wrote with store_shared() before they came can be read there with load_shared().
+// The last block leaves the counter (one zeroed word in device memory) at zero again.  Every
+// thread of a block must call it.
+__device__ __forceinline__ bool last_block_arrives(unsigned* counter, unsigned total) {
+    __shared__ int fx_last_flag;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's stores have arrived
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        fx_last_flag = (old == total - 1u);
+        if (old == total - 1u) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    return fx_last_flag != 0;
+}
+
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

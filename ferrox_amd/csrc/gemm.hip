@@ -35,12 +35,18 @@ struct GemmArgs {
     const int* expert_offsets;  // [E+1] or null
     int E;
     int M, N, K;
+    const void* norm_w;  // skinny bf16 kernel only: A is the float32 residual stream and RMSNorm with these weights
+    int norm_dtype;      //   is applied on the way in; norm_w is [K]
+    float norm_eps;
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
 
 // block -> (first logical row, end of rows, expert).  Plain: tiles of TM rows.
-// Grouped: walk the experts' tile counts; blocks past the last tile get r0 = -1.
+// Grouped: expert e has ceil(rows_e / TM) tiles, in the order of the experts; a tile past the
+// last one gets r0 = -1.  Every wave finds its tile by itself, 64 experts at a time: each lane
+// takes one expert's bounds, a scan over the lanes gives the tiles before it, and the lane whose
+// range holds the tile tells the others.  (One load's latency instead of one per expert.)
 template <int TM>
 __device__ __forceinline__ void locate_rows(const GemmArgs& g, int tile, int& r0, int& r_end, int& expert) {
     if (!g.expert_offsets) {
@@ -50,20 +56,31 @@ __device__ __forceinline__ void locate_rows(const GemmArgs& g, int tile, int& r0
         if (r0 >= g.M) r0 = -1;
         return;
     }
-    int acc = 0;
+    const int lane = threadIdx.x & 63;
+    int before = 0;
     r0 = -1;
     r_end = 0;
     expert = 0;
-    for (int e = 0; e < g.E; ++e) {
-        const int b = g.expert_offsets[e], en = g.expert_offsets[e + 1];
+    for (int base = 0; base < g.E; base += 64) {
+        const int e = base + lane;
+        const int b = e < g.E ? g.expert_offsets[e] : 0, en = e < g.E ? g.expert_offsets[e + 1] : 0;
         const int nt = (en - b + TM - 1) / TM;
-        if (tile < acc + nt) {
-            r0 = b + (tile - acc) * TM;
-            r_end = en;
-            expert = e;
+        int incl = nt;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int u = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += u;
+        }
+        const int first = before + incl - nt;
+        const unsigned long long hit = __ballot(tile >= first && tile < first + nt);
+        if (hit) {
+            const int src = __ffsll((long long)hit) - 1;
+            r0 = __shfl(b + (tile - first) * TM, src, 64);
+            r_end = __shfl(en, src, 64);
+            expert = base + src;
             return;
         }
-        acc += nt;
+        before += __shfl(incl, 63, 64);
     }
 }
 
@@ -252,9 +269,27 @@ __device__ __forceinline__ uint4 load16(const bf16* row, int k, int K) {
     return (row && k < K) ? *(const uint4*)(row + k) : make_uint4(0, 0, 0, 0);
 }
 
-template <int MT, int WAVES, int NW, bool DUAL, int EPI>   // NW: sets of 16 weight rows per wave (dual: gate and up)
+// NORM: the rows of A are float32 and are normed on the way in, y = x * rsqrt(mean(x^2) + eps) * w
+// (ferrox-core/src/matmul.rs:62-69): x * w is rounded to bfloat16 and multiplied, the sums of
+// squares that the waves gather over their parts of K are added up, and the product is scaled by
+// the row's rsqrt before the bias is added.
+__device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+    if (ok) {
+        a = *(const float4*)p;
+        b = *(const float4*)(p + 4);
+    }
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false>   // NW: sets of 16 weight rows per wave (dual: gate and up)
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
     static_assert(!DUAL || NW == 2, "dual mode multiplies two matrices");
+    static_assert(!NORM || (!DUAL && EPI == EPI_STORE), "the fused norm feeds a plain product");
+    __shared__ float red_ss[NORM ? WAVES : 1][MT][64];
+    float ss[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) ss[mt] = 0.f;
     constexpr int NACC = MT * NW;
     constexpr int COLS = DUAL ? 16 : 16 * NW;   // output columns of a block
     __shared__ f32x4_t red[WAVES][NACC][64];
@@ -271,11 +306,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         const int n = DUAL ? n0 + li : n0 + a * 16 + li;
         wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + ((DUAL && a) ? g.up_offset : 0) : nullptr;
     }
-    const bf16* xrow[MT];
+    const bf16* xrow[MT];       // NORM: float rows, kept under the same name
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = r0 + mt * 16 + li;
-        xrow[mt] = (m < r_end) ? (const bf16*)g.A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : nullptr;
+        const size_t off = (m < r_end) ? (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : 0;
+        xrow[mt] = (m < r_end) ? (NORM ? (const bf16*)((const float*)g.A + off) : (const bf16*)g.A + off) : nullptr;
     }
     f32x4_t acc[MT][NW];
 #pragma unroll
@@ -286,7 +322,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     const int n_super = (g.K + 127) / 128;
     const int per = (n_super + WAVES - 1) / WAVES;
     const int s_end = min(n_super, (wave + 1) * per);
-    constexpr int UN = (MT * NW <= 4) ? 2 : 1;     // pieces whose loads are issued together
+    constexpr int UN = (MT * NW <= 4 && !NORM) ? 2 : 1;     // pieces whose loads are issued together
     for (int s = wave * per; s < s_end; s += UN) {
         uint4 w[UN][NW][4], x[UN][MT][4];
 #pragma unroll
@@ -297,8 +333,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             for (int u = 0; u < 4; ++u) {
 #pragma unroll
                 for (int a = 0; a < NW; ++a) w[p][a][u] = load16(live ? wrow[a] : nullptr, kb + 32 * u, g.K);
+                if constexpr (NORM) {
+                    const int k = kb + 32 * u;
+                    const bool kin = live && k < g.K;
+                    float gv[8];
+                    if (g.norm_dtype == FX_F32) {
+                        load8f((const float*)g.norm_w + k, kin, gv);
+                    } else {
+                        const uint4 gw = kin ? *(const uint4*)((const bf16*)g.norm_w + k) : make_uint4(0, 0, 0, 0);
+                        gv[0] = __uint_as_float(gw.x << 16); gv[1] = __uint_as_float(gw.x & 0xffff0000u);
+                        gv[2] = __uint_as_float(gw.y << 16); gv[3] = __uint_as_float(gw.y & 0xffff0000u);
+                        gv[4] = __uint_as_float(gw.z << 16); gv[5] = __uint_as_float(gw.z & 0xffff0000u);
+                        gv[6] = __uint_as_float(gw.w << 16); gv[7] = __uint_as_float(gw.w & 0xffff0000u);
+                    }
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 32 * u, g.K);
+                    for (int mt = 0; mt < MT; ++mt) {
+                        float xv[8];
+                        load8f((const float*)xrow[mt] + k, kin && xrow[mt], xv);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) ss[mt] += xv[i] * xv[i];
+                        x[p][mt][u] = make_uint4(pack_bf16(xv[0] * gv[0], xv[1] * gv[1]), pack_bf16(xv[2] * gv[2], xv[3] * gv[3]),
+                                                 pack_bf16(xv[4] * gv[4], xv[5] * gv[5]), pack_bf16(xv[6] * gv[6], xv[7] * gv[7]));
+                    }
+                } else {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 32 * u, g.K);
+                }
             }
         }
 #pragma unroll
@@ -318,6 +378,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int a = 0; a < NW; ++a) red[wave][mt * NW + a][lane] = acc[mt][a];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) red_ss[wave][mt][lane] = ss[mt];
+    }
     __syncthreads();
     constexpr int OUTS = DUAL ? MT : MT * NW;     // accumulator tiles that become output tiles
     for (int idx = tid; idx < OUTS * 64; idx += WAVES * 64) {
@@ -332,11 +396,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         const int ml = r0 + mt * 16 + (L & 15);
         if (ml >= r_end) continue;
         const int m = g.c_rows ? g.c_rows[ml] : ml;
+        float rstd = 1.f;
+        if constexpr (NORM) {
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) total += red_ss[w][mt][(L & 15) + 16 * q];
+            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n0 + a * 16 + (L >> 4) * 4 + r;
             if (n >= g.N) continue;
-            float o = v[r];
+            float o = v[r] * rstd;
             if (DUAL) {
                 from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(o) * v2[r]);
                 continue;
@@ -470,6 +543,10 @@ template <int MT, int WAVES, int NW>
 static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
     dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 16 : 16 * NW), m_tiles);
     if constexpr (MT * NW * WAVES <= 32) {       // the partial sums of all waves fit in LDS
+        if (g.norm_w) {
+            gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE, true><<<grid, WAVES * 64, 0, s>>>(g);
+            return;
+        }
         switch (epi) {
             case EPI_STORE: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE><<<grid, WAVES * 64, 0, s>>>(g); break;
             case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
@@ -501,7 +578,7 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int nw
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
-                   int E, int M, int N, int K) {
+                   int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -510,7 +587,15 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     FX_REQUIRE(!expert_offsets || E > 0, "gemm: grouped mode needs E > 0");
     FX_REQUIRE(!bias || bias_dtype == FX_F32 || bias_dtype == FX_BF16, "gemm: unknown bias dtype %d", bias_dtype);
     if (M == 0) return 0;
+    if (norm_w) {
+        FX_REQUIRE(dtype == FX_BF16 && epi == EPI_STORE, "gemm: the fused norm feeds a bfloat16 product that is stored");
+        FX_REQUIRE(norm_dtype == FX_F32 || norm_dtype == FX_BF16, "gemm: unknown norm weight dtype %d", norm_dtype);
+        FX_REQUIRE((expert_offsets ? (M + E - 1) / E : M) <= 32 && K % 8 == 0 && lda % 4 == 0 && w_stride % 8 == 0 &&
+                       (((uintptr_t)A | (uintptr_t)W | (uintptr_t)norm_w) % 16 == 0),
+                   "gemm: the fused norm takes up to 32 rows per group, K a multiple of 8 and 16-byte aligned rows");
+    }
     GemmArgs g;
+    g.norm_w = norm_w; g.norm_dtype = norm_dtype; g.norm_eps = norm_eps;
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
@@ -529,8 +614,9 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         FX_CHECK_LAUNCH("gemm_f32");
         return 0;
     }
-    g.vec_ok = (K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
-               (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+    g.vec_ok = norm_w != nullptr ||
+               ((K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
+                (((uintptr_t)A | (uintptr_t)W) % 16 == 0));
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
     if (g.vec_ok && per_group <= 64) {
         const int mt = per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4);

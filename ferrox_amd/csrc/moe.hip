@@ -201,6 +201,137 @@ __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* 
     align_block(ids_s, T * k, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
 }
 
+// ---------------------------------------------------------------------------
+// Few tokens (decode): everything in front of the experts in one launch.
+// Block (r, t): RMSNorm of row t of the float32 residual stream (same formula and
+// rounding as rmsnorm_kernel; block r = 0 writes it out as bfloat16 for the
+// experts), then the products of that rounded row with router rows 8r .. 8r+7,
+// two rows per wave, k in a fixed order, into `logits`.  The block that finishes
+// last selects the experts of every token (a wave per token) and sorts the pairs.
+// ---------------------------------------------------------------------------
+#define FRONT_THREADS 256
+#define FRONT_WAVES (FRONT_THREADS / 64)
+#define FRONT_ROWS (2 * FRONT_WAVES)   // router rows per block
+
+__device__ __forceinline__ float dot8(uint4 w, const float* x) {
+    float a = 0.f;
+    a = fmaf(__uint_as_float(w.x << 16), x[0], a);
+    a = fmaf(__uint_as_float(w.x & 0xffff0000u), x[1], a);
+    a = fmaf(__uint_as_float(w.y << 16), x[2], a);
+    a = fmaf(__uint_as_float(w.y & 0xffff0000u), x[3], a);
+    a = fmaf(__uint_as_float(w.z << 16), x[4], a);
+    a = fmaf(__uint_as_float(w.z & 0xffff0000u), x[5], a);
+    a = fmaf(__uint_as_float(w.w << 16), x[6], a);
+    a = fmaf(__uint_as_float(w.w & 0xffff0000u), x[7], a);
+    return a;
+}
+
+__global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
+    const float* __restrict__ h, long ldh, const void* __restrict__ gamma, int gamma_dtype, float eps,
+    bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm,
+    int gating, float* logits, int* ids, float* __restrict__ weights, float* __restrict__ gate_out,
+    int* __restrict__ expert_offsets, int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
+    int* __restrict__ inv, unsigned* counter) {
+    extern __shared__ int lds[];
+    __shared__ float red[FRONT_WAVES];
+    float* xs = (float*)lds;            // H: the normed row as the experts will read it
+    const int t = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_rows = E + has_gate, chunks = H >> 3;
+
+    // this wave's two router rows: their first loads leave before the norm is done
+    const int e_a = blockIdx.x * FRONT_ROWS + wave, e_b = e_a + FRONT_WAVES;
+    const bf16* wa = e_a < n_rows ? W + (size_t)e_a * H : nullptr;
+    const bf16* wb = e_b < n_rows ? W + (size_t)e_b * H : nullptr;
+    uint4 pa = make_uint4(0, 0, 0, 0), pb = pa;
+    if (lane < chunks) {
+        if (wa) pa = *(const uint4*)(wa + lane * 8);
+        if (wb) pb = *(const uint4*)(wb + lane * 8);
+    }
+
+    const float* row = h + (size_t)t * ldh;
+    float ss = 0.f;
+    for (int c = tid; c < H; c += FRONT_THREADS) {
+        const float v = row[c];
+        xs[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum<FRONT_WAVES>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = tid; c < H; c += FRONT_THREADS) {
+        const bf16 b = float_to_bf16(xs[c] * scale * load_as_float(gamma, gamma_dtype, c));
+        if (blockIdx.x == 0) x_out[(size_t)t * H + c] = b;
+        xs[c] = bf16_to_float(b);
+    }
+    __syncthreads();
+
+    float acc_a = 0.f, acc_b = 0.f;
+    for (int c = lane; c < chunks; c += 64) {
+        const int cn = c + 64;
+        uint4 na = make_uint4(0, 0, 0, 0), nb = na;
+        if (cn < chunks) {
+            if (wa) na = *(const uint4*)(wa + cn * 8);
+            if (wb) nb = *(const uint4*)(wb + cn * 8);
+        }
+        acc_a += dot8(pa, xs + c * 8);
+        acc_b += dot8(pb, xs + c * 8);
+        pa = na;
+        pb = nb;
+    }
+    acc_a = wave_sum(acc_a);
+    acc_b = wave_sum(acc_b);
+    if (lane == 0) {
+        if (wa) store_shared(logits + (size_t)t * n_rows + e_a, acc_a);
+        if (wb) store_shared(logits + (size_t)t * n_rows + e_b, acc_b);
+    }
+
+    if (!last_block_arrives(counter, gridDim.x * gridDim.y)) return;
+    const int n = T * k;
+    float* score = (float*)lds;                     // FRONT_WAVES x E
+    float* lrow = score + FRONT_WAVES * E;          // FRONT_WAVES x n_rows: a token's logits
+    int* ids_s = (int*)(lrow + FRONT_WAVES * n_rows);   // n
+    int* offs = ids_s + n;                          // E + 1
+    uint16_t* cnt = (uint16_t*)(offs + E + 1);      // rows x E
+    for (int tt = wave; tt < T; tt += FRONT_WAVES) {
+        float* mine = lrow + wave * n_rows;
+        for (int e = lane; e < n_rows; e += 64) mine[e] = load_shared(logits + (size_t)tt * n_rows + e);
+        __builtin_amdgcn_wave_barrier();
+        select_token(mine, score + wave * E, tt, E, k, renorm, gating, ids, weights, has_gate ? gate_out : nullptr, ids_s);
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    align_block(ids_s, n, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
+}
+
+// Returns 2 (and launches nothing) for sizes this kernel does not take; the caller then runs the
+// norm, the router product and the two routing kernels one after the other.  `logits` holds
+// T x (E + has_gate) floats; `counter` is one zeroed unsigned in device memory that launches on
+// one stream may share.
+FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamma, int gamma_dtype, float eps,
+                        void* x_out, const void* W, int H, int T, int E, int has_gate, int k, int renorm, int gating,
+                        float* logits, int* ids, float* weights, float* gate_out, int* expert_offsets,
+                        int* sorted_token, int* sorted_pair, int* inv, unsigned* counter) {
+    FX_REQUIRE(T >= 0 && H > 0, "moe_front: bad sizes T=%d H=%d", T, H);
+    FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
+    FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
+    FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
+    FX_REQUIRE(gamma_dtype == FX_F32 || gamma_dtype == FX_BF16, "moe_front: unknown norm weight dtype %d", gamma_dtype);
+    FX_REQUIRE(ldh >= H, "moe_front: rows of %ld hold fewer than %d columns", ldh, H);
+    FX_REQUIRE(!has_gate || gate_out, "moe_front: a gate row needs a place for its output");
+    const long n = (long)T * k;
+    const long rows = n < FRONT_THREADS ? n : FRONT_THREADS;
+    const size_t front = (size_t)H * 4;
+    const size_t back = (size_t)(FRONT_WAVES * (2 * E + 1) + n + E + 1) * 4 + (size_t)rows * E * 2;
+    const size_t shm = front > back ? front : back;
+    if (T > 16 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
+    if (T == 0) return 0;
+    dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
+    moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(
+        h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out, (const bf16*)W, H, T, E, has_gate, k, renorm, gating, logits, ids,
+        weights, gate_out, expert_offsets, sorted_token, sorted_pair, inv, counter);
+    FX_CHECK_LAUNCH("moe_front");
+    return 0;
+}
+
 FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
                         int* sorted_token, int* sorted_pair, int* inv) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);

@@ -227,6 +227,7 @@ __global__ __launch_bounds__(SB) void sample_kernel(SampleArgs a) {
     float* s = a.work + (size_t)r * V;
     const float temp = a.temperature ? a.temperature[r] : 0.f;
 
+    #pragma unroll 4
     for (int i = threadIdx.x; i < V; i += SB) s[i] = logits[i];
     __syncthreads();
 
@@ -271,6 +272,7 @@ __global__ __launch_bounds__(SB) void sample_kernel(SampleArgs a) {
 
     // softmax(scores / temperature)
     float mx = -INFINITY;
+    #pragma unroll 4
     for (int i = threadIdx.x; i < V; i += SB) {
         const float v = s[i] / temp;
         s[i] = v;
@@ -283,12 +285,14 @@ __global__ __launch_bounds__(SB) void sample_kernel(SampleArgs a) {
     mx = red_f[0];
     for (int w = 1; w < SW; ++w) mx = fmaxf(mx, red_f[w]);
     float sum = 0.f;
+    #pragma unroll 4
     for (int i = threadIdx.x; i < V; i += SB) {
         const float e = expf(s[i] - mx);
         s[i] = e;
         sum += e;
     }
     sum = block_sum_f(sum, red_f);
+    #pragma unroll 4
     for (int i = threadIdx.x; i < V; i += SB) s[i] = s[i] / sum;
     __syncthreads();
 
@@ -331,6 +335,66 @@ __global__ __launch_bounds__(SB) void sample_kernel(SampleArgs a) {
     __syncthreads();
     // if rounding left the draw above the last sum, the last token with p > 0 is taken
     if (threadIdx.x == 0) a.out[r] = found != 0x7fffffff ? found : max(last_pos, 0);
+}
+
+// Greedy choice without history penalties, many blocks per row: block (b, r) finds the best of
+// its slice of row r (lowest index on ties, NaN never wins) and leaves it in `part`; the row's
+// last block to finish picks among the slices.
+#define GREEDY_THREADS 256
+__global__ __launch_bounds__(GREEDY_THREADS) void greedy_kernel(const float* __restrict__ logits, long ldl, int V,
+                                                                int per_block, ArgBest* part, unsigned* counters,
+                                                                int* __restrict__ out) {
+    __shared__ ArgBest red[GREEDY_THREADS / 64];
+    const int r = blockIdx.y, nb = gridDim.x;
+    const float* row = logits + (size_t)r * ldl;
+    const int b0 = blockIdx.x * per_block, b1 = min(V, b0 + per_block);
+    ArgBest best = {-INFINITY, 0x7fffffff};
+#pragma unroll 4
+    for (int i = b0 + threadIdx.x; i < b1; i += GREEDY_THREADS) {
+        const float v = row[i];
+        if (v > best.v) best = {v, i};       // ascending i within a thread: the first maximum is kept
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgBest other = {__shfl_xor(best.v, o, 64), __shfl_xor(best.i, o, 64)};
+        best = better(best, other);
+    }
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < GREEDY_THREADS / 64; ++w) best = better(best, red[w]);
+        store_shared(&part[(size_t)r * nb + blockIdx.x].v, best.v);
+        store_shared(&part[(size_t)r * nb + blockIdx.x].i, best.i);
+    }
+    if (!last_block_arrives(counters + r, nb)) return;
+    if (threadIdx.x < 64) {
+        ArgBest b = {-INFINITY, 0x7fffffff};
+        for (int i = threadIdx.x; i < nb; i += 64) {
+            const ArgBest other = {load_shared(&part[(size_t)r * nb + i].v), load_shared(&part[(size_t)r * nb + i].i)};
+            b = better(b, other);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            ArgBest other = {__shfl_xor(b.v, o, 64), __shfl_xor(b.i, o, 64)};
+            b = better(b, other);
+        }
+        if (threadIdx.x == 0) out[r] = b.i == 0x7fffffff ? 0 : b.i;
+    }
+}
+
+// part: R * 64 pairs (float, int); counters: R zeroed unsigned that the kernel leaves at zero
+FX_API int fx_sample_greedy(void* stream, const float* logits, long ldl, int R, int V, void* part, unsigned* counters,
+                            int* out) {
+    FX_REQUIRE(R >= 0 && V > 0 && ldl >= V, "sample: bad sizes R=%d V=%d ldl=%ld", R, V, ldl);
+    FX_REQUIRE(part && counters && out, "sample: scratch, counters and output are required");
+    if (R == 0) return 0;
+    int nb = ceil_div(V, 4 * GREEDY_THREADS);       // at least four elements per thread
+    if (nb > 64) nb = 64;
+    const int per_block = ceil_div(V, nb);
+    greedy_kernel<<<dim3(nb, R), GREEDY_THREADS, 0, (hipStream_t)stream>>>(logits, ldl, V, per_block, (ArgBest*)part,
+                                                                          counters, out);
+    FX_CHECK_LAUNCH("sample_greedy");
+    return 0;
 }
 
 FX_API int fx_sample(void* stream, const float* logits, long ldl, float* work, int R, int V,

@@ -55,7 +55,8 @@ _sigs = {
                                         c_int, c_int, c_int],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
-                          c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
+                          c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_void_p, c_int, c_float],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -67,7 +68,10 @@ _sigs = {
                                   c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
+                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 9,
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
 _fns: dict = {}
@@ -184,7 +188,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          bias: torch.Tensor | None = None, row_scale: torch.Tensor | None = None,
          a_rows: torch.Tensor | None = None, c_rows: torch.Tensor | None = None,
          expert_offsets: torch.Tensor | None = None,
-         n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0) -> torch.Tensor:
+         n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
+         norm: tuple | None = None) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -193,8 +198,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores silu(gate)*up.
     `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.  `c_rows`
     scatters the rows of the output (row_scale stays indexed by the logical row).
+    `norm` = (weight [K], eps): `a` is the float32 residual stream and RMSNorm is applied on the way
+    in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     """
-    if a.dtype != w.dtype:
+    if norm is not None:
+        if a.dtype != torch.float32 or w.dtype != torch.bfloat16 or epilogue != EPI_STORE:
+            raise KernelError("gemm: the fused norm reads float32 rows for a stored bfloat16 product")
+        if norm[0].numel() != a.shape[1] or not norm[0].is_contiguous():
+            raise KernelError("gemm: the norm's weight does not fit the rows")
+    elif a.dtype != w.dtype:
         raise KernelError(f"gemm: activations are {a.dtype}, weights {w.dtype}")
     if a.dim() != 2 or a.stride(1) != 1:
         raise KernelError("gemm: activations must be 2-D with unit inner stride")
@@ -222,7 +234,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
             raise KernelError("gemm: gate/up rows exceed the weight matrix")
     else:
         N = n_out if n_out is not None else n_w
-    out_dtype = a.dtype if epilogue in (EPI_STORE, EPI_SILU_MUL) else torch.float32
+    out_dtype = w.dtype if epilogue in (EPI_STORE, EPI_SILU_MUL) else torch.float32
     if out is None:
         if epilogue == EPI_RESID:
             raise KernelError("gemm: the residual epilogue needs `out`")
@@ -231,11 +243,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
         raise KernelError(f"gemm: output {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {out_dtype}")
     if bias is not None and bias.numel() != N:
         raise KernelError(f"gemm: bias has {bias.numel()} elements for {N} columns")
-    _call("gemm", "fx_gemm", _stream(), dtype_code(a.dtype), epilogue, _p(a), a.stride(0), _p(w), w_stride, up_offset,
+    _call("gemm", "fx_gemm", _stream(), dtype_code(w.dtype), epilogue, _p(a), a.stride(0), _p(w), w_stride, up_offset,
           _p(bias), dtype_code(bias.dtype) if bias is not None else 0, _p(out), out.stride(0),
           _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
-          _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K)
+          _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K,
+          _p(norm[0]) if norm is not None else None, dtype_code(norm[0].dtype) if norm is not None else 0,
+          float(norm[1]) if norm is not None else 0.0)
     return out
+
+
+def can_fuse_norm(h: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:
+    """Whether gemm(h, w, norm=...) takes these operands: few rows, bfloat16 weights, aligned rows."""
+    return (h.dtype == torch.float32 and w.dtype == torch.bfloat16 and w.dim() == 2 and n_rows <= 32
+            and h.shape[1] % 8 == 0 and h.stride(0) % 4 == 0 and h.stride(1) == 1
+            and h.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
@@ -312,6 +333,52 @@ def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False)
     return (ids, weights, gate) + moe_align(ids, n_experts)
 
 
+_counters: dict = {}
+
+
+def _counter(device, n: int = 1) -> torch.Tensor:
+    """At least n zeroed words for kernels whose last block finishes the work; a kernel leaves its
+    words at zero, so launches that follow each other on a stream share them.  Buffers are never
+    freed: a recorded graph may hold their address."""
+    key = torch.device(device)
+    if key.index is None:
+        key = torch.device(key.type, torch.cuda.current_device())
+    held = _counters.setdefault(key, [])
+    if not held or held[-1].numel() < n:
+        held.append(torch.zeros(max(1024, 2 * n), dtype=torch.int32, device=key))
+    return held[-1]
+
+
+def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+    """For up to 16 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
+    products, selection and the sort by expert.  Returns None for sizes the kernel does not take, else
+    (x, ids, weights, gate, expert_offsets, sorted_token, sorted_pair, inv)."""
+    T, H = h.shape
+    if (T > 16 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
+            or not router.is_contiguous() or router.shape != (n_experts + (1 if has_gate else 0), H)
+            or norm_weight.numel() != H):
+        return None
+    dev = h.device
+    n = T * top_k
+    x = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+    weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
+    gate = torch.empty((T,), dtype=torch.float32, device=dev) if has_gate else None
+    offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
+    buf = torch.empty((3, n), dtype=torch.int32, device=dev)
+    logits = torch.empty((T, router.shape[0]), dtype=torch.float32, device=dev)
+    f, handle = _fn("moe", "fx_moe_front")
+    rc = f(_stream(), _p(h), h.stride(0), _p(norm_weight), dtype_code(norm_weight.dtype), float(eps), _p(x), _p(router),
+           H, T, n_experts, 1 if has_gate else 0, top_k, 1 if renorm else 0, gating, _p(logits), _p(ids), _p(weights),
+           _p(gate),
+           _p(offsets), _p(buf[0]), _p(buf[1]), _p(buf[2]), _p(_counter(dev)))
+    if rc == 2:
+        return None
+    if rc:
+        raise KernelError(handle.fx_last_error().decode())
+    return x, ids, weights, gate, offsets, buf[0], buf[1], buf[2]
+
+
 def moe_align(ids: torch.Tensor, n_experts: int):
     """For ids [T, k]: (expert_offsets [E+1], sorted_token [n], sorted_pair [n], inv [n]): sorted row i
     belongs to pair sorted_pair[i] = t*k + j of token sorted_token[i]; inv is the inverse map."""
@@ -332,8 +399,13 @@ def sample(logits: torch.Tensor, *, temperature=None, draw=None, top_k=None, top
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("sample: logits must be float32 [R, V] with unit inner stride")
     R, V = logits.shape
-    work = torch.empty((R, V), dtype=torch.float32, device=logits.device)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    if temperature is None and hist is None:      # plain greedy: many blocks per row
+        part = torch.empty((R, 64, 2), dtype=torch.int32, device=logits.device)
+        _call("sampling", "fx_sample_greedy", _stream(), _p(logits), logits.stride(0), R, V, _p(part),
+              _p(_counter(logits.device, R)), _p(out))
+        return out
+    work = torch.empty((R, V), dtype=torch.float32, device=logits.device)
     _call("sampling", "fx_sample", _stream(), _p(logits), logits.stride(0), _p(work), R, V,
           _p(temperature), _p(_i32(top_k, "top_k")), _p(top_p), _p(rep_penalty), _p(presence), _p(frequency),
           _p(draw), _p(_i32(hist, "hist")), _p(_i32(hist_start, "hist_start")), _p(out))

@@ -91,8 +91,18 @@ class PagedAttention(Mixer):
         return {"k": (self.n_kv_heads, block_size, self.head_dim),
                 "v": (self.n_kv_heads, self.head_dim, block_size)}
 
-    def forward(self, x, ctx, cache, residual) -> None:
-        qkv = self.qkv(x)
+    def forward_from_residual(self, norm, ctx, cache, residual) -> bool:
+        """Few tokens: the norm is applied inside the q/k/v product."""
+        if (ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm"
+                or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
+            return False
+        qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=(norm.weight, norm.eps))
+        self.forward(None, ctx, cache, residual, qkv=qkv)
+        return True
+
+    def forward(self, x, ctx, cache, residual, qkv=None) -> None:
+        if qkv is None:
+            qkv = self.qkv(x)
         q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
@@ -103,7 +113,7 @@ class PagedAttention(Mixer):
         ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
                           k_pages if cache.writes else None, v_pages if cache.writes else None,
                           self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1], rot[2])
-        out = torch.empty((ctx.n_tokens, self.qw), dtype=x.dtype, device=x.device)
+        out = torch.empty((ctx.n_tokens, self.qw), dtype=qkv.dtype, device=qkv.device)
         items = ctx.memo("attention_items", lambda: attention_items(ctx))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
         if items["n_tiles"]:

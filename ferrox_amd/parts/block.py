@@ -17,7 +17,11 @@ class PreNormBlock(Block):
         return [(self._prefixes[s], getattr(self, s)) for s in ("norm1", "mixer", "norm2", "ffn")]
 
     def forward(self, h, ctx, cache) -> None:
-        x = self.norm1.forward(h, ctx)
-        self.mixer.forward(x, ctx, cache, h)
-        x = self.norm2.forward(h, ctx)
-        self.ffn.forward(x, ctx, h)
+        # a part may offer `forward_from_residual(norm, ...)`: it then applies the norm itself, fused
+        # into its first kernel, and says False when it cannot for this step
+        fused = getattr(self.mixer, "forward_from_residual", None)
+        if fused is None or not fused(self.norm1, ctx, cache, h):
+            self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
+        fused = getattr(self.ffn, "forward_from_residual", None)
+        if fused is None or not fused(self.norm2, ctx, h):
+            self.ffn.forward(self.norm2.forward(h, ctx), ctx, h)

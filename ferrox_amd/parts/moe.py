@@ -75,7 +75,18 @@ class SparseMoE(FeedForward):
             router = torch.cat(same_dtype([router, fetch("shared_expert_gate.weight").reshape(1, -1)]), dim=0)
         self.router = router.contiguous()
 
-    def forward(self, x, ctx, residual) -> None:
+    def forward_from_residual(self, norm, ctx, residual) -> bool:
+        """Few tokens: the norm, the router and the sort by expert are one launch."""
+        if residual.shape[0] > 16 or ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm":
+            return False
+        front = ops.moe_front(residual, norm.weight, norm.eps, self.router, self.n_experts, self.top_k,
+                              self.norm_topk_prob, self.gating, self.has_shared_gate)
+        if front is None:
+            return False
+        self.forward(front[0], ctx, residual, routed=front[1:])
+        return True
+
+    def forward(self, x, ctx, residual, routed=None) -> None:
         T = x.shape[0]
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
         if overlap:
@@ -88,9 +99,11 @@ class SparseMoE(FeedForward):
             with torch.cuda.stream(side):
                 shared_out = self.shared.output(x)
                 join.record(side)
-        logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
-        ids, weights, gate, offsets, sorted_token, sorted_pair, _ = ops.route(
-            logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating, self.has_shared_gate)
+        if routed is None:
+            logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
+            routed = ops.route(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
+                               self.has_shared_gate)
+        ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
         act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,

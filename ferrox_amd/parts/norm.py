@@ -9,6 +9,7 @@ from .base import NORMS, Norm, ParamSpec
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     kernel_libraries = ("elementwise",)
+    kind = "rmsnorm"       # parts that fuse this norm into their first kernel ask for it by this name
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)

@@ -201,6 +201,8 @@ def compare(got: dict, folder: str, requests: dict, atol: float, rtol: float, wh
                                      f"plain {float(ref[p][i]):.7f}, |diff| {float(err[i]):.3e} > {float(bound[i]):.3e}")
             if float(err.max()) > worst:
                 worst, worst_at = float(err.max()), (rid, p)
-    assert flips <= 0.1 * total, f"{what}: {flips} of {total} positions were routed differently"
+    # a flip is only accepted above where the plain model's own margin is below `flip_margin`; their
+    # share must stay small (one position is the least a short trace can show)
+    assert flips <= max(1, 0.1 * total), f"{what}: {flips} of {total} positions were routed differently"
     print(f"[{what}] largest |engine - plain| = {worst:.3e} at {worst_at}; {flips}/{total} positions routed on a near-tie")
     return worst

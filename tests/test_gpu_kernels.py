@@ -258,6 +258,57 @@ def test_sampling_kernel():
             assert got == want, f"{case} trial {trial}: kernel {got}, plain {want}"
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 2048), (8, 6144, 2048), (5, 100, 96), (16, 48, 264), (31, 257, 520),
+                                    (32, 2560, 1792)])
+@pytest.mark.parametrize("gamma_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_with_fused_norm(M, N, K, gamma_dtype):
+    """RMSNorm applied inside the product against norm kernel + product and against the plain norm"""
+    from ferrox_amd import ops
+    h = rnd(M, K, scale=2.0)
+    gamma = (1.0 + rnd(K, seed=3, scale=0.2)).to(gamma_dtype)
+    w, bias = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.05), rnd(N, dtype=torch.bfloat16, seed=2)
+    eps = 1e-6
+    assert ops.can_fuse_norm(h, w, M)
+    got = ops.gemm(h, w, bias=bias, norm=(gamma, eps))
+    two = ops.gemm(ops.rmsnorm(h, gamma, eps, torch.bfloat16), w, bias=bias)
+    want = plain.rms_norm(h.double().cpu(), gamma.double().cpu(), eps) @ w.double().cpu().T + bias.double().cpu()
+    close(got, want, torch.bfloat16, "fused norm product")
+    close(two, want, torch.bfloat16, "norm, then product")
+    assert not ops.can_fuse_norm(rnd(33, K), w, 33)
+
+
+@pytest.mark.parametrize("T,H,E,k,renorm,has_gate", [(1, 2048, 60, 4, False, True), (8, 2048, 60, 4, False, True),
+                                                      (16, 264, 7, 3, True, False), (5, 1792, 130, 8, True, True),
+                                                      (3, 64, 4, 4, False, True)])
+def test_moe_front(T, H, E, k, renorm, has_gate):
+    """norm + router products + selection + sort in one launch, twice in a row (the kernel's counter
+    must be back at zero), against the plain norm and router on the rounded activations"""
+    from ferrox_amd import ops
+    h = rnd(T + 2, H, scale=1.5)[1:T + 1]                                    # a view that starts past row 0
+    gamma = (1.0 + rnd(H, seed=3, scale=0.2)).to(torch.bfloat16)
+    router = rnd(E + (1 if has_gate else 0), H, dtype=torch.bfloat16, seed=4, scale=0.3)
+    eps = 1e-5
+    x_sep = ops.rmsnorm(h.contiguous(), gamma, eps, torch.bfloat16)
+    for rep in range(2):
+        got = ops.moe_front(h, gamma, eps, router, E, k, renorm, has_gate=has_gate)
+        assert got is not None
+        x, ids, w, gate, offsets, sorted_token, sorted_pair, inv = got
+        assert torch.equal(x, x_sep), "the fused norm rounds like the norm kernel"
+        want_x = plain.rms_norm(h.double().cpu(), gamma.double().cpu(), eps)
+        close(x, want_x, torch.bfloat16, "normed rows")
+        logits = router.double().cpu() @ x.double().cpu().T                  # [E(+1), T]
+        for t in range(T):
+            want_ids, want_w = plain.route_top_k(logits[:E, t], k, renorm)
+            assert ids[t].tolist() == want_ids, f"rep {rep} token {t}: experts {ids[t].tolist()} != {want_ids}"
+            close(w[t], want_w, torch.float32, f"router weights token {t}")
+        if has_gate:
+            close(gate, torch.sigmoid(logits[E]), torch.float32, "shared gate")
+        for a, b in zip((offsets, sorted_token, sorted_pair, inv), ops.moe_align(ids, E)):
+            assert torch.equal(a, b)
+    assert int(ops._counter(DEV).abs().sum()) == 0
+    assert ops.moe_front(rnd(17, H), gamma, eps, router, E, k, renorm, has_gate=has_gate) is None     # too many rows
+
+
 @pytest.mark.parametrize("T,E,k", [(1, 8, 2), (8, 60, 4), (64, 60, 4), (33, 130, 8), (65, 6, 3), (300, 60, 4)])
 def test_route_in_one_launch_equals_two(T, E, k):
     """selection and sort fused for small batches give what the two kernels give"""
