@@ -255,6 +255,167 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 }
 
 // ---------------------------------------------------------------------------
+// Many rows, K a multiple of 64: tiles of up to 256 rows x TN weight rows, eight
+// waves.  K advances in steps of 64 through a ring of NS stages in LDS; tiles
+// travel from global memory straight into LDS (no registers in between), NS-1
+// steps ahead of their use, and one barrier per step separates the waves that
+// still read a stage from the loads that refill it.  A wave-load fills 1 KB of
+// LDS, 8 rows of 64 k; inside a row the eight 16-byte chunks are stored at
+// chunk ^ ((row / 2) % 8), which the loading lanes achieve by choosing which
+// chunk they fetch, so that the 16 rows an MFMA operand reads fall on distinct
+// banks without padding.  Waves form a 2 x 4 grid: a wave owns TN/4 weight rows
+// and every second block of 16 rows (so a tile with few rows, an expert's share,
+// still spreads over both halves); row blocks past the tile's rows are not
+// multiplied.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void* fx_global_ptr;
+typedef __attribute__((address_space(3))) void* fx_lds_ptr;
+
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// The K loop of one wave for NA active row blocks (blocks wm, wm+2, ... of the tile).
+template <int NA, int MT, int NT, int TM, int TN, int NS>
+__device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* const (&a_src)[TM / 64],
+                                            const bf16* const (&b_src)[TN / 64], bf16* stages, int K, int wave,
+                                            int a_off, int b_off, int sw, int kq) {
+    constexpr int NLA = TM / 64, NLB = TN / 64, L = NLA + NLB;     // wave-loads per wave and step
+    constexpr int STAGE = (TM + TN) * 64;
+    const int nk = K >> 6;
+    auto issue = [&](int kt) {
+        const int k0 = min(kt, nk - 1) << 6;         // past the end: a tile nobody reads, so that counts stay even
+        bf16* st = stages + (kt % NS) * STAGE;
+#pragma unroll
+        for (int i = 0; i < NLA; ++i)
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(a_src[i] + k0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NLB; ++i)
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + k0),
+                                             (fx_lds_ptr)(st + TM * 64 + (wave + 8 * i) * 512), 16, 0, 0);
+    };
+#pragma unroll
+    for (int p = 0; p < NS - 1; ++p) issue(p);
+    for (int kt = 0; kt < nk; ++kt) {
+        wait_loads_but<(NS - 2) * L>();        // this wave's part of step kt has landed
+        __builtin_amdgcn_s_barrier();          // ... everyone's has, and the stage of step kt-1 is free
+        issue(kt + NS - 1);
+        const bf16* base = stages + (kt % NS) * STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int koff = ((ks * 4 + kq) ^ sw) * 8;
+            bf16x8_t bfr[NT], af[NA];
+#pragma unroll
+            for (int j = 0; j < NT; ++j) bfr[j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff);
+#pragma unroll
+            for (int i = 0; i < NA; ++i) af[i] = *(const bf16x8_t*)(base + a_off + i * 32 * 64 + koff);
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    wait_loads_but<0>();                       // the loads past the end, before the block leaves
+}
+
+template <int TMB, int TN, int NS, bool DUAL, int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
+    constexpr int TM = TMB * 16;
+    constexpr int MT = TMB / 2;            // row blocks per wave
+    constexpr int NT = TN / 64;            // 16-row blocks of W per wave
+    constexpr int WN = TN / 4;
+    constexpr int OUT_TN = DUAL ? TN / 2 : TN;
+    constexpr int NLA = TM / 64, NLB = TN / 64;   // wave-loads (8 rows each) per wave and K step
+    static_assert(TM % 64 == 0 && TN % 64 == 0, "eight waves load 64 rows at a time");
+    __shared__ __attribute__((aligned(1024))) bf16 stages[NS * (TM + TN) * 64];
+
+    const int per_xcd = (g.n_col_tiles * g.n_row_tiles + 7) / 8;
+    const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (logical >= g.n_col_tiles * g.n_row_tiles) return;
+    int r0, r_end, expert;
+    locate_rows<TM>(g, logical % g.n_row_tiles, r0, r_end, expert);
+    if (r0 < 0) return;
+    const int n0 = (logical / g.n_row_tiles) * OUT_TN;
+    const int rows_here = min(TM, r_end - r0);
+    const int nblk = (rows_here + 15) >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
+
+    // what this lane fetches in each of its wave-loads: row 8*j + lane/8 of the tile, chunk (lane%8) ^ ((row/2)%8)
+    const bf16* a_src[NLA];
+    const bf16* b_src[NLB];
+#pragma unroll
+    for (int i = 0; i < NLA; ++i) {
+        const int j = wave + 8 * i, row = 8 * j + (lane >> 3);
+        const int chunk = (lane & 7) ^ (4 * (j & 1) + (lane >> 4));
+        const int m = r0 + min(row, rows_here - 1);          // rows past the end repeat the last one, unused
+        a_src[i] = (const bf16*)g.A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda + chunk * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < NLB; ++i) {
+        const int j = wave + 8 * i, row = 8 * j + (lane >> 3);
+        const int chunk = (lane & 7) ^ (4 * (j & 1) + (lane >> 4));
+        int col = DUAL ? n0 + (row >> 5) * 16 + (row & 15) : n0 + row;
+        col = min(col, g.N - 1);
+        b_src[i] = Wbase + (size_t)col * g.K + ((DUAL && ((row >> 4) & 1)) ? g.up_offset : 0) + chunk * 8;
+    }
+
+    f32x4_t acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    const int sw = (lane & 15) >> 1, kq = lane >> 4;
+    const int a_off = (wm * 16 + (lane & 15)) * 64, b_off = (TM + wn * WN + (lane & 15)) * 64;
+    const int na = (nblk - wm + 1) >> 1;         // this wave's active row blocks
+#define FX_LOOP(NA) wide_k_loop<NA, MT, NT, TM, TN, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq)
+    if (na > 3 * MT / 4) FX_LOOP(MT);
+    else if (na > MT / 2) FX_LOOP(3 * MT / 4);
+    else if (na > MT / 4) FX_LOOP(MT / 2);
+    else FX_LOOP(MT / 4);
+#undef FX_LOOP
+
+    // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
+            if (ml >= r_end || ml >= r0 + TM) continue;
+            const int m = g.c_rows ? g.c_rows[ml] : ml;
+            if (DUAL) {
+#pragma unroll
+                for (int j = 0; j < NT; j += 2) {
+                    const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
+                    if (n < g.N)
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(acc[i][j][r]) * acc[i][j + 1][r]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const int n = n0 + wn * WN + j * 16 + (lane & 15);
+                    if (n >= g.N) continue;
+                    float v = acc[i][j][r];
+                    if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
+                    if (EPI == EPI_STORE) {
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
+                    } else if (EPI == EPI_STORE_F32) {
+                        ((float*)g.C)[(size_t)m * g.ldc + n] = v;
+                    } else {
+                        if (g.row_scale) v *= g.row_scale[ml];
+                        ((float*)g.C)[(size_t)m * g.ldc + n] += v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Few rows (decode): the weights are streamed once from memory straight into
 // MFMA operands, no LDS staging.  A block owns 16 output columns (16 rows of W)
 // and up to 16*MT logical rows; its WAVES waves split K between them in pieces
@@ -539,6 +700,22 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 #undef FX_TILED
 }
 
+static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
+FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; }
+
+template <int TMB, int TN, int NS>
+static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
+    g.n_col_tiles = ceil_div(g.N, epi == EPI_SILU_MUL ? TN / 2 : TN);
+    g.n_row_tiles = m_tiles;
+    dim3 grid(8 * ceil_div((long)g.n_col_tiles * g.n_row_tiles, 8));
+    switch (epi) {
+        case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE><<<grid, 512, 0, s>>>(g); break;
+        case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32><<<grid, 512, 0, s>>>(g); break;
+        case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID><<<grid, 512, 0, s>>>(g); break;
+        default: gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_SILU_MUL><<<grid, 512, 0, s>>>(g); break;
+    }
+}
+
 template <int MT, int WAVES, int NW>
 static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
     dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 16 : 16 * NW), m_tiles);
@@ -634,6 +811,23 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     if (per_group <= 64) {
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
+    } else if (g.vec_ok && K % 64 == 0 && !g_no_wide) {
+        // the widest tile that still gives the 256 CUs (one block each) an even share of the work
+        const bool dual = epi == EPI_SILU_MUL;
+        auto tiles = [&](int tm, int tn) {
+            return (long)ceil_div(N, dual ? tn / 2 : tn) * (M / tm + (expert_offsets ? nonempty : (M % tm != 0)));
+        };
+        auto score = [&](int tm, int tn, double quality) {
+            const long t = tiles(tm, tn);
+            return quality * (double)t / (double)(ceil_div(t, 256) * 256L);
+        };
+        const double s256 = score(256, 256, 1.0), s128 = score(256, 128, 0.85), s64 = score(128, 128, 0.7);
+        if (s256 >= s128 && s256 >= s64)
+            launch_wide<16, 256, 2>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);
+        else if (s128 >= s64)
+            launch_wide<16, 128, 3>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);
+        else
+            launch_wide<8, 128, 4>(g, epi, M / 128 + (expert_offsets ? nonempty : (M % 128 != 0)), s);
     } else {
         const int m_tiles = M / 128 + (expert_offsets ? nonempty : (M % 128 != 0));
         const bool dual = epi == EPI_SILU_MUL;

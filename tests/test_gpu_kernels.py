@@ -27,7 +27,8 @@ def close(got, want, dtype, what, k=1):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 100, 96), (16, 256, 128), (17, 257, 200), (33, 72, 40),
-                                    (64, 64, 64), (130, 300, 520), (257, 129, 1032), (3, 50, 100)])
+                                    (64, 64, 64), (130, 300, 520), (257, 129, 1032), (3, 50, 100),
+                                    (130, 300, 512), (257, 129, 1024), (300, 520, 64), (513, 72, 128), (65, 16, 192)])
 def test_gemm_plain_and_epilogues(dtype, M, N, K):
     from ferrox_amd import ops
     a, w = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1)
@@ -44,7 +45,8 @@ def test_gemm_plain_and_epilogues(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,I,K", [(1, 32, 64), (7, 48, 96), (40, 100, 72), (200, 176, 256)])
+@pytest.mark.parametrize("M,I,K", [(1, 32, 64), (7, 48, 96), (40, 100, 72), (200, 176, 256), (300, 100, 128),
+                                    (257, 129, 64)])
 def test_gemm_gate_up(dtype, M, I, K):
     from ferrox_amd import ops
     a, w = rnd(M, K, dtype=dtype), rnd(2 * I, K, dtype=dtype, seed=1, scale=0.5)
@@ -54,7 +56,7 @@ def test_gemm_gate_up(dtype, M, I, K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,E,k,I,H", [(1, 4, 2, 32, 64), (9, 6, 3, 48, 96), (70, 5, 1, 40, 120), (300, 8, 2, 64, 128),
-                                        (64, 3, 2, 24, 72)])
+                                        (64, 3, 2, 24, 72), (520, 4, 3, 128, 256), (700, 3, 2, 200, 192)])
 def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     """router ids -> align -> grouped gate/up -> grouped down -> combine, against per-token loops."""
     from ferrox_amd import ops
