@@ -107,50 +107,81 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // [page][kv_head][slot][head_dim]; value pages hold the transpose
 // [page][kv_head][head_dim][slot], which is what the attention kernels read.
 // ---------------------------------------------------------------------------
+// Blocks 0 .. T-1 rotate one token each: the angles' sines and cosines once, then every head of q
+// (in place) and of k (into its page).  The blocks after them write v: one block per (eight
+// consecutive tokens, kv head), so that eight tokens that follow each other in one page go out as
+// one 16-byte store per head dimension into the transposed page.
 template <typename T>
-__global__ __launch_bounds__(128) void rope_kv_write_kernel(
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
-    // one block per (token, head): query heads first, then the kv heads
-    const int t = blockIdx.x, head = blockIdx.y;
-    const int pos = positions[t];
+    int n_tokens, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
+    __shared__ float cs[128], sn[128];     // rot / 2 <= 128
+    const int tid = threadIdx.x;
     const int half = rot >> 1;
-    if (head < nh) {
-        T* row = q + (size_t)t * ldq + (size_t)head * hd;
-        for (int p = threadIdx.x; p < half; p += 128) {
+    if ((int)blockIdx.x < n_tokens) {
+        const int t = blockIdx.x;
+        const int pos = positions[t];
+        for (int p = tid; p < half; p += 256) {
             const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
-            float sn, cs;
-            sincosf((float)pos * freq, &sn, &cs);
+            sincosf((float)pos * freq, &sn[p], &cs[p]);
+        }
+        __syncthreads();
+        T* k_dst = nullptr;
+        if (k_pages) {
+            const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+            k_dst = k_pages + ((size_t)page * nkv * bs + pos % bs) * hd;      // + kv head * bs * hd
+        }
+        const int heads = nh + (k_pages ? nkv : 0);
+        for (int i = tid; i < heads * half; i += 256) {
+            const int head = i / half, p = i - head * half;
             const int ia = interleaved ? 2 * p : p;
             const int ib = interleaved ? 2 * p + 1 : p + half;
-            const float a = to_float(row[ia]), b = to_float(row[ib]);
-            from_float(row + ia, a * cs - b * sn);
-            from_float(row + ib, a * sn + b * cs);
+            const T* src = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)(head - nh) * hd;
+            T* dst = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k_dst + (size_t)(head - nh) * bs * hd;
+            const float a = to_float(src[ia]), b = to_float(src[ib]);
+            from_float(dst + ia, a * cs[p] - b * sn[p]);
+            from_float(dst + ib, a * sn[p] + b * cs[p]);
+        }
+        if (k_pages && rot < hd) {         // beyond the rotated dimensions
+            const int rest = hd - rot;
+            for (int i = tid; i < nkv * rest; i += 256) {
+                const int kh = i / rest, d = rot + i - kh * rest;
+                k_dst[(size_t)kh * bs * hd + d] = k[(size_t)t * ldk + (size_t)kh * hd + d];
+            }
         }
         return;
     }
-    if (!k_pages) return;
-    const int kh = head - nh;
-    const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
-    const int slot = pos % bs;
-    T* k_dst = k_pages + (((size_t)page * nkv + kh) * bs + slot) * hd;
-    T* v_dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + slot;
-    const T* krow = k + (size_t)t * ldk + (size_t)kh * hd;
-    const T* vrow = v + (size_t)t * ldv + (size_t)kh * hd;
-    for (int p = threadIdx.x; p < half; p += 128) {
-        const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
-        float sn, cs;
-        sincosf((float)pos * freq, &sn, &cs);
-        const int ia = interleaved ? 2 * p : p;
-        const int ib = interleaved ? 2 * p + 1 : p + half;
-        const float a = to_float(krow[ia]), b = to_float(krow[ib]);
-        from_float(k_dst + ia, a * cs - b * sn);
-        from_float(k_dst + ib, a * sn + b * cs);
+    if (!v_pages) return;
+    const int b = blockIdx.x - n_tokens;
+    const int kh = b % nkv, t0 = (b / nkv) * 8;
+    const int n = min(8, n_tokens - t0);
+    const int pos0 = positions[t0], seq0 = token_seq[t0];
+    bool together = sizeof(T) == 2 && n == 8 && (bs & 7) == 0 && (pos0 & 7) == 0;
+    for (int i = 1; together && i < 8; ++i) together = positions[t0 + i] == pos0 + i && token_seq[t0 + i] == seq0;
+    if (together) {
+        const int page = block_table[(size_t)seq0 * max_blocks + pos0 / bs];
+        T* dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + pos0 % bs;
+        for (int d = tid; d < hd; d += 256) {
+            uint16_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)(v + (size_t)(t0 + i) * ldv + (size_t)kh * hd + d);
+            uint4 o;
+            o.x = e[0] | ((uint32_t)e[1] << 16);
+            o.y = e[2] | ((uint32_t)e[3] << 16);
+            o.z = e[4] | ((uint32_t)e[5] << 16);
+            o.w = e[6] | ((uint32_t)e[7] << 16);
+            *(uint4*)(dst + (size_t)d * bs) = o;
+        }
+        return;
     }
-    for (int d = rot + threadIdx.x; d < hd; d += 128) k_dst[d] = krow[d];     // beyond the rotated dimensions
-    for (int d = threadIdx.x; d < hd; d += 128) v_dst[(size_t)d * bs] = vrow[d];
+    for (int i = 0; i < n; ++i) {
+        const int t = t0 + i, pos = positions[t];
+        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+        T* dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + pos % bs;
+        for (int d = tid; d < hd; d += 256) dst[(size_t)d * bs] = v[(size_t)t * ldv + (size_t)kh * hd + d];
+    }
 }
 
 FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const void* k, int ldk,
@@ -159,20 +190,23 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
                             int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
     FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
     FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
-    FX_REQUIRE(nh + nkv <= 65535, "rope_kv_write: too many heads");
+    FX_REQUIRE(rot <= 256, "rope_kv_write: rotary dim %d is more than this kernel's 256", rot);
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const long n_blocks = (long)T + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
+    FX_REQUIRE(n_blocks < (1L << 31), "rope_kv_write: too many tokens and heads for one launch");
+    const unsigned blocks = (unsigned)n_blocks;
     if (dtype == FX_F32)
-        rope_kv_write_kernel<float><<<dim3(T, nh + nkv), 128, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
-                                                      positions, token_seq, block_table, max_blocks,
-                                                      (float*)k_pages, (float*)v_pages, nh, nkv, hd, bs, rot,
-                                                      interleaved, theta);
+        rope_kv_write_kernel<float><<<blocks, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
+                                                           positions, token_seq, block_table, max_blocks,
+                                                           (float*)k_pages, (float*)v_pages, T, nh, nkv, hd, bs, rot,
+                                                           interleaved, theta);
     else if (dtype == FX_BF16)
-        rope_kv_write_kernel<bf16><<<dim3(T, nh + nkv), 128, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
-                                                     positions, token_seq, block_table, max_blocks,
-                                                     (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, bs, rot,
-                                                     interleaved, theta);
+        rope_kv_write_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
+                                                          positions, token_seq, block_table, max_blocks,
+                                                          (bf16*)k_pages, (bf16*)v_pages, T, nh, nkv, hd, bs, rot,
+                                                          interleaved, theta);
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("rope_kv_write");

@@ -28,25 +28,26 @@ enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
 //   (ferrox-moe/src/lib.rs:100-121).
 //   gate_out[t] = sigmoid(logits[t, E])  (decoder.rs:2670-2672).
 // selection for one token by one wave; `score` is E floats of LDS owned by the wave
+// (`es`: distance between the logits of neighbouring experts, 1 for a row of a [T, E] matrix)
 __device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm,
                                              int gating, int* __restrict__ ids, float* __restrict__ weights,
-                                             float* __restrict__ gate_out, int* ids_copy) {
+                                             float* __restrict__ gate_out, int* ids_copy, long es = 1) {
     const int lane = threadIdx.x & 63;
-    if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E]));
+    if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E * es]));
     if (gating == GATE_SOFTMAX) {
         float mx = NEG_INFINITY_F;
-        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, row[e]);
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, row[e * es]);
         mx = wave_max(mx);
         float sum = 0.f;
         for (int e = lane; e < E; e += 64) {
-            const float ex = expf(row[e] - mx);
+            const float ex = expf(row[e * es] - mx);
             score[e] = ex;
             sum += ex;
         }
         sum = wave_sum(sum);
         for (int e = lane; e < E; e += 64) score[e] = score[e] / sum;
     } else {
-        for (int e = lane; e < E; e += 64) score[e] = 1.0f / (1.0f + expf(-row[e]));
+        for (int e = lane; e < E; e += 64) score[e] = 1.0f / (1.0f + expf(-row[e * es]));
     }
     __builtin_amdgcn_wave_barrier();
     // k rounds of "largest remaining", lower index on ties
@@ -84,26 +85,29 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
     if (lane < k) weights[t * k + lane] = renorm ? my_w / wsum : my_w;
 }
 
-__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, int T, int E,
-                                                            int k, int renorm, int gating, int* __restrict__ ids,
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, long es, int T,
+                                                            int E, int k, int renorm, int gating, int* __restrict__ ids,
                                                             float* __restrict__ weights, float* __restrict__ gate_out) {
     extern __shared__ float score_all[];   // 4 x E
     const int wave = threadIdx.x >> 6;
     const int t = blockIdx.x * 4 + wave;
     if (t >= T) return;
-    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr);
+    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr, es);
 }
 
-FX_API int fx_router_select(void* stream, const float* logits, long ld, int T, int E, int k, int renorm,
+// logits of token t and expert e stand at logits[t * ld + e * es] (either of the two may be 1)
+FX_API int fx_router_select(void* stream, const float* logits, long ld, long es, int T, int E, int k, int renorm,
                             int gating, int* ids, float* weights, float* gate_out) {
     FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
+    FX_REQUIRE(ld >= 1 && es >= 1, "router: bad strides %ld, %ld", ld, es);
     FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
     FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
-    FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
+    FX_REQUIRE(T <= 1 || es > 1 || ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns",
+               ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     if (T == 0) return 0;
-    router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating,
-                                                                                         ids, weights, gate_out);
+    router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, es, T, E, k, renorm,
+                                                                                         gating, ids, weights, gate_out);
     FX_CHECK_LAUNCH("router_select");
     return 0;
 }

@@ -64,7 +64,7 @@ _sigs = {
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
                                       c_void_p, c_void_p, c_int, c_int],
-    ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+    ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -293,17 +293,18 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
 
 
 def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
-    """From float32 router logits [T, >= E (+1)]: (ids int32 [T,k], weights float32 [T,k],
-    gate float32 [T] = sigmoid(logits[:, E]) or None)."""
-    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
-        raise KernelError("router_select: logits must be float32 [T, E] with unit inner stride")
+    """From float32 router logits [T, >= E (+1)] (any strides, so also the transpose of an
+    [E (+1), T] product): (ids int32 [T,k], weights float32 [T,k], gate float32 [T] =
+    sigmoid(logits[:, E]) or None)."""
+    if logits.dtype != torch.float32 or logits.dim() != 2 or min(logits.stride()) < 1:
+        raise KernelError("router_select: logits must be a float32 [T, E] matrix")
     T = logits.shape[0]
     ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
     gate = torch.empty((T,), dtype=torch.float32, device=logits.device) if has_gate else None
     if logits.shape[1] < n_experts + (1 if has_gate else 0):
         raise KernelError(f"router_select: {logits.shape[1]} columns for {n_experts} experts")
-    _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), T, n_experts, top_k,
+    _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), logits.stride(1), T, n_experts, top_k,
           1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
     return ids, weights, gate
 
@@ -311,11 +312,11 @@ def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gat
 def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
     """router_select followed by moe_align; one launch when the batch is small.
     Returns (ids, weights, gate, expert_offsets, sorted_token, sorted_pair, inv)."""
-    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
-        raise KernelError("route: logits must be float32 [T, E] with unit inner stride")
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelError("route: logits must be a float32 [T, E] matrix")
     T = logits.shape[0]
     dev = logits.device
-    if T <= 16 and logits.shape[1] >= n_experts + (1 if has_gate else 0):
+    if T <= 16 and logits.stride(1) == 1 and logits.shape[1] >= n_experts + (1 if has_gate else 0):
         n = T * top_k
         ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
         weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)

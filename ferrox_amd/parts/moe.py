@@ -100,7 +100,12 @@ class SparseMoE(FeedForward):
                 shared_out = self.shared.output(x)
                 join.record(side)
         if routed is None:
-            logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
+            if T > 64 and self.router.shape[0] <= 64 and self.router.dtype == x.dtype:
+                # few experts, many tokens: the router's rows are the short side of the product, so the
+                # kernel for few rows streams the activations once; the logits come out transposed
+                logits = ops.gemm(self.router, x, epilogue=ops.EPI_STORE_F32).t()
+            else:
+                logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
             routed = ops.route(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
                                self.has_shared_gate)
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed

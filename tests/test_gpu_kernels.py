@@ -210,6 +210,13 @@ def test_router(dtype, T, H, E, k, renorm):
         assert ids[t].tolist() == want_ids, f"token {t}: experts {ids[t].tolist()} != {want_ids}"
         close(w[t], want_w, torch.float32, f"router weights token {t}")
     close(gate, torch.sigmoid(xd @ sg.double().cpu()), torch.float32, "shared gate")
+    # the product the other way round (router rows as the short side), read through its transpose
+    logits_t = ops.gemm(torch.cat([wr, sg[None]]).contiguous(), x, epilogue=ops.EPI_STORE_F32).t()
+    assert logits_t.shape == logits.shape and logits_t.stride(1) != 1 or T == 1
+    ids_t, w_t, gate_t = ops.router_select(logits_t, E, k, renorm, has_gate=True)
+    assert torch.equal(ids_t, ids)
+    close(w_t, w, torch.float32, "router weights from transposed logits")
+    close(gate_t, gate, torch.float32, "shared gate from transposed logits")
 
 
 def test_router_golden_vector():
