@@ -14,6 +14,7 @@
 // Dual mode: two weight matrices (gate, up) are multiplied at once and the
 // epilogue stores silu(gate) * up  (ferrox-moe/src/lib.rs:655-658).
 #include "common.h"
+#include <utility>
 
 FX_DEFINE_LAST_ERROR()
 
@@ -271,6 +272,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 typedef __attribute__((address_space(1))) const void* fx_global_ptr;
 typedef __attribute__((address_space(3))) void* fx_lds_ptr;
 
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for(std::integer_sequence<int, Is...>, F&& f) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -281,6 +287,7 @@ template <int NA, int MT, int NT, int TM, int TN, int NS>
 __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* const (&a_src)[TM / 64],
                                             const bf16* const (&b_src)[TN / 64], bf16* stages, int K, int wave,
                                             int a_off, int b_off, int sw, int kq) {
+    const int koff0 = (kq ^ sw) * 8, koff1 = ((4 + kq) ^ sw) * 8;
     constexpr int NLA = TM / 64, NLB = TN / 64, L = NLA + NLB;     // wave-loads per wave and step
     constexpr int STAGE = (TM + TN) * 64;
     const int nk = K >> 6;
@@ -302,20 +309,29 @@ __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* 
         __builtin_amdgcn_s_barrier();          // ... everyone's has, and the stage of step kt-1 is free
         issue(kt + NS - 1);
         const bf16* base = stages + (kt % NS) * STAGE;
+        // 2*NA units of one operand of rows against NT operands of weights; the rows' operands are
+        // read from LDS a few units ahead of the products that use them
+        constexpr int U = 2 * NA, D = U > 3 ? 3 : U - 1;
+        bf16x8_t bfr[2][NT], fr[U];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const int koff = ((ks * 4 + kq) ^ sw) * 8;
-            bf16x8_t bfr[NT], af[NA];
+        for (int j = 0; j < NT; ++j) bfr[0][j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff0);
 #pragma unroll
-            for (int j = 0; j < NT; ++j) bfr[j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff);
+        for (int u = 0; u < D; ++u)
+            fr[u] = *(const bf16x8_t*)(base + a_off + (u % NA) * 32 * 64 + ((u / NA) ? koff1 : koff0));
+        static_for(std::make_integer_sequence<int, U>{}, [&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if (u + D < U)
+                fr[u + D] = *(const bf16x8_t*)(base + a_off + ((u + D) % NA) * 32 * 64 + (((u + D) / NA) ? koff1 : koff0));
+            if (u == 0) {
 #pragma unroll
-            for (int i = 0; i < NA; ++i) af[i] = *(const bf16x8_t*)(base + a_off + i * 32 * 64 + koff);
+                for (int j = 0; j < NT; ++j) bfr[1][j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff1);
+            }
+            __builtin_amdgcn_sched_barrier(0);      // the reads above stay ahead of the products below
 #pragma unroll
-            for (int i = 0; i < NA; ++i)
-#pragma unroll
-                for (int j = 0; j < NT; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
+            for (int j = 0; j < NT; ++j)
+                acc[u % NA][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fr[u], bfr[u / NA][j], acc[u % NA][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
     }
     wait_loads_but<0>();                       // the loads past the end, before the block leaves
 }
