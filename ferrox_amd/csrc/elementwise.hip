@@ -107,8 +107,9 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // [page][kv_head][slot][head_dim]; value pages hold the transpose
 // [page][kv_head][head_dim][slot], which is what the attention kernels read.
 // ---------------------------------------------------------------------------
-// Blocks 0 .. T-1 rotate one token each: the angles' sines and cosines once, then every head of q
-// (in place) and of k (into its page).  The blocks after them write v: one block per (eight
+// The first T * split blocks rotate: `split` blocks share a token, each computes the angles' sines
+// and cosines once and takes its part of the heads of q (in place) and of k (into its page); few
+// tokens get several blocks each, many tokens one.  The blocks after them write v: one block per (eight
 // consecutive tokens, kv head), so that eight tokens that follow each other in one page go out as
 // one 16-byte store per head dimension into the transposed page.
 template <typename T>
@@ -116,12 +117,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_tokens, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
+    int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
     __shared__ float cs[128], sn[128];     // rot / 2 <= 128
     const int tid = threadIdx.x;
     const int half = rot >> 1;
-    if ((int)blockIdx.x < n_tokens) {
-        const int t = blockIdx.x;
+    if ((int)blockIdx.x < n_tokens * split) {
+        const int t = blockIdx.x / split, part = blockIdx.x % split, step = 256 * split;
         const int pos = positions[t];
         for (int p = tid; p < half; p += 256) {
             const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
             k_dst = k_pages + ((size_t)page * nkv * bs + pos % bs) * hd;      // + kv head * bs * hd
         }
         const int heads = nh + (k_pages ? nkv : 0);
-        for (int i = tid; i < heads * half; i += 256) {
+        for (int i = part * 256 + tid; i < heads * half; i += step) {
             const int head = i / half, p = i - head * half;
             const int ia = interleaved ? 2 * p : p;
             const int ib = interleaved ? 2 * p + 1 : p + half;
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         }
         if (k_pages && rot < hd) {         // beyond the rotated dimensions
             const int rest = hd - rot;
-            for (int i = tid; i < nkv * rest; i += 256) {
+            for (int i = part * 256 + tid; i < nkv * rest; i += step) {
                 const int kh = i / rest, d = rot + i - kh * rest;
                 k_dst[(size_t)kh * bs * hd + d] = k[(size_t)t * ldk + (size_t)kh * hd + d];
             }
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         return;
     }
     if (!v_pages) return;
-    const int b = blockIdx.x - n_tokens;
+    const int b = blockIdx.x - n_tokens * split;
     const int kh = b % nkv, t0 = (b / nkv) * 8;
     const int n = min(8, n_tokens - t0);
     const int pos0 = positions[t0], seq0 = token_seq[t0];
@@ -176,11 +177,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         }
         return;
     }
-    for (int i = 0; i < n; ++i) {
+    for (int idx = tid; idx < n * hd; idx += 256) {      // tokens of different pages: element by element
+        const int i = idx / hd, d = idx - i * hd;
         const int t = t0 + i, pos = positions[t];
         const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
-        T* dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + pos % bs;
-        for (int d = tid; d < hd; d += 256) dst[(size_t)d * bs] = v[(size_t)t * ldv + (size_t)kh * hd + d];
+        v_pages[(((size_t)page * nkv + kh) * hd + d) * bs + pos % bs] = v[(size_t)t * ldv + (size_t)kh * hd + d];
     }
 }
 
@@ -194,18 +195,19 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const long n_blocks = (long)T + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
+    const int split = T <= 32 ? 8 : (T <= 128 ? 2 : 1);
+    const long n_blocks = (long)T * split + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
     FX_REQUIRE(n_blocks < (1L << 31), "rope_kv_write: too many tokens and heads for one launch");
     const unsigned blocks = (unsigned)n_blocks;
     if (dtype == FX_F32)
         rope_kv_write_kernel<float><<<blocks, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
                                                            positions, token_seq, block_table, max_blocks,
-                                                           (float*)k_pages, (float*)v_pages, T, nh, nkv, hd, bs, rot,
+                                                           (float*)k_pages, (float*)v_pages, T, split, nh, nkv, hd, bs, rot,
                                                            interleaved, theta);
     else if (dtype == FX_BF16)
         rope_kv_write_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
                                                           positions, token_seq, block_table, max_blocks,
-                                                          (bf16*)k_pages, (bf16*)v_pages, T, nh, nkv, hd, bs, rot,
+                                                          (bf16*)k_pages, (bf16*)v_pages, T, split, nh, nkv, hd, bs, rot,
                                                           interleaved, theta);
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);

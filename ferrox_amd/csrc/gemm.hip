@@ -34,6 +34,8 @@ struct GemmArgs {
     const int* a_rows;       // [M] or null: row of A to read for logical row m
     const int* c_rows;       // [M] or null: row of C to write for logical row m
     const int* expert_offsets;  // [E+1] or null
+    const int* pair_ids;        // few rows, unsorted: expert of logical row ("pair") m, instead of expert_offsets
+    int pair_div;               //   pair m reads row m / pair_div of A and writes row m of C
     int E;
     int M, N, K;
     const void* norm_w;  // skinny bf16 kernel only: A is the float32 residual stream and RMSNorm with these weights
@@ -83,6 +85,52 @@ __device__ __forceinline__ void locate_rows(const GemmArgs& g, int tile, int& r0
         }
         before += __shfl(incl, 63, 64);
     }
+}
+
+// lanes (of the 64 of a wave) whose `e` equals this lane's; e < 2^bits, e < 0 matches nothing
+__device__ __forceinline__ unsigned long long same_expert_lanes(int e, int bits) {
+    unsigned long long m = __ballot(e >= 0);
+    for (int b = 0; b < bits; ++b) {
+        const unsigned long long set = __ballot((e >> b) & 1);
+        m &= ((e >> b) & 1) ? set : ~set;
+    }
+    return e >= 0 ? m : 0ull;
+}
+
+// Up to 64 unsorted pairs: the experts that occur, in ascending order, get one tile per 16 of their
+// pairs, and a tile's rows are those pairs in their order.  Every wave works this out by itself
+// from the ids (a lane per pair).  Returns false for a tile past the last one; else the expert,
+// and in `my_pair` the pair of tile row lane % 16 (or -1).
+__device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& expert, int& my_pair) {
+    const int lane = threadIdx.x & 63;
+    int e = lane < g.M ? g.pair_ids[lane] : -1;
+    if (e >= g.E) e = -1;
+    int bits = 0;
+    while ((1 << bits) < g.E) ++bits;
+    const unsigned long long same = same_expert_lanes(e, bits);
+    const bool first = e >= 0 && lane == __ffsll((long long)same) - 1;
+    const int my_tiles = (__popcll(same) + 15) >> 4;
+    int before = 0;      // tiles of the experts that occur and are smaller than this lane's
+    for (unsigned long long m = __ballot(first); m; m &= m - 1) {
+        const int src = __ffsll((long long)m) - 1;
+        const int oe = __shfl(e, src, 64), ot = __shfl(my_tiles, src, 64);
+        if (oe < e) before += ot;
+    }
+    const unsigned long long sel = __ballot(first && tile >= before && tile < before + my_tiles);
+    if (!sel) return false;
+    const int src = __ffsll((long long)sel) - 1;
+    expert = __shfl(e, src, 64);
+    const int skip = (tile - __shfl(before, src, 64)) * 16;      // pairs of this expert in its earlier tiles
+    unsigned long long rows = ((unsigned long long)(unsigned)__shfl((int)(same >> 32), src, 64) << 32) |
+                              (unsigned)__shfl((int)(unsigned)same, src, 64);
+    const int li = lane & 15;
+    my_pair = -1;
+    for (int j = 0; j < skip + 16 && rows; ++j) {
+        const int p = __ffsll((long long)rows) - 1;
+        rows &= rows - 1;
+        if (j == skip + li) my_pair = p;
+    }
+    return true;
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
@@ -470,9 +518,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     constexpr int NACC = MT * NW;
     constexpr int COLS = DUAL ? 16 : 16 * NW;   // output columns of a block
     __shared__ f32x4_t red[WAVES][NACC][64];
-    int r0, r_end, expert;
-    locate_rows<16 * MT>(g, blockIdx.y, r0, r_end, expert);
-    if (r0 < 0) return;
+    int r0 = 0, r_end = 0, expert = 0, my_pair = -1;
+    const bool pairs = MT == 1 && g.pair_ids != nullptr;
+    if (pairs) {
+        if (!locate_pairs(g, blockIdx.y, expert, my_pair)) return;
+    } else {
+        locate_rows<16 * MT>(g, blockIdx.y, r0, r_end, expert);
+        if (r0 < 0) return;
+    }
     const int n0 = blockIdx.x * COLS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, grp = lane >> 4;
@@ -487,8 +540,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = r0 + mt * 16 + li;
-        const size_t off = (m < r_end) ? (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : 0;
-        xrow[mt] = (m < r_end) ? (NORM ? (const bf16*)((const float*)g.A + off) : (const bf16*)g.A + off) : nullptr;
+        const bool live = pairs ? my_pair >= 0 : m < r_end;
+        const size_t off = !live ? 0 : (size_t)(pairs ? my_pair / g.pair_div : (g.a_rows ? g.a_rows[m] : m)) * g.lda;
+        xrow[mt] = live ? (NORM ? (const bf16*)((const float*)g.A + off) : (const bf16*)g.A + off) : nullptr;
     }
     f32x4_t acc[MT][NW];
 #pragma unroll
@@ -570,9 +624,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             v += red[w][mt * NW + a][L];
             if (DUAL) v2 += red[w][mt * NW + 1][L];
         }
-        const int ml = r0 + mt * 16 + (L & 15);
-        if (ml >= r_end) continue;
-        const int m = g.c_rows ? g.c_rows[ml] : ml;
+        const int ml = pairs ? my_pair : r0 + mt * 16 + (L & 15);     // L % 16 == lane % 16
+        if (pairs ? ml < 0 : ml >= r_end) continue;
+        const int m = (g.c_rows && !pairs) ? g.c_rows[ml] : ml;
         float rstd = 1.f;
         if constexpr (NORM) {
             float total = 0.f;
@@ -771,13 +825,17 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int nw
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
-                   int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps) {
+                   int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
+                   const int* pair_ids, int pair_div) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     FX_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%ld ldc=%ld too small for K=%d N=%d", lda, ldc, K, N);
     FX_REQUIRE(!(epi == EPI_SILU_MUL && bias), "gemm: the gate/up epilogue takes no bias");
-    FX_REQUIRE(!expert_offsets || E > 0, "gemm: grouped mode needs E > 0");
+    FX_REQUIRE(!(expert_offsets || pair_ids) || E > 0, "gemm: grouped mode needs E > 0");
+    FX_REQUIRE(!pair_ids || (!expert_offsets && !a_rows && !c_rows && !row_scale && !norm_w && pair_div >= 1 && M <= 64 &&
+                             dtype == FX_BF16),
+               "gemm: unsorted pairs are for up to 64 bfloat16 rows without other row maps");
     FX_REQUIRE(!bias || bias_dtype == FX_F32 || bias_dtype == FX_BF16, "gemm: unknown bias dtype %d", bias_dtype);
     if (M == 0) return 0;
     if (norm_w) {
@@ -792,6 +850,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
+    g.pair_ids = pair_ids; g.pair_div = pair_div;
     hipStream_t s = (hipStream_t)stream;
     const int nonempty = expert_offsets ? (E < M ? E : M) : 0;
     if (dtype == FX_F32) {
@@ -811,9 +870,11 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                ((K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
                 (((uintptr_t)A | (uintptr_t)W) % 16 == 0));
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
-    if (g.vec_ok && per_group <= 64) {
-        const int mt = per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4);
-        const int m_tiles = M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
+    FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
+    if (g.vec_ok && (per_group <= 64 || pair_ids)) {
+        const int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
+        const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16
+                                     : M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
         const bool dual = epi == EPI_SILU_MUL;
         // two sets of weight rows per wave share the activations they multiply: worth it when
         // there are blocks enough either way

@@ -118,35 +118,62 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, long es,
 //   sorted_token[i]     : token of sorted row i
 //   sorted_pair[i]      : pair t*k + j of sorted row i
 //   inv[t*k + j]        : sorted row of pair (t, j)
-// Thread th owns the contiguous pairs [th*c, (th+1)*c) and counts them per
-// expert in its own row cnt[th][.]; thread e then turns column e into running
-// sums over th; a scan over the experts' totals gives the offsets; each thread
-// walks its pairs again and places them.  The order inside an expert is the
-// order of the pairs, whatever the number of threads.
+// The pairs are taken in groups of 64, a group per wave at a time.  Inside a
+// group the lanes find, with one ballot per bit of the expert id, which lanes hold
+// the same expert: that gives a pair's rank among its group's pairs of that
+// expert and the group's count cnt[group][expert].  Then, per expert, a scan over
+// the groups (lanes = groups) turns the counts into the number of earlier pairs;
+// a scan over the experts' totals gives the offsets; and every pair is placed at
+// offset + earlier groups + rank.  The order inside an expert is the order of the
+// pairs, whatever the number of waves.
 // ---------------------------------------------------------------------------
-// the sort itself, by one block; `offs` (E+1 ints) and `cnt` (rows*E uint16) are LDS
-__device__ __forceinline__ void align_block(const int* ids, int n, int k, int E, int* offs, uint16_t* cnt,
+// lanes (of the 64 of a wave) whose `e` equals this lane's; e < 2^bits, e < 0 matches nothing
+__device__ __forceinline__ unsigned long long same_expert_lanes(int e, int bits) {
+    unsigned long long m = __ballot(e >= 0);
+    for (int b = 0; b < bits; ++b) {
+        const unsigned long long set = __ballot((e >> b) & 1);
+        m &= ((e >> b) & 1) ? set : ~set;
+    }
+    return e >= 0 ? m : 0ull;
+}
+
+// the sort itself, by one block of whole waves; `offs` (E+1 ints) and `cnt` (rows*E ints) are LDS;
+// a row is `per_row` consecutive groups, rows = ceil(ceil(n/64) / per_row)
+__device__ __forceinline__ void align_block(const int* ids, int n, int k, int E, int per_row, int* offs, int* cnt,
                                             int* __restrict__ expert_offsets, int* __restrict__ sorted_token,
                                             int* __restrict__ sorted_pair, int* __restrict__ inv) {
-    const int nt = blockDim.x, th = threadIdx.x, lane = th & 63;
-    const int c = max(1, (n + nt - 1) / nt);
-    const int rows = min(nt, (n + c - 1) / c);    // threads that own at least one pair
-    const int b = min(n, th * c), b_end = min(n, (th + 1) * c);
-    for (int i = th; i < rows * E; i += nt) cnt[i] = 0;
+    const int nt = blockDim.x, th = threadIdx.x, lane = th & 63, wave = th >> 6, n_waves = nt >> 6;
+    const int G = (n + 63) >> 6, R = (G + per_row - 1) / per_row;
+    int bits = 0;
+    while ((1 << bits) < E) ++bits;
+    for (int i = th; i < R * E; i += nt) cnt[i] = 0;
     __syncthreads();
-    for (int i = b; i < b_end; ++i) {
-        const int e = ids[i];
-        if (e >= 0 && e < E) cnt[th * E + e] += 1;
+    for (int r = wave; r < R; r += n_waves) {          // a row belongs to one wave, its groups in order
+        for (int g = r * per_row; g < min(G, (r + 1) * per_row); ++g) {
+            const int i = g * 64 + lane;
+            int e = i < n ? ids[i] : -1;
+            if (e >= E) e = -1;
+            const unsigned long long same = same_expert_lanes(e, bits);
+            if (e >= 0 && lane == __ffsll((long long)same) - 1) cnt[r * E + e] += __popcll(same);
+        }
     }
     __syncthreads();
-    for (int e = th; e < E; e += nt) {
-        int run = 0;
-        for (int r = 0; r < rows; ++r) {
-            const int v = cnt[r * E + e];
-            cnt[r * E + e] = (uint16_t)run;
-            run += v;
+    // per expert: counts of the rows -> pairs in earlier rows; the total goes to offs[e + 1]
+    for (int e = wave; e < E; e += n_waves) {
+        int carry = 0;
+        for (int base = 0; base < R; base += 64) {
+            const int r = base + lane;
+            const int c = r < R ? cnt[r * E + e] : 0;
+            int v = c;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int u = __shfl_up(v, o, 64);
+                if (lane >= o) v += u;
+            }
+            if (r < R) cnt[r * E + e] = carry + v - c;
+            carry += __shfl(v, 63, 64);
         }
-        offs[e + 1] = run;  // total of expert e, scanned below
+        if (lane == 0) offs[e + 1] = carry;
     }
     __syncthreads();
     if (th < 64) {   // inclusive scan of the totals by the first wave, 64 experts at a time
@@ -166,24 +193,45 @@ __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E,
     }
     __syncthreads();
     for (int e = th; e <= E; e += nt) expert_offsets[e] = offs[e];
-    for (int i = b; i < b_end; ++i) {
-        const int e = ids[i];
-        if (e >= 0 && e < E) {
-            const int dst = offs[e] + cnt[th * E + e];
-            cnt[th * E + e] += 1;
-            sorted_token[dst] = i / k;
-            if (sorted_pair) sorted_pair[dst] = i;
-            if (inv) inv[i] = dst;
+    for (int r = wave; r < R; r += n_waves) {
+        for (int g = r * per_row; g < min(G, (r + 1) * per_row); ++g) {
+            const int i = g * 64 + lane;
+            int e = i < n ? ids[i] : -1;
+            if (e >= E) e = -1;
+            const unsigned long long same = same_expert_lanes(e, bits);
+            int before = 0;
+            if (e >= 0) before = cnt[r * E + e];       // pairs of this expert in earlier rows and groups
+            __builtin_amdgcn_wave_barrier();
+            if (e >= 0) {
+                const int dst = offs[e] + before + __popcll(same & ((1ull << lane) - 1ull));
+                sorted_token[dst] = i / k;
+                if (sorted_pair) sorted_pair[dst] = i;
+                if (inv) inv[i] = dst;
+                if (lane == __ffsll((long long)same) - 1) cnt[r * E + e] = before + __popcll(same);
+            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
 }
 
-__global__ __launch_bounds__(256) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E,
-                                                        int* __restrict__ expert_offsets,
+// groups per row such that the rows' counters fit `bytes` of LDS beside the offsets
+static int align_groups_per_row(long n, int E, size_t bytes, size_t* shm) {
+    const long G = (n + 63) / 64;
+    long max_rows = ((long)bytes - (long)(E + 1) * 4) / ((long)E * 4);
+    if (max_rows < 1) max_rows = 1;
+    long per_row = (G + max_rows - 1) / max_rows;
+    if (per_row < 1) per_row = 1;
+    const long R = (G + per_row - 1) / per_row;
+    *shm = (size_t)(E + 1) * 4 + (size_t)(R > 0 ? R : 1) * E * 4;
+    return (int)per_row;
+}
+
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E, int per_row,
+                                                         int* __restrict__ expert_offsets,
                                                         int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
                                                         int* __restrict__ inv) {
     extern __shared__ int lds[];
-    align_block(ids, n, k, E, lds, (uint16_t*)(lds + E + 1), expert_offsets, sorted_token, sorted_pair, inv);
+    align_block(ids, n, k, E, per_row, lds, lds + E + 1, expert_offsets, sorted_token, sorted_pair, inv);
 }
 
 // few tokens: selection (a wave per token) and the sort in one block of 16 waves
@@ -197,12 +245,12 @@ __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* 
     float* score = (float*)lds;                 // 16 x E
     int* ids_s = lds + 16 * E;                  // T * k
     int* offs = ids_s + T * k;                  // E + 1
-    uint16_t* cnt = (uint16_t*)(offs + E + 1);  // rows x E
+    int* cnt = offs + E + 1;                    // groups x E
     const int wave = threadIdx.x >> 6;
     if (wave < T)
         select_token(logits + (size_t)wave * ld, score + wave * E, wave, E, k, renorm, gating, ids, weights, gate_out, ids_s);
     __syncthreads();
-    align_block(ids_s, T * k, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
+    align_block(ids_s, T * k, k, E, 1, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
 }
 
 // ---------------------------------------------------------------------------
@@ -210,8 +258,9 @@ __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* 
 // Block (r, t): RMSNorm of row t of the float32 residual stream (same formula and
 // rounding as rmsnorm_kernel; block r = 0 writes it out as bfloat16 for the
 // experts), then the products of that rounded row with router rows 8r .. 8r+7,
-// two rows per wave, k in a fixed order, into `logits`.  The block that finishes
-// last selects the experts of every token (a wave per token) and sorts the pairs.
+// two rows per wave, k in a fixed order, into `logits`.  The token's block that
+// finishes last selects its experts.  Nothing is sorted: with so few rows the
+// expert products group the (token, slot) pairs themselves.
 // ---------------------------------------------------------------------------
 #define FRONT_THREADS 256
 #define FRONT_WAVES (FRONT_THREADS / 64)
@@ -233,9 +282,8 @@ __device__ __forceinline__ float dot8(uint4 w, const float* x) {
 __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
     const float* __restrict__ h, long ldh, const void* __restrict__ gamma, int gamma_dtype, float eps,
     bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm,
-    int gating, float* logits, int* ids, float* __restrict__ weights, float* __restrict__ gate_out,
-    int* __restrict__ expert_offsets, int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
-    int* __restrict__ inv, unsigned* counter) {
+    int gating, float* logits, int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ gate_out,
+    unsigned* counters) {
     extern __shared__ int lds[];
     __shared__ float red[FRONT_WAVES];
     float* xs = (float*)lds;            // H: the normed row as the experts will read it
@@ -288,32 +336,22 @@ __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
         if (wb) store_shared(logits + (size_t)t * n_rows + e_b, acc_b);
     }
 
-    if (!last_block_arrives(counter, gridDim.x * gridDim.y)) return;
-    const int n = T * k;
-    float* score = (float*)lds;                     // FRONT_WAVES x E
-    float* lrow = score + FRONT_WAVES * E;          // FRONT_WAVES x n_rows: a token's logits
-    int* ids_s = (int*)(lrow + FRONT_WAVES * n_rows);   // n
-    int* offs = ids_s + n;                          // E + 1
-    uint16_t* cnt = (uint16_t*)(offs + E + 1);      // rows x E
-    for (int tt = wave; tt < T; tt += FRONT_WAVES) {
-        float* mine = lrow + wave * n_rows;
-        for (int e = lane; e < n_rows; e += 64) mine[e] = load_shared(logits + (size_t)tt * n_rows + e);
+    if (!last_block_arrives(counters + t, gridDim.x)) return;
+    if (wave == 0) {
+        float* mine = (float*)lds;                  // n_rows logits, then E scores
+        for (int e = lane; e < n_rows; e += 64) mine[e] = load_shared(logits + (size_t)t * n_rows + e);
         __builtin_amdgcn_wave_barrier();
-        select_token(mine, score + wave * E, tt, E, k, renorm, gating, ids, weights, has_gate ? gate_out : nullptr, ids_s);
-        __builtin_amdgcn_wave_barrier();
+        select_token(mine, mine + n_rows, t, E, k, renorm, gating, ids, weights, has_gate ? gate_out : nullptr, nullptr);
     }
-    __syncthreads();
-    align_block(ids_s, n, k, E, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
 }
 
 // Returns 2 (and launches nothing) for sizes this kernel does not take; the caller then runs the
 // norm, the router product and the two routing kernels one after the other.  `logits` holds
-// T x (E + has_gate) floats; `counter` is one zeroed unsigned in device memory that launches on
-// one stream may share.
+// T x (E + has_gate) floats; `counters` are T zeroed unsigned in device memory, left at zero, that
+// launches on one stream may share.
 FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamma, int gamma_dtype, float eps,
                         void* x_out, const void* W, int H, int T, int E, int has_gate, int k, int renorm, int gating,
-                        float* logits, int* ids, float* weights, float* gate_out, int* expert_offsets,
-                        int* sorted_token, int* sorted_pair, int* inv, unsigned* counter) {
+                        float* logits, int* ids, float* weights, float* gate_out, unsigned* counters) {
     FX_REQUIRE(T >= 0 && H > 0, "moe_front: bad sizes T=%d H=%d", T, H);
     FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
     FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
@@ -321,17 +359,14 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
     FX_REQUIRE(gamma_dtype == FX_F32 || gamma_dtype == FX_BF16, "moe_front: unknown norm weight dtype %d", gamma_dtype);
     FX_REQUIRE(ldh >= H, "moe_front: rows of %ld hold fewer than %d columns", ldh, H);
     FX_REQUIRE(!has_gate || gate_out, "moe_front: a gate row needs a place for its output");
-    const long n = (long)T * k;
-    const long rows = n < FRONT_THREADS ? n : FRONT_THREADS;
-    const size_t front = (size_t)H * 4;
-    const size_t back = (size_t)(FRONT_WAVES * (2 * E + 1) + n + E + 1) * 4 + (size_t)rows * E * 2;
+    const size_t front = (size_t)H * 4, back = (size_t)(2 * E + 1) * 4;
     const size_t shm = front > back ? front : back;
-    if (T > 16 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
+    if (T > 16 || (long)T * k > 64 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
     dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
-    moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(
-        h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out, (const bf16*)W, H, T, E, has_gate, k, renorm, gating, logits, ids,
-        weights, gate_out, expert_offsets, sorted_token, sorted_pair, inv, counter);
+    moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out,
+                                                                        (const bf16*)W, H, T, E, has_gate, k, renorm,
+                                                                        gating, logits, ids, weights, gate_out, counters);
     FX_CHECK_LAUNCH("moe_front");
     return 0;
 }
@@ -340,12 +375,12 @@ FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* 
                         int* sorted_token, int* sorted_pair, int* inv) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
     FX_REQUIRE(E >= 1, "moe_align: E=%d", E);
-    int nt = 256;
-    while (nt > 64 && (size_t)nt * E * 2 + (E + 1) * 4 > 48 * 1024) nt >>= 1;
-    const size_t shm = (size_t)nt * E * 2 + (E + 1) * 4;
-    FX_REQUIRE(shm <= 48 * 1024, "moe_align: %d experts exceed this kernel's limit of about 380", E);
-    FX_REQUIRE((n + nt - 1) / nt < 65536, "moe_align: %d pairs are too many for one block", n);
-    moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, expert_offsets, sorted_token, sorted_pair, inv);
+    FX_REQUIRE(E <= 4096, "moe_align: %d experts are more than this kernel's 4096", E);
+    size_t shm;
+    const int per_row = align_groups_per_row(n, E, 60 * 1024, &shm);
+    const int nt = n > 4096 ? 1024 : (n > 256 ? 512 : 256);
+    moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, per_row, expert_offsets, sorted_token, sorted_pair,
+                                                          inv);
     FX_CHECK_LAUNCH("moe_align");
     return 0;
 }
@@ -361,8 +396,8 @@ FX_API int fx_router_select_align(void* stream, const float* logits, long ld, in
     FX_REQUIRE(ld >= E + (gate_out ? 1 : 0), "router: logits rows of %ld hold fewer than %d columns", ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     const long n = (long)T * k;
-    const long rows = n < 1024 ? n : 1024;
-    const size_t shm = (size_t)(16 * E + n + E + 1) * 4 + (size_t)rows * E * 2;
+    const long groups = (n + 63) / 64;
+    const size_t shm = (size_t)(16 * E + n + E + 1) * 4 + (size_t)groups * E * 4;
     if (T > 16 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
     router_select_align_kernel<<<1, 1024, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,

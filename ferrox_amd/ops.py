@@ -56,7 +56,7 @@ _sigs = {
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float],
+                          c_void_p, c_int, c_float, c_void_p, c_int],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -69,7 +69,7 @@ _sigs = {
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
-                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 9,
+                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 5,
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
@@ -189,7 +189,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          a_rows: torch.Tensor | None = None, c_rows: torch.Tensor | None = None,
          expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
-         norm: tuple | None = None) -> torch.Tensor:
+         norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -198,6 +198,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores silu(gate)*up.
     `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.  `c_rows`
     scatters the rows of the output (row_scale stays indexed by the logical row).
+    `pair_ids` (int32, up to 64 entries) replaces the sorted layout for
+    few rows: logical row m belongs to expert pair_ids[m], reads row m // pair_div of `a` and
+    writes row m of the output; the kernel groups the rows by expert itself.
     `norm` = (weight [K], eps): `a` is the float32 residual stream and RMSNorm is applied on the way
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     """
@@ -213,7 +216,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     if not w.is_contiguous():
         raise KernelError("gemm: weights must be contiguous")
     K = a.shape[1]
-    grouped = expert_offsets is not None
+    grouped = expert_offsets is not None or pair_ids is not None
+    if pair_ids is not None:
+        n_rows = pair_ids.numel()
     if grouped:
         if w.dim() != 3:
             raise KernelError("gemm: grouped weights must be [E, N, K]")
@@ -248,7 +253,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
           _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K,
           _p(norm[0]) if norm is not None else None, dtype_code(norm[0].dtype) if norm is not None else 0,
-          float(norm[1]) if norm is not None else 0.0)
+          float(norm[1]) if norm is not None else 0.0, _p(_i32(pair_ids, "pair_ids")), int(pair_div))
     return out
 
 
@@ -351,33 +356,29 @@ def _counter(device, n: int = 1) -> torch.Tensor:
 
 
 def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
-    """For up to 16 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
-    products, selection and the sort by expert.  Returns None for sizes the kernel does not take, else
-    (x, ids, weights, gate, expert_offsets, sorted_token, sorted_pair, inv)."""
+    """For up to 16 rows of the float32 residual stream (and up to 64 (token, slot) pairs), in one
+    launch: RMSNorm into bfloat16, router products and selection.  Returns None for sizes the kernel
+    does not take, else (x, ids, weights, gate); the expert products take `ids` as `pair_ids`."""
     T, H = h.shape
-    if (T > 16 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
+    if (T > 16 or T * top_k > 64 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
             or not router.is_contiguous() or router.shape != (n_experts + (1 if has_gate else 0), H)
             or norm_weight.numel() != H):
         return None
     dev = h.device
-    n = T * top_k
     x = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
     weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
     gate = torch.empty((T,), dtype=torch.float32, device=dev) if has_gate else None
-    offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
-    buf = torch.empty((3, n), dtype=torch.int32, device=dev)
     logits = torch.empty((T, router.shape[0]), dtype=torch.float32, device=dev)
     f, handle = _fn("moe", "fx_moe_front")
     rc = f(_stream(), _p(h), h.stride(0), _p(norm_weight), dtype_code(norm_weight.dtype), float(eps), _p(x), _p(router),
            H, T, n_experts, 1 if has_gate else 0, top_k, 1 if renorm else 0, gating, _p(logits), _p(ids), _p(weights),
-           _p(gate),
-           _p(offsets), _p(buf[0]), _p(buf[1]), _p(buf[2]), _p(_counter(dev)))
+           _p(gate), _p(_counter(dev, T)))
     if rc == 2:
         return None
     if rc:
         raise KernelError(handle.fx_last_error().decode())
-    return x, ids, weights, gate, offsets, buf[0], buf[1], buf[2]
+    return x, ids, weights, gate
 
 
 def moe_align(ids: torch.Tensor, n_experts: int):

@@ -76,14 +76,16 @@ class SparseMoE(FeedForward):
         self.router = router.contiguous()
 
     def forward_from_residual(self, norm, ctx, residual) -> bool:
-        """Few tokens: the norm, the router and the sort by expert are one launch."""
+        """Few tokens: the norm and the router are one launch, and the expert products group the
+        (token, slot) pairs themselves instead of reading a sorted layout."""
         if residual.shape[0] > 16 or ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm":
             return False
         front = ops.moe_front(residual, norm.weight, norm.eps, self.router, self.n_experts, self.top_k,
                               self.norm_topk_prob, self.gating, self.has_shared_gate)
         if front is None:
             return False
-        self.forward(front[0], ctx, residual, routed=front[1:])
+        x, ids, weights, gate = front
+        self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None))
         return True
 
     def forward(self, x, ctx, residual, routed=None) -> None:
@@ -111,10 +113,14 @@ class SparseMoE(FeedForward):
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
-        act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
-                     expert_offsets=offsets, n_rows=T * self.top_k)
-        # each expert's rows go back to the place of their (token, slot) pair
-        y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+        if offsets is None:      # few pairs, unsorted: row p of `act` and of `y` is pair p
+            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k)
+            y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids)
+        else:
+            act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
+                         expert_offsets=offsets, n_rows=T * self.top_k)
+            # each expert's rows go back to the place of their (token, slot) pair
+            y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
         if overlap:
             main.wait_event(join)
             shared_out.record_stream(main)

@@ -98,6 +98,34 @@ def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     close(h, ref, dtype, "moe")
 
 
+@pytest.mark.parametrize("T,E,k,I,H", [(1, 4, 2, 32, 64), (8, 60, 4, 1408, 2048), (16, 60, 4, 176, 256), (16, 5, 4, 48, 96),
+                                        (3, 700, 8, 64, 128), (7, 1, 1, 40, 72)])
+def test_grouped_gemm_from_unsorted_pairs(T, E, k, I, H):
+    """few rows: the products group the (token, slot) pairs by expert themselves; same numbers as
+    the sorted layout gives, row for row"""
+    from ferrox_amd import ops
+    dtype = torch.bfloat16
+    x = rnd(T, H, dtype=dtype)
+    w_gu, w_dn = rnd(E, 2 * I, H, dtype=dtype, seed=1, scale=0.3), rnd(E, H, I, dtype=dtype, seed=2, scale=0.3)
+    g = torch.Generator().manual_seed(11)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    if T >= 8 and E >= 8:
+        ids[:, 0] = 5            # one expert with a row of every token
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
+    act_s = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    y_s = ops.gemm(act_s, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+    act_p = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k)
+    y_p = ops.gemm(act_p, w_dn, epilogue=ops.EPI_STORE_F32, pair_ids=ids)
+    assert torch.equal(act_p, act_s[inv.long()])
+    assert torch.equal(y_p, y_s)
+    xd, gud, dnd = x.double().cpu(), w_gu.double().cpu(), w_dn.double().cpu()
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            a = (plain.silu(xd[t] @ gud[e, :I].T) * (xd[t] @ gud[e, I:].T)).to(torch.bfloat16).double()
+            close(y_p[t * k + j], a @ dnd[e].T, dtype, f"pair ({t}, {j})")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_and_embed(dtype):
     from ferrox_amd import ops
@@ -287,7 +315,7 @@ def test_gemm_with_fused_norm(M, N, K, gamma_dtype):
 
 
 @pytest.mark.parametrize("T,H,E,k,renorm,has_gate", [(1, 2048, 60, 4, False, True), (8, 2048, 60, 4, False, True),
-                                                      (16, 264, 7, 3, True, False), (5, 1792, 130, 8, True, True),
+                                                      (16, 264, 7, 3, True, False), (5, 1792, 130, 8, True, True), (16, 2048, 60, 4, False, True),
                                                       (3, 64, 4, 4, False, True)])
 def test_moe_front(T, H, E, k, renorm, has_gate):
     """norm + router products + selection + sort in one launch, twice in a row (the kernel's counter
@@ -301,7 +329,7 @@ def test_moe_front(T, H, E, k, renorm, has_gate):
     for rep in range(2):
         got = ops.moe_front(h, gamma, eps, router, E, k, renorm, has_gate=has_gate)
         assert got is not None
-        x, ids, w, gate, offsets, sorted_token, sorted_pair, inv = got
+        x, ids, w, gate = got
         assert torch.equal(x, x_sep), "the fused norm rounds like the norm kernel"
         want_x = plain.rms_norm(h.double().cpu(), gamma.double().cpu(), eps)
         close(x, want_x, torch.bfloat16, "normed rows")
@@ -312,10 +340,23 @@ def test_moe_front(T, H, E, k, renorm, has_gate):
             close(w[t], want_w, torch.float32, f"router weights token {t}")
         if has_gate:
             close(gate, torch.sigmoid(logits[E]), torch.float32, "shared gate")
-        for a, b in zip((offsets, sorted_token, sorted_pair, inv), ops.moe_align(ids, E)):
-            assert torch.equal(a, b)
     assert int(ops._counter(DEV).abs().sum()) == 0
     assert ops.moe_front(rnd(17, H), gamma, eps, router, E, k, renorm, has_gate=has_gate) is None     # too many rows
+
+
+@pytest.mark.parametrize("T,E,k", [(5000, 60, 4), (3000, 700, 2), (1, 3, 1), (130, 1, 1)])
+def test_sort_by_expert_at_large_sizes(T, E, k):
+    """more pairs than one round of counters holds: rows of several groups; against a stable sort"""
+    from ferrox_amd import ops
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
+    flat = ids.flatten().long().cpu()
+    order = torch.sort(flat, stable=True).indices
+    assert sorted_pair.cpu().tolist() == order.tolist()
+    assert sorted_token.cpu().tolist() == (order // k).tolist()
+    assert offsets.cpu().tolist() == [0] + torch.cumsum(torch.bincount(flat, minlength=E), 0).tolist()
+    assert inv.cpu()[order].tolist() == list(range(T * k))
 
 
 @pytest.mark.parametrize("T,E,k", [(1, 8, 2), (8, 60, 4), (64, 60, 4), (33, 130, 8), (65, 6, 3), (300, 60, 4)])
