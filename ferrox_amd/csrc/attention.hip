@@ -463,10 +463,15 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
     }
 }
 
-// decode: item = one token; block = one wave = (item, kv head x group block of 16 query heads, split)
-template <int HD>
-__global__ __launch_bounds__(64) void attn_mfma_decode_kernel(AttnArgs a) {
-    const int item = blockIdx.x, split = blockIdx.z, lane = threadIdx.x, li = lane & 15, g = lane >> 4;
+// decode, several waves per block: block = (item, kv head x group block of 16 query heads, split);
+// its waves take the split's tiles of 64 keys in turn and their results are merged through LDS in
+// wave order.  With one split the block writes the output itself, no second launch.
+template <int HD, int MAX_THREADS>
+__global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(AttnArgs a) {
+    extern __shared__ float wave_out[];      // [waves][rows][HD + 2]: o, then m and l
+    const int item = blockIdx.x, split = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int li = lane & 15, g = lane >> 4;
     const int group = a.nh / a.nkv, gblocks = (group + 15) / 16;
     const int kvh = blockIdx.y / gblocks, hb = blockIdx.y % gblocks;
     const int tok = a.item_tok[item];
@@ -483,23 +488,44 @@ __global__ __launch_bounds__(64) void attn_mfma_decode_kernel(AttnArgs a) {
     w.init(row_ok && !empty ? (const bf16*)a.q + (size_t)tok * a.ldq + (size_t)(h0 + li) * hd : nullptr, hd);
     if (!empty) {
         const int lo = row_ok ? kv_begin : 1, hi = row_ok ? kv_end - 1 : 0;
-        for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
+        for (int kt0 = (kv_begin / 64) * 64 + wave * 64; kt0 < kv_end; kt0 += n_waves * 64)
+            w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
     }
-    if (li < n && g == 0) {
-        float* pml = a.part_ml + (((size_t)item * a.nh + h0 + li) * a.splits + split) * 2;
-        pml[0] = empty ? NEG_INF : w.m * LN2;        // the running maximum is kept in base 2
-        pml[1] = empty ? 0.f : w.l;
+    const int stride = HD + 2;
+    float* mine = wave_out + (size_t)wave * n * stride;
+    if (row_ok && g == 0) {
+        mine[li * stride + HD] = w.m;            // base 2
+        mine[li * stride + HD + 1] = w.l;
     }
-    if (empty) return;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
         if (row < n) {
-            float* po = a.part_o + (((size_t)item * a.nh + h0 + row) * a.splits + split) * hd;
 #pragma unroll
-            for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
-                const int d = 16 * cb + li;
-                if (d < hd) po[d] = w.o[cb][r];
+            for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) mine[row * stride + 16 * cb + li] = w.o[cb][r];
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < n * hd; idx += blockDim.x) {
+        const int row = idx / hd, d = idx - row * hd;
+        float m = NEG_INF;
+        for (int u = 0; u < n_waves; ++u) m = fmaxf(m, wave_out[((size_t)u * n + row) * stride + HD]);
+        float l = 0.f, o = 0.f;
+        for (int u = 0; u < n_waves; ++u) {
+            const float* src = wave_out + ((size_t)u * n + row) * stride;
+            const float f = src[HD] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(src[HD] - m);
+            l += f * src[HD + 1];
+            o += f * src[d];
+        }
+        const int h = h0 + row;
+        if (a.splits == 1) {
+            from_float((bf16*)a.out + (size_t)tok * a.ldo + (size_t)h * hd + d, o / l);
+        } else {
+            a.part_o[(((size_t)item * a.nh + h) * a.splits + split) * hd + d] = o;
+            if (d == 0) {
+                float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
+                pml[0] = m == NEG_INF ? NEG_INF : m * LN2;
+                pml[1] = l;
             }
         }
     }
@@ -743,11 +769,17 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
         const int group = nh / nkv;
         dim3 gridm(n_items, nkv * ((group + 15) / 16), splits);
-        if (hd <= 32) attn_mfma_decode_kernel<32><<<gridm, 64, 0, s>>>(a);
-        else if (hd <= 64) attn_mfma_decode_kernel<64><<<gridm, 64, 0, s>>>(a);
-        else if (hd <= 128) attn_mfma_decode_kernel<128><<<gridm, 64, 0, s>>>(a);
-        else attn_mfma_decode_kernel<256><<<gridm, 64, 0, s>>>(a);
-        attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);
+        // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS
+        const int rows = group < 16 ? group : 16;
+        const int hdc = hd <= 32 ? 32 : (hd <= 64 ? 64 : (hd <= 128 ? 128 : 256));
+        int nw = hd <= 128 ? 8 : 4;      // the widest heads need the registers of half a block
+        while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk)) nw >>= 1;
+        const size_t shm = (size_t)nw * rows * (hdc + 2) * 4;
+        if (hd <= 32) attn_mfma_decode_block_kernel<32, 512><<<gridm, nw * 64, shm, s>>>(a);
+        else if (hd <= 64) attn_mfma_decode_block_kernel<64, 512><<<gridm, nw * 64, shm, s>>>(a);
+        else if (hd <= 128) attn_mfma_decode_block_kernel<128, 512><<<gridm, nw * 64, shm, s>>>(a);
+        else attn_mfma_decode_block_kernel<256, 256><<<gridm, nw * 64, shm, s>>>(a);
+        if (splits > 1) attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);
     } else {
         attn_decode_kernel<bf16><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);

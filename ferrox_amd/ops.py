@@ -277,16 +277,16 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None) -> None:
     """Single queries.  The keys are cut into chunks of `chunk` positions that are merged in
     ascending order; by default float32 uses 256 always (so that a result does not depend on the
-    batch) and bfloat16 picks the chunk that fills the GPU."""
+    batch) and bfloat16, whose blocks of eight waves share a chunk, takes the fewest chunks that
+    still put about two thousand waves on the GPU: one chunk, and no merge launch, from 256
+    (sequence, kv head) pairs on."""
     n = item_seq.numel()
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
             pairs = n * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
-            want = max(1, 4096 // max(1, pairs))
-            chunk = 64
-            while chunk < 4096 and -(-max_kv_len // chunk) > want:
-                chunk *= 2
+            want = max(1, 2048 // max(1, pairs * 8))
+            chunk = max(64, -(-(-(-max_kv_len // want)) // 64) * 64)
     splits = max(1, -(-max_kv_len // chunk))
     part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n, n_heads, splits, 2), dtype=torch.float32, device=q.device)
