@@ -278,21 +278,25 @@ FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
                                                           const float* __restrict__ shared, const float* __restrict__ gate,
-                                                          int H, int k) {
-    const int t = blockIdx.x;
+                                                          int H, int k, int slabs) {
+    const int t = blockIdx.x, T = gridDim.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= H) return;
     float acc = 0.f;
     for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
-    if (shared) acc += (gate ? gate[t] : 1.f) * shared[(size_t)t * H + c];     // routed first, then shared (lib.rs:746-750)
+    if (shared) {      // routed first, then shared (lib.rs:746-750); the shared output may come as `slabs` partial sums [slab][T][H]
+        float sh = 0.f;
+        for (int s = 0; s < slabs; ++s) sh += shared[((size_t)s * T + t) * H + c];
+        acc += (gate ? gate[t] : 1.f) * sh;
+    }
     h[(size_t)t * H + c] += acc;
 }
 
 FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv, const float* w,
-                          const float* shared, const float* gate, int T, int H, int k) {
-    FX_REQUIRE(T >= 0 && H > 0 && k > 0, "moe_combine: bad sizes");
+                          const float* shared, const float* gate, int T, int H, int k, int slabs) {
+    FX_REQUIRE(T >= 0 && H > 0 && k > 0 && slabs >= 1, "moe_combine: bad sizes");
     if (T == 0) return 0;
-    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, shared, gate, H, k);
+    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, shared, gate, H, k, slabs);
     FX_CHECK_LAUNCH("moe_combine");
     return 0;
 }

@@ -36,6 +36,8 @@ struct GemmArgs {
     const int* expert_offsets;  // [E+1] or null
     const int* pair_ids;        // few rows, unsorted: expert of logical row ("pair") m, instead of expert_offsets
     int pair_div;               //   pair m reads row m / pair_div of A and writes row m of C
+    int n_always, always_rows;  //   experts E .. E+n_always-1 take rows 0 .. always_rows-1 each: their tile s writes rows
+    int always_from_a;          //   M + s*always_rows + t of C and reads row t of A (1) or that same row of A (0)
     int E;
     int M, N, K;
     const void* norm_w;  // skinny bf16 kernel only: A is the float32 residual stream and RMSNorm with these weights
@@ -99,10 +101,11 @@ __device__ __forceinline__ unsigned long long same_expert_lanes(int e, int bits)
 
 // Up to 64 unsorted pairs: the experts that occur, in ascending order, get one tile per 16 of their
 // pairs, and a tile's rows are those pairs in their order.  Every wave works this out by itself
-// from the ids (a lane per pair).  Returns false for a tile past the last one; else the expert,
-// and in `my_pair` the pair of tile row lane % 16 (or -1).
-__device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& expert, int& my_pair) {
-    const int lane = threadIdx.x & 63;
+// from the ids (a lane per pair).  After those tiles come the experts that every row takes
+// (n_always of them, a shared expert cut into pieces), one tile each.  Returns false for a tile
+// past the last one; else the expert, and for tile row lane % 16 the rows of A and C (or -1).
+__device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& expert, int& a_row, int& c_row) {
+    const int lane = threadIdx.x & 63, li = lane & 15;
     int e = lane < g.M ? g.pair_ids[lane] : -1;
     if (e >= g.E) e = -1;
     int bits = 0;
@@ -110,25 +113,37 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
     const unsigned long long same = same_expert_lanes(e, bits);
     const bool first = e >= 0 && lane == __ffsll((long long)same) - 1;
     const int my_tiles = (__popcll(same) + 15) >> 4;
-    int before = 0;      // tiles of the experts that occur and are smaller than this lane's
+    int before = 0, total = 0;      // tiles of the experts that occur and are smaller than this lane's; of all
     for (unsigned long long m = __ballot(first); m; m &= m - 1) {
         const int src = __ffsll((long long)m) - 1;
         const int oe = __shfl(e, src, 64), ot = __shfl(my_tiles, src, 64);
         if (oe < e) before += ot;
+        total += ot;
+    }
+    a_row = c_row = -1;
+    if (tile >= total) {
+        const int s = tile - total;
+        if (s >= g.n_always) return false;
+        expert = g.E + s;
+        if (li < g.always_rows) {
+            c_row = g.M + s * g.always_rows + li;
+            a_row = g.always_from_a ? li : c_row;
+        }
+        return true;
     }
     const unsigned long long sel = __ballot(first && tile >= before && tile < before + my_tiles);
-    if (!sel) return false;
     const int src = __ffsll((long long)sel) - 1;
     expert = __shfl(e, src, 64);
     const int skip = (tile - __shfl(before, src, 64)) * 16;      // pairs of this expert in its earlier tiles
     unsigned long long rows = ((unsigned long long)(unsigned)__shfl((int)(same >> 32), src, 64) << 32) |
                               (unsigned)__shfl((int)(unsigned)same, src, 64);
-    const int li = lane & 15;
-    my_pair = -1;
     for (int j = 0; j < skip + 16 && rows; ++j) {
         const int p = __ffsll((long long)rows) - 1;
         rows &= rows - 1;
-        if (j == skip + li) my_pair = p;
+        if (j == skip + li) {
+            c_row = p;
+            a_row = p / g.pair_div;
+        }
     }
     return true;
 }
@@ -518,10 +533,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     constexpr int NACC = MT * NW;
     constexpr int COLS = DUAL ? 16 : 16 * NW;   // output columns of a block
     __shared__ f32x4_t red[WAVES][NACC][64];
-    int r0 = 0, r_end = 0, expert = 0, my_pair = -1;
+    int r0 = 0, r_end = 0, expert = 0, pair_a = -1, pair_c = -1;
     const bool pairs = MT == 1 && g.pair_ids != nullptr;
     if (pairs) {
-        if (!locate_pairs(g, blockIdx.y, expert, my_pair)) return;
+        if (!locate_pairs(g, blockIdx.y, expert, pair_a, pair_c)) return;
     } else {
         locate_rows<16 * MT>(g, blockIdx.y, r0, r_end, expert);
         if (r0 < 0) return;
@@ -540,8 +555,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = r0 + mt * 16 + li;
-        const bool live = pairs ? my_pair >= 0 : m < r_end;
-        const size_t off = !live ? 0 : (size_t)(pairs ? my_pair / g.pair_div : (g.a_rows ? g.a_rows[m] : m)) * g.lda;
+        const bool live = pairs ? pair_a >= 0 : m < r_end;
+        const size_t off = !live ? 0 : (size_t)(pairs ? pair_a : (g.a_rows ? g.a_rows[m] : m)) * g.lda;
         xrow[mt] = live ? (NORM ? (const bf16*)((const float*)g.A + off) : (const bf16*)g.A + off) : nullptr;
     }
     f32x4_t acc[MT][NW];
@@ -624,7 +639,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             v += red[w][mt * NW + a][L];
             if (DUAL) v2 += red[w][mt * NW + 1][L];
         }
-        const int ml = pairs ? my_pair : r0 + mt * 16 + (L & 15);     // L % 16 == lane % 16
+        const int ml = pairs ? pair_c : r0 + mt * 16 + (L & 15);      // L % 16 == lane % 16
         if (pairs ? ml < 0 : ml >= r_end) continue;
         const int m = (g.c_rows && !pairs) ? g.c_rows[ml] : ml;
         float rstd = 1.f;
@@ -826,7 +841,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
-                   const int* pair_ids, int pair_div) {
+                   const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -851,6 +866,9 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
     g.pair_ids = pair_ids; g.pair_div = pair_div;
+    g.n_always = n_always; g.always_rows = always_rows; g.always_from_a = always_from_a;
+    FX_REQUIRE(n_always >= 0 && (n_always == 0 || (pair_ids && always_rows >= 1 && always_rows <= 16)),
+               "gemm: experts that every row takes come with unsorted pairs and at most 16 rows");
     hipStream_t s = (hipStream_t)stream;
     const int nonempty = expert_offsets ? (E < M ? E : M) : 0;
     if (dtype == FX_F32) {
@@ -873,7 +891,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
     if (g.vec_ok && (per_group <= 64 || pair_ids)) {
         const int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
-        const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16
+        const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16 + n_always
                                      : M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
         const bool dual = epi == EPI_SILU_MUL;
         // two sets of weight rows per wave share the activations they multiply: worth it when

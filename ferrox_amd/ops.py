@@ -52,11 +52,11 @@ _sigs = {
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                        c_int, c_int, c_int],
+                                        c_int, c_int, c_int, c_int],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -174,14 +174,18 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
 
 def moe_combine(h, y_sorted, inv, weights, top_k, shared=None, gate=None) -> None:
     """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]] (inv None: y is in pair order t*k + j)
-    + gate[t] * shared[t] if the float32 output of a shared expert is given."""
+    + gate[t] * shared[t] if the float32 output of a shared expert is given; `shared` may also be
+    [S, T, H], partial outputs that are summed first."""
     T, H = h.shape
     if y_sorted.dtype != torch.float32 or h.dtype != torch.float32:
         raise KernelError("moe_combine works on float32")
-    if shared is not None and (shared.dtype != torch.float32 or shared.shape != h.shape or not shared.is_contiguous()):
-        raise KernelError("moe_combine: the shared expert's output must be float32 of h's shape")
+    slabs = 1
+    if shared is not None:
+        if shared.dtype != torch.float32 or not shared.is_contiguous() or shared.shape[-2:] != h.shape or shared.dim() > 3:
+            raise KernelError("moe_combine: the shared expert's output must be float32 [T, H] or [S, T, H]")
+        slabs = shared.shape[0] if shared.dim() == 3 else 1
     _call("elementwise", "fx_moe_combine", _stream(), _p(h), _p(y_sorted), _p(_i32(inv, "inv")), _p(weights),
-          _p(shared), _p(gate), T, H, top_k)
+          _p(shared), _p(gate), T, H, top_k, slabs)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: torch.Tensor | None = None,
@@ -189,7 +193,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          a_rows: torch.Tensor | None = None, c_rows: torch.Tensor | None = None,
          expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
-         norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1) -> torch.Tensor:
+         norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
+         always: tuple | None = None) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -200,7 +205,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     scatters the rows of the output (row_scale stays indexed by the logical row).
     `pair_ids` (int32, up to 64 entries) replaces the sorted layout for
     few rows: logical row m belongs to expert pair_ids[m], reads row m // pair_div of `a` and
-    writes row m of the output; the kernel groups the rows by expert itself.
+    writes row m of the output; the kernel groups the rows by expert itself.  `always` = (S, T,
+    from_a): the last S experts of `w` are taken by each of T rows (a shared expert cut into S
+    pieces); piece s writes output rows n_pairs + s*T + t and reads row t of `a` (from_a) or that
+    same row of `a`.
     `norm` = (weight [K], eps): `a` is the float32 residual stream and RMSNorm is applied on the way
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     """
@@ -217,12 +225,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
         raise KernelError("gemm: weights must be contiguous")
     K = a.shape[1]
     grouped = expert_offsets is not None or pair_ids is not None
+    n_always, always_rows, always_from_a = (int(always[0]), int(always[1]), 1 if always[2] else 0) if always else (0, 0, 0)
     if pair_ids is not None:
         n_rows = pair_ids.numel()
     if grouped:
         if w.dim() != 3:
             raise KernelError("gemm: grouped weights must be [E, N, K]")
         E, n_w, kw = w.shape
+        E -= n_always
         w_stride = n_w * kw
     else:
         if w.dim() != 2:
@@ -240,11 +250,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     else:
         N = n_out if n_out is not None else n_w
     out_dtype = w.dtype if epilogue in (EPI_STORE, EPI_SILU_MUL) else torch.float32
+    out_rows = M + n_always * always_rows
     if out is None:
         if epilogue == EPI_RESID:
             raise KernelError("gemm: the residual epilogue needs `out`")
-        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    if out.dtype != out_dtype or out.dim() != 2 or out.stride(1) != 1 or out.shape[0] < M or out.shape[1] < N:
+        out = torch.empty((out_rows, N), dtype=out_dtype, device=a.device)
+    if out.dtype != out_dtype or out.dim() != 2 or out.stride(1) != 1 or out.shape[0] < out_rows or out.shape[1] < N:
         raise KernelError(f"gemm: output {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {out_dtype}")
     if bias is not None and bias.numel() != N:
         raise KernelError(f"gemm: bias has {bias.numel()} elements for {N} columns")
@@ -253,7 +264,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
           _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K,
           _p(norm[0]) if norm is not None else None, dtype_code(norm[0].dtype) if norm is not None else 0,
-          float(norm[1]) if norm is not None else 0.0, _p(_i32(pair_ids, "pair_ids")), int(pair_div))
+          float(norm[1]) if norm is not None else 0.0, _p(_i32(pair_ids, "pair_ids")), int(pair_div),
+          n_always, always_rows, always_from_a)
     return out
 
 

@@ -69,8 +69,24 @@ class SparseMoE(FeedForward):
             gu.append(torch.cat(same_dtype([fetch(f"experts.{e}.gate_proj.weight"),
                                             fetch(f"experts.{e}.up_proj.weight")]), dim=0))
             dn.append(fetch(f"experts.{e}.down_proj.weight"))
-        self.w_gate_up = torch.stack(same_dtype(gu)).contiguous()     # [E, 2*I, H]
-        self.w_down = torch.stack(same_dtype(dn)).contiguous()        # [E, H, I]
+        # A shared expert whose width is a multiple of the experts' is also kept cut into pieces of their
+        # shape, after the experts in the same tensors: for few tokens it then runs as experts that every
+        # token takes, inside the experts' two launches (its own copy serves many tokens).
+        I, E = self.expert_intermediate_size, self.n_experts
+        self.shared_pieces = 0
+        if self.shared is not None and self.shared.intermediate_size % I == 0:
+            sg, su, sdn = (fetch("shared_expert." + n) for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight"))
+            if all(t.dtype == gu[0].dtype for t in gu + dn + [sg, su, sdn]):
+                S = self.shared.intermediate_size // I
+                for s in range(S):
+                    gu.append(torch.cat([sg[s * I:(s + 1) * I], su[s * I:(s + 1) * I]], dim=0))
+                    dn.append(sdn[:, s * I:(s + 1) * I])
+                self.shared_pieces = S
+            del sg, su, sdn
+        all_gu = torch.stack(same_dtype(gu)).contiguous()             # [E (+S), 2*I, H]
+        all_dn = torch.stack(same_dtype(dn)).contiguous()             # [E (+S), H, I]
+        self.w_gate_up_all, self.w_down_all = all_gu, all_dn
+        self.w_gate_up, self.w_down = all_gu[:E], all_dn[:E]
         if self.has_shared_gate:     # the gate's row rides along as column E of the router product
             router = torch.cat(same_dtype([router, fetch("shared_expert_gate.weight").reshape(1, -1)]), dim=0)
         self.router = router.contiguous()
@@ -90,6 +106,17 @@ class SparseMoE(FeedForward):
 
     def forward(self, x, ctx, residual, routed=None) -> None:
         T = x.shape[0]
+        if routed is not None and routed[3] is None and self.shared_pieces and x.dtype == self.w_gate_up_all.dtype:
+            # few tokens, unsorted pairs, shared expert as pieces: two launches do all experts
+            ids, weights, gate = routed[:3]
+            if SparseMoE.record is not None:
+                SparseMoE.record.append(ids)
+            S, n = self.shared_pieces, ids.numel()
+            act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k,
+                           always=(S, T, True))
+            y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False))
+            ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate)
+            return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
         if overlap:
             # few tokens: both halves are bound by reading weights, so the shared expert streams its

@@ -126,6 +126,41 @@ def test_grouped_gemm_from_unsorted_pairs(T, E, k, I, H):
             close(y_p[t * k + j], a @ dnd[e].T, dtype, f"pair ({t}, {j})")
 
 
+@pytest.mark.parametrize("T,E,k,I,H,S", [(1, 4, 2, 32, 64, 1), (8, 60, 4, 1408, 2048, 4), (16, 6, 3, 48, 96, 2), (5, 3, 1, 40, 72, 3)])
+def test_shared_expert_as_pieces_beside_unsorted_pairs(T, E, k, I, H, S):
+    """a shared expert of width S*I cut into S pieces that every token takes, in the same two launches
+    as the routed experts: the combine gives routed + gate * shared"""
+    from ferrox_amd import ops
+    dtype = torch.bfloat16
+    x = rnd(T, H, dtype=dtype)
+    w_gu, w_dn = rnd(E, 2 * I, H, dtype=dtype, seed=1, scale=0.3), rnd(E, H, I, dtype=dtype, seed=2, scale=0.3)
+    sg, su = rnd(S * I, H, dtype=dtype, seed=3, scale=0.3), rnd(S * I, H, dtype=dtype, seed=4, scale=0.3)
+    sd = rnd(H, S * I, dtype=dtype, seed=5, scale=0.3)
+    gu_all = torch.cat([w_gu] + [torch.cat([sg[s * I:(s + 1) * I], su[s * I:(s + 1) * I]])[None] for s in range(S)]).contiguous()
+    dn_all = torch.cat([w_dn] + [sd[:, s * I:(s + 1) * I][None] for s in range(S)]).contiguous()
+    g = torch.Generator().manual_seed(13)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    wts, gate = torch.rand(T, k, generator=g).to(DEV), torch.rand(T, generator=g).to(DEV)
+    n = T * k
+    act = ops.gemm(x, gu_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k, always=(S, T, True))
+    y = ops.gemm(act, dn_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False))
+    assert act.shape == (n + S * T, I) and y.shape == (n + S * T, H)
+    # the routed rows are what the products without the pieces give
+    assert torch.equal(act[:n], ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k))
+    h = torch.zeros(T, H, device=DEV)
+    ops.moe_combine(h, y[:n], None, wts, k, shared=y[n:].view(S, T, H), gate=gate)
+    xd = x.double().cpu()
+    ref = torch.zeros(T, H, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            a = (plain.silu(xd[t] @ w_gu[e, :I].double().cpu().T) * (xd[t] @ w_gu[e, I:].double().cpu().T)).to(dtype).double()
+            ref[t] += float(wts[t, j]) * (a @ w_dn[e].double().cpu().T)
+        a = (plain.silu(xd[t] @ sg.double().cpu().T) * (xd[t] @ su.double().cpu().T)).to(dtype).double()
+        ref[t] += float(gate[t]) * (a @ sd.double().cpu().T)
+    close(h, ref, dtype, "routed + gated shared")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_and_embed(dtype):
     from ferrox_amd import ops
