@@ -254,7 +254,7 @@ __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* 
 }
 
 // ---------------------------------------------------------------------------
-// Few tokens (decode): everything in front of the experts in one launch.
+// Few tokens (decode, up to 64): everything in front of the experts in one launch.
 // Block (r, t): RMSNorm of row t of the float32 residual stream (same formula and
 // rounding as rmsnorm_kernel; block r = 0 writes it out as bfloat16 for the
 // experts), then the products of that rounded row with router rows 8r .. 8r+7,
@@ -361,7 +361,7 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
     FX_REQUIRE(!has_gate || gate_out, "moe_front: a gate row needs a place for its output");
     const size_t front = (size_t)H * 4, back = (size_t)(2 * E + 1) * 4;
     const size_t shm = front > back ? front : back;
-    if (T > 16 || (long)T * k > 64 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
+    if (T > 64 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
     dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
     moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out,

@@ -368,11 +368,11 @@ def _counter(device, n: int = 1) -> torch.Tensor:
 
 
 def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
-    """For up to 16 rows of the float32 residual stream (and up to 64 (token, slot) pairs), in one
-    launch: RMSNorm into bfloat16, router products and selection.  Returns None for sizes the kernel
-    does not take, else (x, ids, weights, gate); the expert products take `ids` as `pair_ids`."""
+    """For up to 64 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
+    products and selection.  Returns None for sizes the kernel does not take, else
+    (x, ids, weights, gate)."""
     T, H = h.shape
-    if (T > 16 or T * top_k > 64 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
+    if (T > 64 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
             or not router.is_contiguous() or router.shape != (n_experts + (1 if has_gate else 0), H)
             or norm_weight.numel() != H):
         return None

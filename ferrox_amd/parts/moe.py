@@ -94,14 +94,18 @@ class SparseMoE(FeedForward):
     def forward_from_residual(self, norm, ctx, residual) -> bool:
         """Few tokens: the norm and the router are one launch, and the expert products group the
         (token, slot) pairs themselves instead of reading a sorted layout."""
-        if residual.shape[0] > 16 or ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm":
+        T = residual.shape[0]
+        if T > 64 or ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm":
             return False
         front = ops.moe_front(residual, norm.weight, norm.eps, self.router, self.n_experts, self.top_k,
                               self.norm_topk_prob, self.gating, self.has_shared_gate)
         if front is None:
             return False
         x, ids, weights, gate = front
-        self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None))
+        if T <= 16 and ids.numel() <= 64:       # the expert products take the pairs unsorted
+            self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None))
+        else:
+            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts))
         return True
 
     def forward(self, x, ctx, residual, routed=None) -> None:
