@@ -773,7 +773,10 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
         const int rows = group < 16 ? group : 16;
         const int hdc = hd <= 32 ? 32 : (hd <= 64 ? 64 : (hd <= 128 ? 128 : 256));
         int nw = hd <= 128 ? 8 : 4;      // the widest heads need the registers of half a block
-        while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk)) nw >>= 1;
+        const long n_blocks = (long)n_items * gridm.y * splits;
+        // fewer waves per block when there are blocks enough: a chunk's tiles then divide more evenly
+        while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk || n_blocks * (nw / 2) >= 2048))
+            nw >>= 1;
         const size_t shm = (size_t)nw * rows * (hdc + 2) * 4;
         if (hd <= 32) attn_mfma_decode_block_kernel<32, 512><<<gridm, nw * 64, shm, s>>>(a);
         else if (hd <= 64) attn_mfma_decode_block_kernel<64, 512><<<gridm, nw * 64, shm, s>>>(a);
