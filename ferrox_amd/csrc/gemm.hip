@@ -26,6 +26,8 @@ struct GemmArgs {
     const void* W;
     long w_stride;      // elements between experts (grouped)
     long up_offset;     // elements from the gate matrix to the up matrix (dual)
+    long kb_stride;     // 0: rows of W are K long.  Else W is stored [K/64][rows][64] (64 k of every row, then the
+                        // next 64 k of every row, ...) and this is rows * 64, the elements between two such slabs
     const void* bias;   // [N] or null
     int bias_dtype;
     void* C;
@@ -349,20 +351,21 @@ __device__ __forceinline__ void wait_loads_but() {
 template <int NA, int MT, int NT, int TM, int TN, int NS>
 __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* const (&a_src)[TM / 64],
                                             const bf16* const (&b_src)[TN / 64], bf16* stages, int K, int wave,
-                                            int a_off, int b_off, int sw, int kq) {
+                                            int a_off, int b_off, int sw, int kq, long kb_stride) {
     const int koff0 = (kq ^ sw) * 8, koff1 = ((4 + kq) ^ sw) * 8;
     constexpr int NLA = TM / 64, NLB = TN / 64, L = NLA + NLB;     // wave-loads per wave and step
     constexpr int STAGE = (TM + TN) * 64;
     const int nk = K >> 6;
     auto issue = [&](int kt) {
         const int k0 = min(kt, nk - 1) << 6;         // past the end: a tile nobody reads, so that counts stay even
+        const size_t w0 = kb_stride ? (size_t)min(kt, nk - 1) * kb_stride : (size_t)k0;
         bf16* st = stages + (kt % NS) * STAGE;
 #pragma unroll
         for (int i = 0; i < NLA; ++i)
             __builtin_amdgcn_global_load_lds((fx_global_ptr)(a_src[i] + k0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < NLB; ++i)
-            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + k0),
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0),
                                              (fx_lds_ptr)(st + TM * 64 + (wave + 8 * i) * 512), 16, 0, 0);
     };
 #pragma unroll
@@ -410,13 +413,28 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     static_assert(TM % 64 == 0 && TN % 64 == 0, "eight waves load 64 rows at a time");
     __shared__ __attribute__((aligned(1024))) bf16 stages[NS * (TM + TN) * 64];
 
-    const int per_xcd = (g.n_col_tiles * g.n_row_tiles + 7) / 8;
-    const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (logical >= g.n_col_tiles * g.n_row_tiles) return;
+    // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), each with an L2 of its own.  Plain: an XCD
+    // works through a contiguous range of column tiles, rows fastest, so the weights of those columns stay in
+    // its L2.  Grouped: XCD x takes the row tiles x, x + 8, ... and runs through the column tiles of each, so an
+    // expert's rows are fetched once and stay in its L2 while its weights, which nothing reads twice, stream by
+    // (the row tiles past the last expert are empty; dealing them out in turn spreads them over the XCDs).
+    int row_tile, col_tile;
+    if (g.expert_offsets) {
+        const int i = blockIdx.x / 8;
+        row_tile = (i / g.n_col_tiles) * 8 + blockIdx.x % 8;
+        col_tile = i % g.n_col_tiles;
+        if (row_tile >= g.n_row_tiles) return;
+    } else {
+        const int per_xcd = (g.n_col_tiles * g.n_row_tiles + 7) / 8;
+        const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+        if (logical >= g.n_col_tiles * g.n_row_tiles) return;
+        row_tile = logical % g.n_row_tiles;
+        col_tile = logical / g.n_row_tiles;
+    }
     int r0, r_end, expert;
-    locate_rows<TM>(g, logical % g.n_row_tiles, r0, r_end, expert);
+    locate_rows<TM>(g, row_tile, r0, r_end, expert);
     if (r0 < 0) return;
-    const int n0 = (logical / g.n_row_tiles) * OUT_TN;
+    const int n0 = col_tile * OUT_TN;
     const int rows_here = min(TM, r_end - r0);
     const int nblk = (rows_here + 15) >> 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -439,7 +457,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
         const int chunk = (lane & 7) ^ (4 * (j & 1) + (lane >> 4));
         int col = DUAL ? n0 + (row >> 5) * 16 + (row & 15) : n0 + row;
         col = min(col, g.N - 1);
-        b_src[i] = Wbase + (size_t)col * g.K + ((DUAL && ((row >> 4) & 1)) ? g.up_offset : 0) + chunk * 8;
+        const bool up = DUAL && ((row >> 4) & 1);
+        b_src[i] = g.kb_stride ? Wbase + ((size_t)col + (up ? g.up_offset / g.K : 0)) * 64 + chunk * 8
+                               : Wbase + (size_t)col * g.K + (up ? g.up_offset : 0) + chunk * 8;
     }
 
     f32x4_t acc[MT][NT];
@@ -451,7 +471,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     const int sw = (lane & 15) >> 1, kq = lane >> 4;
     const int a_off = (wm * 16 + (lane & 15)) * 64, b_off = (TM + wn * WN + (lane & 15)) * 64;
     const int na = (nblk - wm + 1) >> 1;         // this wave's active row blocks
-#define FX_LOOP(NA) wide_k_loop<NA, MT, NT, TM, TN, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq)
+#define FX_LOOP(NA) \
+    wide_k_loop<NA, MT, NT, TM, TN, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride)
     if (na > 3 * MT / 4) FX_LOOP(MT);
     else if (na > MT / 2) FX_LOOP(3 * MT / 4);
     else if (na > MT / 4) FX_LOOP(MT / 2);
@@ -508,6 +529,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 __device__ __forceinline__ uint4 load16(const bf16* row, int k, int K) {
     return (row && k < K) ? *(const uint4*)(row + k) : make_uint4(0, 0, 0, 0);
 }
+// the same from weights stored in slabs of 64 k (kb_stride elements apart; 0: plain rows)
+__device__ __forceinline__ uint4 load16w(const bf16* row, int k, int K, long kb_stride) {
+    if (!row || k >= K) return make_uint4(0, 0, 0, 0);
+    return kb_stride ? *(const uint4*)(row + (size_t)(k >> 6) * kb_stride + (k & 63)) : *(const uint4*)(row + k);
+}
 
 // NORM: the rows of A are float32 and are normed on the way in, y = x * rsqrt(mean(x^2) + eps) * w
 // (ferrox-core/src/matmul.rs:62-69): x * w is rounded to bfloat16 and multiplied, the sums of
@@ -549,7 +575,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
         const int n = DUAL ? n0 + li : n0 + a * 16 + li;
-        wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + ((DUAL && a) ? g.up_offset : 0) : nullptr;
+        if (g.kb_stride)
+            wrow[a] = (n < g.N) ? Wbase + ((size_t)n + ((DUAL && a) ? g.up_offset / g.K : 0)) * 64 : nullptr;
+        else
+            wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + ((DUAL && a) ? g.up_offset : 0) : nullptr;
     }
     const bf16* xrow[MT];       // NORM: float rows, kept under the same name
 #pragma unroll
@@ -578,7 +607,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
 #pragma unroll
-                for (int a = 0; a < NW; ++a) w[p][a][u] = load16(live ? wrow[a] : nullptr, kb + 32 * u, g.K);
+                for (int a = 0; a < NW; ++a) w[p][a][u] = load16w(live ? wrow[a] : nullptr, kb + 32 * u, g.K, g.kb_stride);
                 if constexpr (NORM) {
                     const int k = kb + 32 * u;
                     const bool kin = live && k < g.K;
@@ -792,7 +821,7 @@ template <int TMB, int TN, int NS>
 static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
     g.n_col_tiles = ceil_div(g.N, epi == EPI_SILU_MUL ? TN / 2 : TN);
     g.n_row_tiles = m_tiles;
-    dim3 grid(8 * ceil_div((long)g.n_col_tiles * g.n_row_tiles, 8));
+    dim3 grid(g.expert_offsets ? 8 * ceil_div(m_tiles, 8) * g.n_col_tiles : 8 * ceil_div((long)g.n_col_tiles * m_tiles, 8));
     switch (epi) {
         case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE><<<grid, 512, 0, s>>>(g); break;
         case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32><<<grid, 512, 0, s>>>(g); break;
@@ -841,7 +870,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
-                   const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a) {
+                   const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -866,6 +895,10 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
     g.pair_ids = pair_ids; g.pair_div = pair_div;
+    g.kb_stride = kb_rows * 64;
+    FX_REQUIRE(kb_rows >= 0 && (kb_rows == 0 || (dtype == FX_BF16 && K % 64 == 0 && ((uintptr_t)W % 16) == 0 && lda % 8 == 0 &&
+                                                 ((uintptr_t)A % 16) == 0 && (up_offset % K) == 0)),
+               "gemm: weights in slabs of 64 k are bfloat16 with K a multiple of 64 and aligned operands");
     g.n_always = n_always; g.always_rows = always_rows; g.always_from_a = always_from_a;
     FX_REQUIRE(n_always >= 0 && (n_always == 0 || (pair_ids && always_rows >= 1 && always_rows <= 16)),
                "gemm: experts that every row takes come with unsorted pairs and at most 16 rows");
@@ -903,6 +936,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }
+    const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
+    FX_REQUIRE(!g.kb_stride || (per_group > 64 && wide_ok), "gemm: no kernel for weights in slabs of 64 k at these sizes");
     if (per_group <= 64) {
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);

@@ -56,7 +56,7 @@ _sigs = {
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -194,7 +194,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
          norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
-         always: tuple | None = None) -> torch.Tensor:
+         always: tuple | None = None, w_kblocked: bool = False) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -209,6 +209,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     from_a): the last S experts of `w` are taken by each of T rows (a shared expert cut into S
     pieces); piece s writes output rows n_pairs + s*T + t and reads row t of `a` (from_a) or that
     same row of `a`.
+    `w_kblocked`: `w` is stored as `to_kblocked` makes it, [.., K/64, N, 64] (bfloat16, K % 64 == 0).
     `norm` = (weight [K], eps): `a` is the float32 residual stream and RMSNorm is applied on the way
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     """
@@ -228,7 +229,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     n_always, always_rows, always_from_a = (int(always[0]), int(always[1]), 1 if always[2] else 0) if always else (0, 0, 0)
     if pair_ids is not None:
         n_rows = pair_ids.numel()
-    if grouped:
+    if w_kblocked:
+        if w.dim() != (4 if grouped else 3) or w.shape[-1] != 64 or w.dtype != torch.bfloat16:
+            raise KernelError("gemm: weights in slabs must be bfloat16 [(E,) K/64, N, 64]")
+        n_w, kw = w.shape[-2], w.shape[-3] * 64
+        E, w_stride = (w.shape[0] - n_always, n_w * kw) if grouped else (0, 0)
+    elif grouped:
         if w.dim() != 3:
             raise KernelError("gemm: grouped weights must be [E, N, K]")
         E, n_w, kw = w.shape
@@ -265,8 +271,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K,
           _p(norm[0]) if norm is not None else None, dtype_code(norm[0].dtype) if norm is not None else 0,
           float(norm[1]) if norm is not None else 0.0, _p(_i32(pair_ids, "pair_ids")), int(pair_div),
-          n_always, always_rows, always_from_a)
+          n_always, always_rows, always_from_a, n_w if w_kblocked else 0)
     return out
+
+
+def to_kblocked(w: torch.Tensor) -> torch.Tensor:
+    """[.., N, K] -> [.., K/64, N, 64]: 64 k of every row, then the next 64 k of every row.  A tile of
+    rows then reads one contiguous stretch of memory per K step instead of a short piece of every
+    row, which is what the memory likes when the weights are streamed."""
+    *lead, N, K = w.shape
+    if K % 64:
+        raise KernelError(f"to_kblocked: K={K} is not a multiple of 64")
+    return w.reshape(*lead, N, K // 64, 64).transpose(-3, -2).contiguous()
 
 
 def can_fuse_norm(h: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:

@@ -72,7 +72,7 @@ class SparseMoE(FeedForward):
         # A shared expert whose width is a multiple of the experts' is also kept cut into pieces of their
         # shape, after the experts in the same tensors: for few tokens it then runs as experts that every
         # token takes, inside the experts' two launches (its own copy serves many tokens).
-        I, E = self.expert_intermediate_size, self.n_experts
+        I, E, H = self.expert_intermediate_size, self.n_experts, self.hidden_size
         self.shared_pieces = 0
         if self.shared is not None and self.shared.intermediate_size % I == 0:
             sg, su, sdn = (fetch("shared_expert." + n) for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight"))
@@ -85,6 +85,11 @@ class SparseMoE(FeedForward):
             del sg, su, sdn
         all_gu = torch.stack(same_dtype(gu)).contiguous()             # [E (+S), 2*I, H]
         all_dn = torch.stack(same_dtype(dn)).contiguous()             # [E (+S), H, I]
+        del gu, dn
+        # streamed weights are kept in slabs of 64 k where the kernels take that
+        self.kblocked = all_gu.dtype == torch.bfloat16 and all_dn.dtype == torch.bfloat16 and H % 64 == 0 and I % 64 == 0
+        if self.kblocked:
+            all_gu, all_dn = ops.to_kblocked(all_gu), ops.to_kblocked(all_dn)
         self.w_gate_up_all, self.w_down_all = all_gu, all_dn
         self.w_gate_up, self.w_down = all_gu[:E], all_dn[:E]
         if self.has_shared_gate:     # the gate's row rides along as column E of the router product
@@ -117,8 +122,9 @@ class SparseMoE(FeedForward):
                 SparseMoE.record.append(ids)
             S, n = self.shared_pieces, ids.numel()
             act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k,
-                           always=(S, T, True))
-            y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False))
+                           always=(S, T, True), w_kblocked=self.kblocked)
+            y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False),
+                         w_kblocked=self.kblocked)
             ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate)
             return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
@@ -144,14 +150,15 @@ class SparseMoE(FeedForward):
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
         if SparseMoE.record is not None:
             SparseMoE.record.append(ids)
+        kb = dict(w_kblocked=True) if self.kblocked else {}
         if offsets is None:      # few pairs, unsorted: row p of `act` and of `y` is pair p
-            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k)
-            y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids)
+            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k, **kb)
+            y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids, **kb)
         else:
             act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
-                         expert_offsets=offsets, n_rows=T * self.top_k)
+                         expert_offsets=offsets, n_rows=T * self.top_k, **kb)
             # each expert's rows go back to the place of their (token, slot) pair
-            y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+            y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
         if overlap:
             main.wait_event(join)
             shared_out.record_stream(main)

@@ -161,6 +161,39 @@ def test_shared_expert_as_pieces_beside_unsorted_pairs(T, E, k, I, H, S):
     close(h, ref, dtype, "routed + gated shared")
 
 
+@pytest.mark.parametrize("T,E,k,I,H", [(1, 4, 2, 64, 64), (8, 60, 4, 1408, 2048), (40, 6, 3, 128, 192), (300, 8, 2, 64, 128),
+                                        (520, 4, 3, 128, 256), (2048, 60, 4, 192, 256)])
+def test_weights_in_slabs_of_64_k(T, E, k, I, H):
+    """the same products from weights stored [K/64][rows][64]: bit for bit what plain rows give, for
+    few rows, many rows, sorted and unsorted pairs, and a plain (not grouped) matrix"""
+    from ferrox_amd import ops
+    dtype = torch.bfloat16
+    x = rnd(T, H, dtype=dtype)
+    w_gu, w_dn = rnd(E, 2 * I, H, dtype=dtype, seed=1, scale=0.3), rnd(E, H, I, dtype=dtype, seed=2, scale=0.3)
+    kb_gu, kb_dn = ops.to_kblocked(w_gu), ops.to_kblocked(w_dn)
+    assert kb_gu.shape == (E, H // 64, 2 * I, 64) and torch.equal(kb_gu[1, 0, 5], w_gu[1, 5, :64])
+    g = torch.Generator().manual_seed(17)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    act_kb = ops.gemm(x, kb_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k,
+                      w_kblocked=True)
+    assert torch.equal(act, act_kb)
+    y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+    y_kb = ops.gemm(act, kb_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, w_kblocked=True)
+    assert torch.equal(y, y_kb)
+    if T * k <= 64:
+        assert torch.equal(ops.gemm(x, kb_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k, w_kblocked=True),
+                           ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k))
+    # a plain matrix with bias, stored, and added into a residual
+    bias = rnd(2 * I, dtype=dtype, seed=3)
+    assert torch.equal(ops.gemm(x, kb_gu[0], bias=bias, w_kblocked=True), ops.gemm(x, w_gu[0], bias=bias))
+    h1, h2 = rnd(T, 2 * I, seed=4), rnd(T, 2 * I, seed=4)
+    ops.gemm(x, w_gu[0], epilogue=ops.EPI_RESID, out=h1)
+    ops.gemm(x, kb_gu[0], epilogue=ops.EPI_RESID, out=h2, w_kblocked=True)
+    assert torch.equal(h1, h2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_and_embed(dtype):
     from ferrox_amd import ops
