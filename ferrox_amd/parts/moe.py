@@ -107,7 +107,8 @@ class SparseMoE(FeedForward):
         if front is None:
             return False
         x, ids, weights, gate = front
-        if T <= 16 and ids.numel() <= 64:       # the expert products take the pairs unsorted
+        aligned = self.hidden_size % 8 == 0 and self.expert_intermediate_size % 8 == 0
+        if T <= 16 and ids.numel() <= 64 and aligned:       # the expert products take the pairs unsorted
             self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None))
         else:
             self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts))

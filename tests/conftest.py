@@ -63,7 +63,17 @@ WIDE_E = {
     "max_position_embeddings": 8192, "use_sliding_window": True, "sliding_window": 100,
     "max_window_layers": 1, "tie_word_embeddings": True,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4)}
+# widths that are multiples of 4 only (no 16-byte rows), three experts, head_dim 16: the kernels' guarded paths
+ODD_F = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 2, "hidden_size": 68, "num_attention_heads": 2, "num_key_value_heads": 1,
+    "head_dim": 16, "num_experts": 3, "num_experts_per_tok": 2, "norm_topk_prob": False,
+    "moe_intermediate_size": 20, "shared_expert_intermediate_size": 36, "intermediate_size": 52,
+    "decoder_sparse_step": 1, "mlp_only_layers": [], "vocab_size": 101, "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-5, "max_position_embeddings": 512, "use_sliding_window": False, "sliding_window": 64,
+    "max_window_layers": 2, "tie_word_embeddings": False,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5)}
 
 
 @pytest.fixture(scope="session")
