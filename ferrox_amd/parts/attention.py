@@ -64,11 +64,12 @@ class PagedAttention(Mixer):
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # attention.rs:433
         self.position = POSITION_ENCODINGS.build(position)
+        self._position_prefix = position.prefix or ""       # where the encoding's own tensors (if any) are named
         self.qw, self.kvw = n_heads * head_dim, n_kv_heads * head_dim
         self.qkv = self.o_proj = None
 
     def children(self):
-        return [("", self.position)]
+        return [(self._position_prefix, self.position)]
 
     def param_specs(self):
         H = self.hidden_size

@@ -12,8 +12,8 @@ import replay_util as ru
 from ferrox_amd import ops
 from ferrox_amd.engine.model import Model
 from ferrox_amd.engine.runner import ModelRunner, StepEntry
-from ferrox_amd.parts import (FEED_FORWARDS, MIXERS, FeedForward, LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec,
-                              ScheduleEntry)
+from ferrox_amd.parts import (FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, FeedForward, LayerSpec, Mixer, ModelSpec,
+                              ParamSpec, PartSpec, PositionEncoding, ScheduleEntry)
 from ferrox_amd.weights import RandomSource
 
 pytestmark = pytest.mark.gpu
@@ -66,6 +66,61 @@ class RunningMean(Mixer):
             mean = run / (ctx.positions[b:e].float()[:, None] + 1.0)
             y = mean.to(self.weight.dtype) @ self.weight.T
             ops.residual_add(residual[b:e], y.contiguous())
+
+
+@POSITION_ENCODINGS.register("test_decay_positions")
+class DecayPositions(PositionEncoding):
+    """Not a rotation: q_t is scaled by g^t and k_s by g^-s per head dimension, with a gain g of its own
+    (a tensor of the checkpoint), so that a score carries g^(t-s).  Each token is scaled by its own
+    position only, which is what lets keys be cached.  Written with torch operations."""
+
+    def __init__(self, head_dim: int):
+        self.head_dim = head_dim
+        self.gain = None
+
+    def param_specs(self):
+        return {"gain": ParamSpec((self.head_dim,))}
+
+    def load(self, fetch):
+        self.gain = fetch("gain")
+
+    @staticmethod
+    def factors(gain, positions):
+        """[T, head_dim] of g^t with g = 1 + gain / 64 (float32)"""
+        return torch.exp(positions.float()[:, None] * torch.log1p(gain.float() / 64.0)[None, :])
+
+    def apply(self, q, k, ctx):
+        f = self.factors(self.gain, ctx.positions)
+        hd = self.head_dim
+        qv, kv = q.view(q.shape[0], -1, hd), k.view(k.shape[0], -1, hd)
+        qv.copy_((qv.float() * f[:, None, :]).to(q.dtype))
+        kv.copy_((kv.float() / f[:, None, :]).to(k.dtype))
+
+
+@FEED_FORWARDS.register("test_top1_ffn")
+class Top1Linear(FeedForward):
+    """y = sigmoid(r_e) * W_e x for the one expert e with the largest router logit r = R x: a
+    feed-forward with routing of its own, written with torch operations."""
+
+    def __init__(self, hidden_size: int, n_experts: int):
+        self.hidden_size, self.n_experts = hidden_size, n_experts
+        self.router = self.experts = None
+
+    def param_specs(self):
+        H = self.hidden_size
+        specs = {"router.weight": ParamSpec((self.n_experts, H))}
+        specs.update({f"expert.{e}.weight": ParamSpec((H, H)) for e in range(self.n_experts)})
+        return specs
+
+    def load(self, fetch):
+        self.router = fetch("router.weight")
+        self.experts = torch.stack([fetch(f"expert.{e}.weight") for e in range(self.n_experts)])
+
+    def forward(self, x, ctx, residual):
+        r = x.float() @ self.router.float().T
+        best = r.argmax(-1)
+        y = torch.bmm(self.experts[best].float(), x.float()[:, :, None])[:, :, 0] * torch.sigmoid(r.max(-1).values)[:, None]
+        ops.residual_add(residual, y.to(x.dtype).contiguous())
 
 
 def norm(H, eps, prefix):
@@ -263,3 +318,36 @@ def test_layer_order_is_data():
         Model(spec_of(H, V, layers, [ScheduleEntry(0, cache=1), ScheduleEntry(1)]))      # only an earlier entry's cache
     with pytest.raises(KeyError):
         Model(spec_of(H, V, [layer(0, H, PartSpec("no_such_mixer"), PartSpec("test_no_ffn"))]))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_another_position_encoding_and_a_feed_forward_with_routing(dtype, tol):
+    """both registered above from outside the package, with tensors of their own in the checkpoint;
+    attention caches the keys as that encoding left them, so portions and single tokens must agree
+    with whole prompts, and all with a plain computation"""
+    H, V, nh, nkv, hd, E, T = 32, 50, 2, 1, 16, 3, len(TOKS)
+    mixer = PartSpec("paged_attention", {"hidden_size": H, "n_heads": nh, "n_kv_heads": nkv, "head_dim": hd, "bias": False,
+                                         "window": None, "position": PartSpec("test_decay_positions", {"head_dim": hd},
+                                                                              prefix="pos.")}, prefix="attn.")
+    ffn = PartSpec("test_top1_ffn", {"hidden_size": H, "n_experts": E}, prefix="route.")
+    model, w = build(spec_of(H, V, [layer(0, H, mixer, ffn)]), dtype, std=0.2)
+    assert {"l0.attn.pos.gain", "l0.route.router.weight", "l0.route.expert.2.weight"} <= set(model.named_params())
+    whole, cut = run_whole_and_cut(model, TOKS)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    x = plain.rms_norm(h, w["l0.n1.weight"], 1e-5)
+    f = DecayPositions.factors(w["l0.attn.pos.gain"], torch.arange(T)).double()
+    q = (x @ w["l0.attn.q_proj.weight"].T).reshape(T, nh, hd) * f[:, None, :]
+    k = (x @ w["l0.attn.k_proj.weight"].T).reshape(T, nkv, hd) / f[:, None, :]
+    v = (x @ w["l0.attn.v_proj.weight"].T).reshape(T, nkv, hd)
+    h = h + plain.causal_attention(q, k, v, nh, nkv, None).reshape(T, nh * hd) @ w["l0.attn.o_proj.weight"].T
+    x = plain.rms_norm(h, w["l0.n2.weight"], 1e-5)
+    r = x @ w["l0.route.router.weight"].T
+    top2 = r.topk(2, -1).values
+    y = torch.stack([torch.sigmoid(r[t].max()) * (w[f"l0.route.expert.{int(r[t].argmax())}.weight"] @ x[t]) for t in range(T)])
+    want = head_of(w, h + y)
+    keep = [t for t in range(T) if dtype == torch.float32 or float(top2[t, 0] - top2[t, 1]) > 0.05]     # clear choices
+    assert len(keep) > 0.7 * T
+    scale = float(want.abs().max())
+    # (the two toy parts call library matrix products, whose rounding depends on the number of rows:
+    # whole and cut agree within the tolerance, not bit for bit)
+    assert float((whole - want)[keep].abs().max()) < tol * scale and float((cut - want)[keep].abs().max()) < tol * scale
