@@ -30,6 +30,7 @@ struct AttnArgs {
     const int* item_tok;   // per work item: first token
     const int* item_n;     // per work item: number of queries (prefill tiles only)
     int nh, nkv, hd, bs, window;
+    int bs_shift;        // log2(bs) if bs is a power of two, else -1
     int n_items;
     float scale;
     // decode only
@@ -37,6 +38,49 @@ struct AttnArgs {
     float* part_ml;  // [items, nh, splits, 2]
     int splits, chunk;
 };
+
+static inline int log2_or_minus_one(int v) {
+    if (v <= 0 || (v & (v - 1))) return -1;
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return s;
+}
+
+// block of the table and slot in its page of key t (a shift when the page size is a power of two)
+__device__ __forceinline__ void page_slot(const AttnArgs& a, int t, int& blk, int& slot) {
+    if (a.bs_shift >= 0) {
+        blk = t >> a.bs_shift;
+        slot = t & (a.bs - 1);
+    } else {
+        blk = t / a.bs;
+        slot = t - blk * a.bs;
+    }
+}
+
+// Page ids of one sequence.  A block copies the entries of the key range it will walk into LDS once
+// (stage_pages), so that finding a tile's pages is an LDS read and not a round trip to memory on
+// which the tile's own loads would then wait; entries outside the copy come from memory.
+#define PAGE_COPY 1024
+struct PageLookup {
+    const int* table;    // the sequence's row of the block table
+    const int* copy;     // LDS
+    int first, count;    // copy[i] = table[first + i], i < count
+    __device__ __forceinline__ int page(int blk) const {
+        const unsigned i = (unsigned)(blk - first);
+        return i < (unsigned)count ? copy[i] : table[blk];
+    }
+};
+// every thread of the block calls this; blocks [first_blk, last_blk] of the table are wanted
+__device__ __forceinline__ PageLookup stage_pages(const int* table, int* lds, int first_blk, int last_blk) {
+    PageLookup pl;
+    pl.table = table;
+    pl.copy = lds;
+    pl.first = first_blk;
+    pl.count = min(PAGE_COPY, max(0, last_blk - first_blk + 1));
+    for (int i = threadIdx.x; i < pl.count; i += blockDim.x) lds[i] = table[first_blk + i];
+    __syncthreads();
+    return pl;
+}
 
 template <typename T>
 __device__ __forceinline__ const T* key_row(const AttnArgs& a, const int* bt, int kvh, int t) {
@@ -352,7 +396,7 @@ struct WaveAttn {
     }
 
     // keys [kt0, kt0 + 64); this lane's row sees key t iff lo <= t <= hi (hi < lo: row unused)
-    __device__ __forceinline__ void tile(const AttnArgs& a, const int* bt, int kvh, int kt0, int kv_begin, int kv_end,
+    __device__ __forceinline__ void tile(const AttnArgs& a, const PageLookup& pl, int kvh, int kt0, int kv_begin, int kv_end,
                                          int lo, int hi) {
         const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
         const int hd = a.hd, bs = a.bs;
@@ -364,7 +408,9 @@ struct WaveAttn {
         const int kg = kt0 + 16 * g;
         const bool vlive = kg < kv_end && kg + 16 > kv_begin;
         const int vkey = vlive ? kg : safe_group;
-        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)bt[vkey / bs] * a.nkv + kvh) * hd * bs + vkey % bs;
+        int vblk, vslot;
+        page_slot(a, vkey, vblk, vslot);
+        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)pl.page(vblk) * a.nkv + kvh) * hd * bs + vslot;
         uint4 vv[EARLY_V ? CB : 1][2];
         if (EARLY_V) {
 #pragma unroll
@@ -384,7 +430,9 @@ struct WaveAttn {
             const int key0 = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
             const bool klive = key0 >= kv_begin && key0 < kv_end;
             const int key = klive ? key0 : safe_group;
-            const bf16* kr = (const bf16*)a.k_pages + (((size_t)bt[key / bs] * a.nkv + kvh) * bs + key % bs) * hd;
+            int kblk, kslot;
+            page_slot(a, key, kblk, kslot);
+            const bf16* kr = (const bf16*)a.k_pages + (((size_t)pl.page(kblk) * a.nkv + kvh) * bs + kslot) * hd;
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
                 const int d = 32 * u + 8 * g;
@@ -448,7 +496,8 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
     }
     WaveAttn<HD> w;
     w.init(qrow, hd);
-    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
+    const PageLookup pl = {bt, nullptr, 0, 0};
+    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, pl, kvh, kt0, kv_begin, kv_end, lo, hi);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
@@ -483,13 +532,20 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
     const int n = min(16, group - hb * 16);        // query heads in this block
     const int h0 = kvh * group + hb * 16;
     const bool empty = kv_begin >= kv_end;
+    __shared__ int page_copy[PAGE_COPY];
+    int first_blk = 0, last_blk = -1, unused;
+    if (!empty) {
+        page_slot(a, kv_begin, first_blk, unused);
+        page_slot(a, kv_end - 1, last_blk, unused);
+    }
+    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
     WaveAttn<HD> w;
     const bool row_ok = li < n;
     w.init(row_ok && !empty ? (const bf16*)a.q + (size_t)tok * a.ldq + (size_t)(h0 + li) * hd : nullptr, hd);
     if (!empty) {
         const int lo = row_ok ? kv_begin : 1, hi = row_ok ? kv_end - 1 : 0;
         for (int kt0 = (kv_begin / 64) * 64 + wave * 64; kt0 < kv_end; kt0 += n_waves * 64)
-            w.tile(a, bt, kvh, kt0, kv_begin, kv_end, lo, hi);
+            w.tile(a, pl, kvh, kt0, kv_begin, kv_end, lo, hi);
     }
     const int stride = HD + 2;
     float* mine = wave_out + (size_t)wave * n * stride;
@@ -597,6 +653,11 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
     // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
     const int safe_group = (kv_end - 1) & ~15;
+    __shared__ int page_copy[PAGE_COPY];
+    int first_blk, last_blk, unused;
+    page_slot(a, kv_begin, first_blk, unused);
+    page_slot(a, kv_end - 1, last_blk, unused);
+    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
     auto fetch = [&](uint4* kreg, uint4* vreg, int kt0) {
         size_t kbase[4], vbase[4];     // page and slot of each group of 16 keys of the tile (the same for all threads)
         bool live[4];
@@ -604,10 +665,11 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         for (int j = 0; j < 4; ++j) {
             const int key0 = kt0 + 16 * j;
             live[j] = key0 < kv_end && key0 + 16 > kv_begin;
-            const int key = live[j] ? key0 : safe_group;
-            const size_t page = bt[key / bs];
-            kbase[j] = ((page * a.nkv + kvh) * bs + key % bs) * hd;
-            vbase[j] = (page * a.nkv + kvh) * hd * bs + key % bs;
+            int blk, slot;
+            page_slot(a, live[j] ? key0 : safe_group, blk, slot);
+            const size_t page = pl.page(blk);
+            kbase[j] = ((page * a.nkv + kvh) * bs + slot) * hd;
+            vbase[j] = (page * a.nkv + kvh) * hd * bs + slot;
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
@@ -728,6 +790,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
+    a.bs_shift = log2_or_minus_one(bs);
     a.n_items = n_items;
     dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
     hipStream_t s = (hipStream_t)stream;
@@ -750,7 +813,7 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
-                          float* part_o, float* part_ml, int splits, int chunk) {
+                          float* part_o, float* part_ml, int splits, int chunk, int waves) {
     if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window)) return 1;
     FX_REQUIRE(splits > 0 && chunk > 0 && chunk % 64 == 0, "attn_decode: chunk %d must be a positive multiple of 64", chunk);
     FX_REQUIRE(splits <= 8192, "attn_decode: %d chunks are more than the merge kernel takes (8192)", splits);
@@ -760,6 +823,7 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = nullptr;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
+    a.bs_shift = log2_or_minus_one(bs);
     a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.chunk = chunk;
     dim3 grid(n_items, nh, splits), grid2(n_items, nh);
     hipStream_t s = (hipStream_t)stream;
@@ -772,11 +836,14 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
         // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS
         const int rows = group < 16 ? group : 16;
         const int hdc = hd <= 32 ? 32 : (hd <= 64 ? 64 : (hd <= 128 ? 128 : 256));
-        int nw = hd <= 128 ? 8 : 4;      // the widest heads need the registers of half a block
+        const int nw_max = hd <= 128 ? 8 : 4;      // the widest heads need the registers of half a block
+        int nw = nw_max;
+        FX_REQUIRE(waves >= 0 && waves <= nw_max, "attn_decode: %d waves per block, this head size takes up to %d", waves, nw_max);
         const long n_blocks = (long)n_items * gridm.y * splits;
         // fewer waves per block when there are blocks enough: a chunk's tiles then divide more evenly
         while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk || n_blocks * (nw / 2) >= 2048))
             nw >>= 1;
+        if (waves > 0 && (size_t)waves * rows * (hdc + 2) * 4 <= 48 * 1024) nw = waves;      // the caller's choice
         const size_t shm = (size_t)nw * rows * (hdc + 2) * 4;
         if (hd <= 32) attn_mfma_decode_block_kernel<32, 512><<<gridm, nw * 64, shm, s>>>(a);
         else if (hd <= 64) attn_mfma_decode_block_kernel<64, 512><<<gridm, nw * 64, shm, s>>>(a);

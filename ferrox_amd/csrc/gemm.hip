@@ -548,16 +548,18 @@ __device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
-template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false>   // NW: sets of 16 weight rows per wave (dual: gate and up)
+// NW: sets of 16 weight rows per wave; in dual mode set a is the gate (a even) or up (a odd) rows of
+// column group a / 2.
+template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
-    static_assert(!DUAL || NW == 2, "dual mode multiplies two matrices");
+    static_assert(!DUAL || NW % 2 == 0, "dual mode multiplies two matrices");
     static_assert(!NORM || (!DUAL && EPI == EPI_STORE), "the fused norm feeds a plain product");
     __shared__ float red_ss[NORM ? WAVES : 1][MT][64];
     float ss[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) ss[mt] = 0.f;
     constexpr int NACC = MT * NW;
-    constexpr int COLS = DUAL ? 16 : 16 * NW;   // output columns of a block
+    constexpr int COLS = DUAL ? 8 * NW : 16 * NW;   // output columns of a block
     __shared__ f32x4_t red[WAVES][NACC][64];
     int r0 = 0, r_end = 0, expert = 0, pair_a = -1, pair_c = -1;
     const bool pairs = MT == 1 && g.pair_ids != nullptr;
@@ -574,11 +576,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     const bf16* wrow[NW];
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
-        const int n = DUAL ? n0 + li : n0 + a * 16 + li;
+        const int n = DUAL ? n0 + (a >> 1) * 16 + li : n0 + a * 16 + li;
+        const bool up = DUAL && (a & 1);
         if (g.kb_stride)
-            wrow[a] = (n < g.N) ? Wbase + ((size_t)n + ((DUAL && a) ? g.up_offset / g.K : 0)) * 64 : nullptr;
+            wrow[a] = (n < g.N) ? Wbase + ((size_t)n + (up ? g.up_offset / g.K : 0)) * 64 : nullptr;
         else
-            wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + ((DUAL && a) ? g.up_offset : 0) : nullptr;
+            wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + (up ? g.up_offset : 0) : nullptr;
     }
     const bf16* xrow[MT];       // NORM: float rows, kept under the same name
 #pragma unroll
@@ -658,15 +661,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         for (int mt = 0; mt < MT; ++mt) red_ss[wave][mt][lane] = ss[mt];
     }
     __syncthreads();
-    constexpr int OUTS = DUAL ? MT : MT * NW;     // accumulator tiles that become output tiles
+    constexpr int SETS = DUAL ? NW / 2 : NW;      // column groups of a block
+    constexpr int OUTS = MT * SETS;               // accumulator tiles (dual: pairs of them) that become output tiles
     for (int idx = tid; idx < OUTS * 64; idx += WAVES * 64) {
         const int t = idx >> 6, L = idx & 63;
-        const int mt = DUAL ? t : t / NW, a = DUAL ? 0 : t % NW;
+        const int mt = t / SETS, a = t % SETS;
         f32x4_t v = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v2 = v;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            v += red[w][mt * NW + a][L];
-            if (DUAL) v2 += red[w][mt * NW + 1][L];
+            v += red[w][mt * NW + (DUAL ? 2 * a : a)][L];
+            if (DUAL) v2 += red[w][mt * NW + 2 * a + 1][L];
         }
         const int ml = pairs ? pair_c : r0 + mt * 16 + (L & 15);      // L % 16 == lane % 16
         if (pairs ? ml < 0 : ml >= r_end) continue;
@@ -814,6 +818,8 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 #undef FX_TILED
 }
 
+static int g_skinny_four = 1024;   // blocks that four-set tiles must still give; 0: never four sets (measurement)
+FX_API void fx_gemm_set_skinny_four(int blocks) { g_skinny_four = blocks; }
 static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
 FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; }
 
@@ -832,7 +838,7 @@ static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 
 template <int MT, int WAVES, int NW>
 static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
-    dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 16 : 16 * NW), m_tiles);
+    dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 8 * NW : 16 * NW), m_tiles);
     if constexpr (MT * NW * WAVES <= 32) {       // the partial sums of all waves fit in LDS
         if (g.norm_w) {
             gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE, true><<<grid, WAVES * 64, 0, s>>>(g);
@@ -843,7 +849,7 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
             case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
             case EPI_RESID: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_RESID><<<grid, WAVES * 64, 0, s>>>(g); break;
             default:
-                if constexpr (NW == 2) gemm_bf16_skinny_kernel<MT, WAVES, 2, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
+                if constexpr (NW % 2 == 0) gemm_bf16_skinny_kernel<MT, WAVES, NW, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
                 break;
         }
     }
@@ -852,7 +858,9 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
 // mt: row tiles per block (1, 2, 4); eight: 8 waves split K instead of 4; nw: 16-row weight sets per wave
 static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int nw, int m_tiles, hipStream_t s) {
 #define FX_SK(MT_, W_, NW_) launch_skinny_cfg<MT_, W_, NW_>(g, epi, m_tiles, s)
-    if (nw == 2) {
+    if (nw == 4) {
+        FX_SK(1, 4, 4);
+    } else if (nw == 2) {
         if (mt == 1) { if (eight) FX_SK(1, 8, 2); else FX_SK(1, 4, 2); }
         else if (mt == 2) { if (eight) FX_SK(2, 8, 2); else FX_SK(2, 4, 2); }
         else FX_SK(4, 4, 2);
@@ -929,8 +937,10 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         const bool dual = epi == EPI_SILU_MUL;
         // two sets of weight rows per wave share the activations they multiply: worth it when
         // there are blocks enough either way
-        const int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 2048) ? 2 : 1;
-        const long blocks = (long)ceil_div(N, dual ? 16 : 16 * nw) * m_tiles;
+        int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 2048) ? 2 : 1;
+        // four sets when even then there are blocks enough: a block's fixed work is spread over more weights
+        if (mt == 1 && !norm_w && g_skinny_four && (long)ceil_div(N, dual ? 32 : 64) * m_tiles >= g_skinny_four) nw = 4;
+        const long blocks = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles;
         const bool eight = blocks < 1024 && mt * nw <= 4 && K >= 2048;
         launch_skinny(g, epi, mt, eight, nw, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");

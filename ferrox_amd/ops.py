@@ -63,7 +63,7 @@ _sigs = {
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
-                                      c_void_p, c_void_p, c_int, c_int],
+                                      c_void_p, c_void_p, c_int, c_int, c_int],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
@@ -302,7 +302,8 @@ def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, 
 
 
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
-                     n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None) -> None:
+                     n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
+                     waves=0) -> None:
     """Single queries.  The keys are cut into chunks of `chunk` positions that are merged in
     ascending order; by default float32 uses 256 always (so that a result does not depend on the
     batch) and bfloat16, whose blocks of eight waves share a chunk, takes the fewest chunks that
@@ -322,7 +323,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")), n,
           n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
-          _p(part_o), _p(part_ml), splits, chunk)
+          _p(part_o), _p(part_ml), splits, chunk, int(waves))
 
 
 def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
