@@ -372,6 +372,18 @@ __device__ __forceinline__ f32x4_t pv_step(f32x4_t acc, bool rescale, const floa
     return acc;
 }
 
+// Eight consecutive keys' values (first_key ..): those outside [kv_begin, kv_end) become zeros.  Their
+// probabilities are zero, but what memory holds there need not be a number.
+__device__ __forceinline__ uint4 keep_keys(uint4 v, int first_key, int kv_begin, int kv_end) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int key = first_key + e;
+        if (key < kv_begin || key >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 template <int HD>   // compile-time bound of head_dim (a.hd <= HD)
 struct WaveAttn {
     static constexpr int KS = HD / 32;   // k-steps of S^T = K Q^T
@@ -406,6 +418,7 @@ struct WaveAttn {
         // values first, so that they arrive while the scores are computed: 16 consecutive keys
         // kt0 + 16g .. of transposed row d = 16*cb + li
         const int kg = kt0 + 16 * g;
+        const bool edge = kt0 < kv_begin || kt0 + 64 > kv_end;      // some key of the tile is outside
         const bool vlive = kg < kv_end && kg + 16 > kv_begin;
         const int vkey = vlive ? kg : safe_group;
         int vblk, vslot;
@@ -469,6 +482,10 @@ struct WaveAttn {
                 const bool ok = vlive && d < hd;
                 v0 = ok ? x0 : make_uint4(0, 0, 0, 0);
                 v1 = ok ? x1 : make_uint4(0, 0, 0, 0);
+            }
+            if (edge) {
+                v0 = keep_keys(v0, kg, kv_begin, kv_end);
+                v1 = keep_keys(v1, kg + 8, kv_begin, kv_end);
             }
             o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, v0, v1);
         }
@@ -688,7 +705,8 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             if (c < VCH) {
                 const int d = c >> 3, k8 = (c & 7) * 8;
                 const bool ok = d < hd && live[k8 >> 4];
-                const uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < hd ? d : 0) * bs + (k8 & 15));
+                uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < hd ? d : 0) * bs + (k8 & 15));
+                if (kt0 < kv_begin || kt0 + 64 > kv_end) v = keep_keys(v, kt0 + k8, kv_begin, kv_end);
                 vreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
         }
@@ -763,6 +781,165 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     }
 }
 
+// Prefill when head_dim is exactly 64 or 128 and a page holds a multiple of 64 keys: a tile of 64
+// keys then lies in one page, 64 * HD contiguous elements of keys and as many of transposed values,
+// and travels from global memory straight into LDS (no registers in between, nothing to unpack),
+// two stages, the next tile's loads in flight while this one is multiplied, one barrier per tile.
+// A wave-load fills 1 KB: 1024 / (2 HD) key rows, or eight value rows of 64 keys.  Key row
+// 16 kb + 4 a + b of LDS holds key 16 a + 4 kb + b (what the MFMA operands want, see above; four
+// such keys follow each other in memory and in LDS alike), and inside a row the 16-byte chunks
+// stand at chunk ^ (row % 16) for rows of 256 bytes and chunk ^ ((row / 2) % 8) for rows of 128, which the loading
+// lanes achieve by choosing which chunk they fetch: the 16 rows an operand reads then fall on
+// distinct banks without padding.  Keys outside [kv_begin, kv_end) come along as whatever memory
+// holds: their scores are masked, and their values are zeroed in LDS before the product.
+typedef __attribute__((address_space(1))) const void* fx_global_ptr;
+typedef __attribute__((address_space(3))) void* fx_lds_ptr;
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
+    constexpr int KS = HD / 32, CB = HD / 16;
+    constexpr int NCH = HD / 8;                 // 16-byte chunks of a key row
+    constexpr int KROWS = 1024 / (2 * HD);      // key rows of a wave-load
+    constexpr int NLOAD = HD / 32;              // wave-loads per wave for the keys of a tile, and as many for the values
+    constexpr int TILE = 2 * 64 * HD;           // elements of a stage: keys, then values
+    __shared__ __attribute__((aligned(1024))) bf16 tiles[2 * TILE];
+    __shared__ int page_copy[PAGE_COPY];
+    const int per_xcd = (a.n_items * a.nh + 7) / 8;
+    const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (logical >= a.n_items * a.nh) return;
+    const int h = logical / a.n_items, item = a.n_items - 1 - logical % a.n_items;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, g = lane >> 4;
+    const int kvh = h / (a.nh / a.nkv);
+    const int tok_first = a.item_tok[item], n_all = a.item_n[item];
+    const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
+    const int bs = a.bs;
+    const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
+    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_end = pmax + 1;
+    const int tok0 = tok_first + 16 * wave, n = min(16, n_all - 16 * wave);
+    int lo = 1, hi = 0;
+    const bf16* qrow = nullptr;
+    if (li < n) {
+        hi = a.positions[tok0 + li];
+        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * HD;
+    }
+    int w_lo = 0x7fffffff, w_hi = -1;
+    int w_lo_max = 0x7fffffff, w_hi_min = -1;
+    if (n > 0) {
+        w_hi = a.positions[tok0 + n - 1];
+        w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
+        if (n == 16) {
+            w_hi_min = a.positions[tok0];
+            w_lo_max = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
+        }
+    }
+    const float c2 = a.scale * LOG2E;
+    float m = NEG_INF, l = 0.f;
+    f32x4_t o[CB];
+    bf16x8_t qf[KS];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) o[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < KS; ++u) {
+        const uint4 v = qrow ? *(const uint4*)(qrow + 32 * u + 8 * g) : make_uint4(0, 0, 0, 0);
+        qf[u] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    int first_blk, last_blk, unused;
+    page_slot(a, kv_begin, first_blk, unused);
+    page_slot(a, kv_end - 1, last_blk, unused);
+    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
+
+    // what this lane fetches in each of its wave-loads, relative to the tile's first key / value row 0
+    int k_src[NLOAD], v_src[NLOAD];
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+        const int j = wave + 4 * i;                          // wave-load j of HD / 8
+        const int row = KROWS * j + lane / NCH;              // LDS key row 16 kb + 4 a + b
+        const int key = 16 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
+        k_src[i] = key * HD + (((lane % NCH) ^ (NCH == 16 ? (row & 15) : ((row >> 1) & 7))) * 8);
+        const int d = 8 * j + (lane >> 3);                   // value row
+        v_src[i] = d * bs + (((lane & 7) ^ ((d >> 1) & 7)) * 8);
+    }
+    auto issue = [&](int kt0, int stage) {
+        int blk, slot;
+        page_slot(a, kt0, blk, slot);
+        const size_t page = (size_t)__builtin_amdgcn_readfirstlane(pl.page(blk));
+        const bf16* kbase = (const bf16*)a.k_pages + ((page * a.nkv + kvh) * bs + slot) * HD;
+        const bf16* vbase = (const bf16*)a.v_pages + (page * a.nkv + kvh) * HD * bs + slot;
+        bf16* st = tiles + stage * TILE;
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i)
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(kbase + k_src[i]), (fx_lds_ptr)(st + (wave + 4 * i) * 512), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i)
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(vbase + v_src[i]),
+                                             (fx_lds_ptr)(st + 64 * HD + (wave + 4 * i) * 512), 16, 0, 0);
+    };
+    // operands: key row 16 kb + li, chunk 4 u + g; value row 16 cb + li, chunks 2 g and 2 g + 1
+    const int k_at = li * HD, v_at = 64 * HD + li * 64;
+    const int ksw = NCH == 16 ? li : (li >> 1) & 7, vsw = (li >> 1) & 7;
+
+    const int kt_first = (kv_begin / 64) * 64;
+    issue(kt_first, 0);
+    int stage = 0;
+    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, stage ^= 1) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's part of the tile has landed
+        __builtin_amdgcn_s_barrier();                           // ... everyone's has, and the other stage is free
+        if (kt0 + 64 < kv_end) issue(kt0 + 64, stage ^ 1);
+        bf16* st = tiles + stage * TILE;
+        if (kt0 < kv_begin || kt0 + 64 > kv_end) {              // a tile at the edge: values of keys outside become zeros
+            for (int idx = tid; idx < HD * 64; idx += 256) {
+                const int d = idx >> 6, key = idx & 63;
+                if (kt0 + key < kv_begin || kt0 + key >= kv_end)
+                    st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
+            }
+            __builtin_amdgcn_s_barrier();
+        }
+        if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;           // nothing in this tile for this wave's rows
+        f32x4_t sc[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < KS; ++u) {
+                const bf16x8_t kf = *(const bf16x8_t*)(st + k_at + kb * 16 * HD + (((4 * u + g) ^ ksw) * 8));
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u], sc[kb], 0, 0, 0);
+            }
+        }
+        const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
+        uint4 p_lo, p_hi;
+        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi);
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+        float al[4] = {1.f, 1.f, 1.f, 1.f};
+        if (rescale) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const bf16* vr = st + v_at + cb * 16 * 64;
+            o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, *(const uint4*)(vr + (((2 * g) ^ vsw) * 8)),
+                            *(const uint4*)(vr + (((2 * g + 1) ^ vsw) * 8)));
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        const float lr = __shfl(l, row, 64);
+        if (row < n) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+                from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * HD + 16 * cb + li, o[cb][r] / lr);
+        }
+    }
+}
+
+static int g_no_direct = 0;     // measurement only: 1 keeps prefill on the kernel that stages tiles through registers
+FX_API void fx_attn_set_direct(int on) { g_no_direct = !on; }
+
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
     return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
@@ -797,7 +974,9 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
-        if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
+        if (bs % 64 == 0 && hd == 128 && !g_no_direct) attn_mfma_direct_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 64 && !g_no_direct) attn_mfma_direct_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
+        else if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 64) attn_mfma_block_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 128) attn_mfma_block_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
         else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);       // too large to stage in LDS

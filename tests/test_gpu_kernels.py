@@ -224,8 +224,9 @@ def paged_setup(dtype, nh, nkv, hd, bs, seq_lens, theta, rot, n_pages, seed=0):
         toks += [(s, p) for p in range(L)]
     T = len(toks)
     q, k, v = rnd(T, nh * hd, dtype=dtype), rnd(T, nkv * hd, dtype=dtype, seed=1), rnd(T, nkv * hd, dtype=dtype, seed=2)
-    k_pages = torch.zeros(n_pages, nkv, bs, hd, dtype=dtype, device=DEV)
-    v_pages = torch.zeros(n_pages, nkv, hd, bs, dtype=dtype, device=DEV)
+    # slots that no token is written to hold NaN: nothing may depend on what lies past a sequence's end
+    k_pages = torch.full((n_pages, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
+    v_pages = torch.full((n_pages, nkv, hd, bs), float("nan"), dtype=dtype, device=DEV)
     pos = torch.tensor([p for _, p in toks], dtype=torch.int32, device=DEV)
     seq = torch.tensor([s for s, _ in toks], dtype=torch.int32, device=DEV)
     q_rot = q.clone()
@@ -251,7 +252,8 @@ def test_rope_and_cache_write(dtype, nh, nkv, hd, bs, rot, theta):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,hd,bs,window", [(4, 4, 16, 16, 0), (3, 1, 32, 8, 16), (6, 3, 48, 4, 40), (2, 2, 128, 64, 0),
-                                                 (8, 2, 80, 16, 7), (4, 1, 256, 32, 100)])
+                                                 (8, 2, 80, 16, 7), (4, 1, 256, 32, 100), (4, 2, 64, 64, 50), (3, 1, 128, 128, 90),
+                                                 (2, 1, 64, 64, 0)])
 def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
     """Whole sequences through the tiled kernel, and their last tokens again through the decode
     kernel, against the plain attention on the same rotated, rounded q/k/v."""
