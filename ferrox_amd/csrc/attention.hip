@@ -795,14 +795,15 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
 typedef __attribute__((address_space(1))) const void* fx_global_ptr;
 typedef __attribute__((address_space(3))) void* fx_lds_ptr;
 
-template <int HD>
+template <int HD, int NS>
 __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
     constexpr int KS = HD / 32, CB = HD / 16;
     constexpr int NCH = HD / 8;                 // 16-byte chunks of a key row
     constexpr int KROWS = 1024 / (2 * HD);      // key rows of a wave-load
     constexpr int NLOAD = HD / 32;              // wave-loads per wave for the keys of a tile, and as many for the values
     constexpr int TILE = 2 * 64 * HD;           // elements of a stage: keys, then values
-    __shared__ __attribute__((aligned(1024))) bf16 tiles[2 * TILE];
+    static_assert(NS == 2 || NS == 3, "two or three stages");
+    __shared__ __attribute__((aligned(1024))) bf16 tiles[NS * TILE];
     __shared__ int page_copy[PAGE_COPY];
     const int per_xcd = (a.n_items * a.nh + 7) / 8;
     const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
@@ -883,11 +884,14 @@ __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
 
     const int kt_first = (kv_begin / 64) * 64;
     issue(kt_first, 0);
+    if (NS == 3 && kt_first + 64 < kv_end) issue(kt_first + 64, 1);
     int stage = 0;
-    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, stage ^= 1) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's part of the tile has landed
-        __builtin_amdgcn_s_barrier();                           // ... everyone's has, and the other stage is free
-        if (kt0 + 64 < kv_end) issue(kt0 + 64, stage ^ 1);
+    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, stage = (stage + 1 == NS ? 0 : stage + 1)) {
+        // this wave's part of the tile has landed (with three stages the next tile's loads may still fly)
+        if (NS == 3 && kt0 + 64 < kv_end) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLOAD) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                           // ... everyone's has, and the stage read last is free
+        if (kt0 + 64 * (NS - 1) < kv_end) issue(kt0 + 64 * (NS - 1), (stage + NS - 1) % NS);
         bf16* st = tiles + stage * TILE;
         if (kt0 < kv_begin || kt0 + 64 > kv_end) {              // a tile at the edge: values of keys outside become zeros
             for (int idx = tid; idx < HD * 64; idx += 256) {
@@ -937,8 +941,8 @@ __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
     }
 }
 
-static int g_no_direct = 0;     // measurement only: 1 keeps prefill on the kernel that stages tiles through registers
-FX_API void fx_attn_set_direct(int on) { g_no_direct = !on; }
+static int g_direct = 2;     // measurement only: 0 keeps prefill on the kernel that stages tiles through registers; 2, 3: stages
+FX_API void fx_attn_set_direct(int stages) { g_direct = stages; }
 
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
     return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
@@ -974,8 +978,9 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
-        if (bs % 64 == 0 && hd == 128 && !g_no_direct) attn_mfma_direct_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
-        else if (bs % 64 == 0 && hd == 64 && !g_no_direct) attn_mfma_direct_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
+        if (bs % 64 == 0 && hd == 128 && g_direct == 3) attn_mfma_direct_kernel<128, 3><<<grid_blocks, 256, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 128 && g_direct) attn_mfma_direct_kernel<128, 2><<<grid_blocks, 256, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 64 && g_direct) attn_mfma_direct_kernel<64, 2><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 64) attn_mfma_block_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 128) attn_mfma_block_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
