@@ -194,6 +194,7 @@ class CacheManager:
         self.slots = _SlotsView(self, n_slots)
         self._handles: dict = {}        # request name -> handle
         self._next = 0
+        self._decode_arrays = None      # what pack_decode keeps between steps
 
     # ---- requests --------------------------------------------------------
     def _handle(self, req) -> int:
@@ -265,6 +266,7 @@ class CacheManager:
         """Everything the request holds goes back; a second call does nothing."""
         h = self._handles.pop(req, None)
         if h is not None:
+            self._decode_arrays = None
             self._lib.fxc_release(self._h, h)
 
     # ---- the step's batch ----------------------------------------------------
@@ -308,6 +310,36 @@ class CacheManager:
                 msg = msg.replace(f"request {h} ", f"request {r!r} ").replace(f"request {h}:", f"request {r!r}:")
             raise ValueError(msg)
         return PackedStep(int(total), int(sizes[0]), int(sizes[1]), int(sizes[2]), starts[:n].tolist(), lens[:n].tolist())
+
+    def pack_decode(self, reqs: list, tokens: list, vocab: int, out_ptr: int, capacity: int, force_blocks: int) -> None:
+        """pack_step for the common step in which every request brings one token and wants its logits;
+        the arrays that do not change from step to step are kept from the last call."""
+        n = len(reqs)
+        key = tuple(reqs)
+        kept = self._decode_arrays
+        if kept is None or kept[0] != key:
+            handles = np.empty(n, dtype=np.int64)
+            for i, r in enumerate(reqs):
+                h = self._handles.get(r)
+                if h is None:
+                    raise ValueError(f"request {r!r} was not admitted")
+                handles[i] = h
+            kept = self._decode_arrays = (key, handles, np.ones(n, dtype=np.int32), np.arange(n + 1, dtype=np.int32),
+                                          np.zeros(n, dtype=np.int32), np.zeros(3, dtype=np.int32),
+                                          np.zeros(n, dtype=np.int32), np.zeros(n, dtype=np.int32))
+        _, handles, ones, want_start, want, sizes, starts, lens = kept
+        try:
+            toks = np.asarray(tokens, dtype=np.int32).reshape(-1)
+        except (OverflowError, TypeError, ValueError) as e:
+            raise ValueError(f"token ids must be integers: {e}") from None
+        if toks.size != n:
+            raise ValueError("one token per request")
+        ip = lambda a: a.ctypes.data_as(_I32P)
+        total = self._lib.fxc_pack_step(self._h, n, handles.ctypes.data_as(_I64P), ip(ones), ip(toks), ip(want_start),
+                                        ip(want), vocab, force_blocks, out_ptr, capacity, ip(sizes), ip(starts), ip(lens))
+        if total < 0:
+            self._decode_arrays = None
+            raise ValueError(self._core.error())
 
     def step_words(self, n_tokens: int, n_seqs: int, n_rows: int, max_blocks: int) -> int:
         return 3 * n_tokens + n_seqs + n_rows + len(self.groups) * n_seqs * max_blocks

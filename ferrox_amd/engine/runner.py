@@ -46,6 +46,7 @@ class DecodeGraph:
         dev = runner.device
         self.meta = torch.zeros(total, dtype=torch.int32, device=dev)
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self._host_ptr, self._host_words = self.host.data_ptr(), total
         self.copied = torch.cuda.Event()
         self.copied.record()
         self.graph = None
@@ -68,9 +69,13 @@ class DecodeGraph:
 
     def run(self, entries) -> torch.Tensor:
         self.copied.synchronize()                  # the last upload has left the staging buffer
-        self.runner.manager.pack_step([e.req for e in entries], [e.tokens for e in entries],
-                                      [e.want for e in entries], self.runner.vocab_size, self.host.data_ptr(),
-                                      self.host.numel(), force_blocks=self.max_blocks)
+        if all(e.want[0] == 0 for e in entries):
+            self.runner.manager.pack_decode([e.req for e in entries], [e.tokens[0] for e in entries],
+                                            self.runner.vocab_size, self._host_ptr, self._host_words, self.max_blocks)
+        else:
+            self.runner.manager.pack_step([e.req for e in entries], [e.tokens for e in entries],
+                                          [e.want for e in entries], self.runner.vocab_size, self._host_ptr,
+                                          self._host_words, force_blocks=self.max_blocks)
         self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
         model, caches = self.runner.model, self.runner.storage.caches

@@ -170,3 +170,27 @@ def test_pack_step_refuses_what_does_not_fit():
         m.extend("a", 20)
         _pack(m, ["a"], [[1, 2]], [[1]], force=2)
     m.check_invariants()
+
+
+def test_pack_decode_writes_what_pack_step_writes():
+    import numpy as np
+    m = CacheManager({FULL: None, WIN: 16}, 16, block_size=8, n_slots=4)
+    for r, n in (("a", 21), ("b", 40), ("c", 9)):
+        m.admit(r)
+        m.extend(r, n)
+    for reqs, toks in ((["b", "a", "c"], [7, 1, 3]), (["b", "a", "c"], [9, 9, 2]), (["c", "b"], [5, 6])):
+        want, buf = _pack(m, reqs, [[t] for t in toks], [[0]] * len(reqs), force=6)
+        got = np.full(4096, -7, dtype=np.int32)
+        m.pack_decode(reqs, toks, 100, got.ctypes.data, 4096, 6)
+        assert (got == buf).all()
+    m.release("b")                     # what was kept for (c, b) must not outlive b
+    m.admit("b")
+    m.extend("b", 3)
+    want, buf = _pack(m, ["c", "b"], [[5], [6]], [[0], [0]], force=6)
+    got = np.full(4096, -7, dtype=np.int32)
+    m.pack_decode(["c", "b"], [5, 6], 100, got.ctypes.data, 4096, 6)
+    assert (got == buf).all()
+    with pytest.raises(ValueError, match="vocabulary"):
+        m.pack_decode(["c", "b"], [5, 100], 100, got.ctypes.data, 4096, 6)
+    with pytest.raises(ValueError, match="not admitted"):
+        m.pack_decode(["zz"], [5], 100, got.ctypes.data, 4096, 6)
