@@ -348,49 +348,62 @@ __device__ __forceinline__ void wait_loads_but() {
 }
 
 // The K loop of one wave for NA active row blocks (blocks wm, wm+2, ... of the tile).
-template <int NA, int MT, int NT, int TM, int TN, int NS>
+template <int NA, int MT, int NT, int TM, int TN, int NSA, int NSB>
 __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* const (&a_src)[TM / 64],
                                             const bf16* const (&b_src)[TN / 64], bf16* stages, int K, int wave,
                                             int a_off, int b_off, int sw, int kq, long kb_stride) {
+    static_assert(NSA >= 2 && NSB >= NSA, "the weights' ring is at least as deep as the rows'");
     const int koff0 = (kq ^ sw) * 8, koff1 = ((4 + kq) ^ sw) * 8;
-    constexpr int NLA = TM / 64, NLB = TN / 64, L = NLA + NLB;     // wave-loads per wave and step
-    constexpr int STAGE = (TM + TN) * 64;
+    constexpr int NLA = TM / 64, NLB = TN / 64;     // wave-loads per wave and step
+    bf16* const ring_b = stages + NSA * TM * 64;
     const int nk = K >> 6;
-    auto issue = [&](int kt) {
-        const int k0 = min(kt, nk - 1) << 6;         // past the end: a tile nobody reads, so that counts stay even
-        const size_t w0 = kb_stride ? (size_t)min(kt, nk - 1) * kb_stride : (size_t)k0;
-        bf16* st = stages + (kt % NS) * STAGE;
+    // past the end: a tile nobody reads, so that the counts of loads in flight stay even
+    auto issue_a = [&](int kt) {
+        const int k0 = min(kt, nk - 1) << 6;
+        bf16* st = stages + (kt % NSA) * (TM * 64);
 #pragma unroll
         for (int i = 0; i < NLA; ++i)
             __builtin_amdgcn_global_load_lds((fx_global_ptr)(a_src[i] + k0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 0);
+    };
+    auto issue_b = [&](int kt) {
+        const size_t w0 = kb_stride ? (size_t)min(kt, nk - 1) * kb_stride : (size_t)(min(kt, nk - 1) << 6);
+        bf16* st = ring_b + (kt % NSB) * (TN * 64);
 #pragma unroll
         for (int i = 0; i < NLB; ++i)
-            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0),
-                                             (fx_lds_ptr)(st + TM * 64 + (wave + 8 * i) * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 0);
     };
+    // Each step issues the rows of step kt + NSA - 1, then the weights of step kt + NSB - 1.  Weights come from
+    // memory and nothing reads them twice, so their ring may be deeper: more of them are on their way at a time.
 #pragma unroll
-    for (int p = 0; p < NS - 1; ++p) issue(p);
+    for (int p = 0; p < NSB - 1; ++p) {
+        if (p >= NSB - NSA) issue_a(p - (NSB - NSA));
+        issue_b(p);
+    }
     for (int kt = 0; kt < nk; ++kt) {
-        wait_loads_but<(NS - 2) * L>();        // this wave's part of step kt has landed
-        __builtin_amdgcn_s_barrier();          // ... everyone's has, and the stage of step kt-1 is free
-        issue(kt + NS - 1);
-        const bf16* base = stages + (kt % NS) * STAGE;
+        // this wave's part of step kt has landed: what may still be on its way are the loads of the NSA - 2
+        // steps issued since the rows of step kt, and the weights issued right after those rows
+        wait_loads_but<(NSA - 2) * (NLA + NLB) + (NSB > NSA ? NLB : 0)>();
+        __builtin_amdgcn_s_barrier();          // ... everyone's has, and the stages of step kt-1 are free
+        issue_a(kt + NSA - 1);
+        issue_b(kt + NSB - 1);
+        const bf16* base_a = stages + (kt % NSA) * (TM * 64);
+        const bf16* base_b = ring_b + (kt % NSB) * (TN * 64);
         // 2*NA units of one operand of rows against NT operands of weights; the rows' operands are
         // read from LDS a few units ahead of the products that use them
         constexpr int U = 2 * NA, D = U > 3 ? 3 : U - 1;
         bf16x8_t bfr[2][NT], fr[U];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) bfr[0][j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff0);
+        for (int j = 0; j < NT; ++j) bfr[0][j] = *(const bf16x8_t*)(base_b + b_off + j * 16 * 64 + koff0);
 #pragma unroll
         for (int u = 0; u < D; ++u)
-            fr[u] = *(const bf16x8_t*)(base + a_off + (u % NA) * 32 * 64 + ((u / NA) ? koff1 : koff0));
+            fr[u] = *(const bf16x8_t*)(base_a + a_off + (u % NA) * 32 * 64 + ((u / NA) ? koff1 : koff0));
         static_for(std::make_integer_sequence<int, U>{}, [&](auto uc) {
             constexpr int u = decltype(uc)::value;
             if (u + D < U)
-                fr[u + D] = *(const bf16x8_t*)(base + a_off + ((u + D) % NA) * 32 * 64 + (((u + D) / NA) ? koff1 : koff0));
+                fr[u + D] = *(const bf16x8_t*)(base_a + a_off + ((u + D) % NA) * 32 * 64 + (((u + D) / NA) ? koff1 : koff0));
             if (u == 0) {
 #pragma unroll
-                for (int j = 0; j < NT; ++j) bfr[1][j] = *(const bf16x8_t*)(base + b_off + j * 16 * 64 + koff1);
+                for (int j = 0; j < NT; ++j) bfr[1][j] = *(const bf16x8_t*)(base_b + b_off + j * 16 * 64 + koff1);
             }
             __builtin_amdgcn_sched_barrier(0);      // the reads above stay ahead of the products below
 #pragma unroll
@@ -402,7 +415,7 @@ __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* 
     wait_loads_but<0>();                       // the loads past the end, before the block leaves
 }
 
-template <int TMB, int TN, int NS, bool DUAL, int EPI>
+template <int TMB, int TN, int NS, bool DUAL, int EPI, int NSA = NS>
 __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     constexpr int TM = TMB * 16;
     constexpr int MT = TMB / 2;            // row blocks per wave
@@ -411,11 +424,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     constexpr int OUT_TN = DUAL ? TN / 2 : TN;
     constexpr int NLA = TM / 64, NLB = TN / 64;   // wave-loads (8 rows each) per wave and K step
     static_assert(TM % 64 == 0 && TN % 64 == 0, "eight waves load 64 rows at a time");
-    __shared__ __attribute__((aligned(1024))) bf16 stages[NS * (TM + TN) * 64];
+    __shared__ __attribute__((aligned(1024))) bf16 stages[(NSA * TM + NS * TN) * 64];    // the rows' ring, then the weights'
 
     // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), each with an L2 of its own.  Plain: an XCD
-    // works through a contiguous range of column tiles, rows fastest, so the weights of those columns stay in
-    // its L2.  Grouped: XCD x takes the row tiles x, x + 8, ... and runs through the column tiles of each, so an
+    // works through a contiguous range of the tiles in an order that keeps neighbours in rows and columns
+    // together, so the operands of the tiles it has at a time stay in its L2.  Grouped: XCD x takes the row tiles x, x + 8, ... and runs through the column tiles of each, so an
     // expert's rows are fetched once and stay in its L2 while its weights, which nothing reads twice, stream by
     // (the row tiles past the last expert are empty; dealing them out in turn spreads them over the XCDs).
     int row_tile, col_tile;
@@ -428,8 +441,12 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
         const int per_xcd = (g.n_col_tiles * g.n_row_tiles + 7) / 8;
         const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
         if (logical >= g.n_col_tiles * g.n_row_tiles) return;
-        row_tile = logical % g.n_row_tiles;
-        col_tile = logical / g.n_row_tiles;
+        // bands of 8 row tiles, rows fastest inside a band: the 32 tiles that an XCD works on at a time are
+        // 8 rows x 4 columns, so 12 operand tiles serve 32 products
+        const int band = logical / (8 * g.n_col_tiles), rem = logical % (8 * g.n_col_tiles);
+        const int band_rows = min(8, g.n_row_tiles - band * 8);
+        row_tile = band * 8 + rem % band_rows;
+        col_tile = rem / band_rows;
     }
     int r0, r_end, expert;
     locate_rows<TM>(g, row_tile, r0, r_end, expert);
@@ -438,7 +455,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     const int rows_here = min(TM, r_end - r0);
     const int nblk = (rows_here + 15) >> 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
+    // waves w and w + 4 share a SIMD: one of each half of the rows, so that a tile with few rows loads the SIMDs evenly
+    const int wm = wave >> 2, wn = wave & 3;
     const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
 
     // what this lane fetches in each of its wave-loads: row 8*j + lane/8 of the tile, chunk (lane%8) ^ ((row/2)%8)
@@ -469,10 +487,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     const int sw = (lane & 15) >> 1, kq = lane >> 4;
-    const int a_off = (wm * 16 + (lane & 15)) * 64, b_off = (TM + wn * WN + (lane & 15)) * 64;
+    const int a_off = (wm * 16 + (lane & 15)) * 64, b_off = (wn * WN + (lane & 15)) * 64;
     const int na = (nblk - wm + 1) >> 1;         // this wave's active row blocks
 #define FX_LOOP(NA) \
-    wide_k_loop<NA, MT, NT, TM, TN, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride)
+    wide_k_loop<NA, MT, NT, TM, TN, NSA, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride)
     if (na > 3 * MT / 4) FX_LOOP(MT);
     else if (na > MT / 2) FX_LOOP(3 * MT / 4);
     else if (na > MT / 4) FX_LOOP(MT / 2);
@@ -821,18 +839,21 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 static int g_skinny_four = 1024;   // blocks that four-set tiles must still give; 0: never four sets (measurement)
 FX_API void fx_gemm_set_skinny_four(int blocks) { g_skinny_four = blocks; }
 static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
-FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; }
+static int g_wide_force = 0;   // measurement only: 256, 192, 128 or 64 picks that wide tile whatever the sizes
+FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; g_wide_force = on > 1 ? on : 0; }
 
-template <int TMB, int TN, int NS>
+template <int TMB, int TN, int NS, int NSA = NS>
 static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
     g.n_col_tiles = ceil_div(g.N, epi == EPI_SILU_MUL ? TN / 2 : TN);
     g.n_row_tiles = m_tiles;
     dim3 grid(g.expert_offsets ? 8 * ceil_div(m_tiles, 8) * g.n_col_tiles : 8 * ceil_div((long)g.n_col_tiles * m_tiles, 8));
     switch (epi) {
-        case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE><<<grid, 512, 0, s>>>(g); break;
-        case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32><<<grid, 512, 0, s>>>(g); break;
-        case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID><<<grid, 512, 0, s>>>(g); break;
-        default: gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_SILU_MUL><<<grid, 512, 0, s>>>(g); break;
+        case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE, NSA><<<grid, 512, 0, s>>>(g); break;
+        case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32, NSA><<<grid, 512, 0, s>>>(g); break;
+        case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID, NSA><<<grid, 512, 0, s>>>(g); break;
+        default:
+            if constexpr (TN % 128 == 0) gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_SILU_MUL, NSA><<<grid, 512, 0, s>>>(g);
+            break;
     }
 }
 
@@ -961,8 +982,19 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
             const long t = tiles(tm, tn);
             return quality * (double)t / (double)(ceil_div(t, 256) * 256L);
         };
-        const double s256 = score(256, 256, 1.0), s128 = score(256, 128, 0.85), s64 = score(128, 128, 0.7);
-        if (s256 >= s128 && s256 >= s64)
+        double s256 = score(256, 256, 1.0), s192 = dual ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
+               s64 = score(128, 128, 0.7);
+        if (g_wide_force) {
+            s256 = g_wide_force == 256; s192 = g_wide_force == 192 && !dual; s128 = g_wide_force == 128; s64 = 0.5 * (g_wide_force == 64);
+        }
+        // an expert's share of up to 192 rows: the product streams the weights once and multiplies little, so it
+        // is bound by how many of them are on their way; a ring of three weight tiles beside two of the rows
+        const bool few_rows = expert_offsets && (g_wide_force ? g_wide_force == 12 : per_group <= 176);
+        if (few_rows)
+            launch_wide<12, 256, 3, 2>(g, epi, M / 192 + nonempty, s);
+        else if (s192 > s256 && s192 >= s128 && s192 >= s64)
+            launch_wide<16, 192, 2>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);
+        else if (s256 >= s128 && s256 >= s64)
             launch_wide<16, 256, 2>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);
         else if (s128 >= s64)
             launch_wide<16, 128, 3>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);

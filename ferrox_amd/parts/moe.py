@@ -17,7 +17,7 @@ from .linear import matmul, same_dtype
 from .mlp import SwiGLU
 
 GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
-OVERLAP_MAX_TOKENS = 256     # up to here the shared expert runs beside the routed ones on a second stream
+OVERLAP_MAX_TOKENS = 8192    # up to here the shared expert runs beside the routed ones on a second stream
 _side_streams: dict = {}
 
 
@@ -130,8 +130,9 @@ class SparseMoE(FeedForward):
             return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
         if overlap:
-            # few tokens: both halves are bound by reading weights, so the shared expert streams its
-            # weights on a second stream while the routed experts run; its output joins in the combine
+            # the shared expert runs on a second stream beside the router and the routed experts, and its output
+            # joins in the combine: with few tokens both halves wait for weights from memory, with many the
+            # blocks of one fill the CUs that the last round of the other's tiles leaves idle
             main, side = torch.cuda.current_stream(), side_stream(x.device)
             fork, join = torch.cuda.Event(), torch.cuda.Event()
             fork.record(main)

@@ -44,6 +44,59 @@ def test_gemm_plain_and_epilogues(dtype, M, N, K):
     close(h, h0.double() + ref * scale.double()[:, None], dtype, "residual")
 
 
+@pytest.mark.parametrize("tile", [256, 192, 128, 64])
+@pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
+def test_gemm_every_wide_tile(tile, M, N, K):
+    """The many-row kernel picks its tile by the sizes; here each tile shape is made to run the same products."""
+    from ferrox_amd import ops
+    from ferrox_amd.csrc.build import load_library
+    lib = load_library("gemm")
+    dtype = torch.bfloat16
+    a, w, bias = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1), rnd(N, dtype=dtype, seed=2)
+    ref = a.double() @ w.double().T
+    h = rnd(M, N, seed=3)
+    h0 = h.clone()
+    lib.fx_gemm_set_wide(tile)
+    try:
+        got = ops.gemm(a, w, bias=bias)
+        ops.gemm(a, w, epilogue=ops.EPI_RESID, out=h)
+        w2 = rnd(2 * N, K, dtype=dtype, seed=4, scale=0.5)
+        act = ops.gemm(a, w2, epilogue=ops.EPI_SILU_MUL)
+    finally:
+        lib.fx_gemm_set_wide(1)
+    close(got, ref + bias.double(), dtype, "store+bias")
+    close(h, h0.double() + ref, dtype, "residual")
+    close(act, plain.silu(a.double() @ w2[:N].double().T) * (a.double() @ w2[N:].double().T), dtype, "silu(gate)*up")
+
+
+@pytest.mark.parametrize("tile", [12, 256])
+def test_grouped_gemm_tiles_agree(tile):
+    """An expert's rows in tiles of 192 (weights three steps deep) and of 256 give the same sums."""
+    from ferrox_amd import ops
+    from ferrox_amd.csrc.build import load_library
+    lib = load_library("gemm")
+    T, E, k, I, H = 900, 6, 2, 64, 256
+    x = rnd(T, H, dtype=torch.bfloat16)
+    w_gu = rnd(E, 2 * I, H, dtype=torch.bfloat16, seed=1, scale=0.3)
+    g = torch.Generator().manual_seed(7)
+    # uneven shares: expert 0 gets a third of all pairs, more than one tile of either kind
+    first = torch.where(torch.rand(T, generator=g) < 0.66, 0, 1)
+    ids = torch.stack([first, 2 + torch.randint(0, E - 2, (T,), generator=g)], dim=1).to(torch.int32).to(DEV)
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
+    lib.fx_gemm_set_wide(tile)
+    try:
+        act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    finally:
+        lib.fx_gemm_set_wide(1)
+    xs = x.double()[sorted_token.long()]
+    off = offsets.cpu().tolist()
+    assert off[1] - off[0] > 256
+    for e in range(E):
+        r = slice(off[e], off[e + 1])
+        want = plain.silu(xs[r] @ w_gu[e, :I].double().T) * (xs[r] @ w_gu[e, I:].double().T)
+        close(act[r], want, torch.bfloat16, f"expert {e}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,I,K", [(1, 32, 64), (7, 48, 96), (40, 100, 72), (200, 176, 256), (300, 100, 128),
                                     (257, 129, 64)])
@@ -56,7 +109,8 @@ def test_gemm_gate_up(dtype, M, I, K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,E,k,I,H", [(1, 4, 2, 32, 64), (9, 6, 3, 48, 96), (70, 5, 1, 40, 120), (300, 8, 2, 64, 128),
-                                        (64, 3, 2, 24, 72), (520, 4, 3, 128, 256), (700, 3, 2, 200, 192)])
+                                        (64, 3, 2, 24, 72), (520, 4, 3, 128, 256), (700, 3, 2, 200, 192),
+                                        (330, 4, 2, 128, 320), (1300, 16, 2, 64, 192)])
 def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     """router ids -> align -> grouped gate/up -> grouped down -> combine, against per-token loops."""
     from ferrox_amd import ops
