@@ -808,7 +808,10 @@ __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
     const int per_xcd = (a.n_items * a.nh + 7) / 8;
     const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (logical >= a.n_items * a.nh) return;
-    const int h = logical / a.n_items, item = a.n_items - 1 - logical % a.n_items;
+    // later items of a prompt see more keys: even heads run them last to first, odd heads first to last, so that
+    // the blocks that come to share a CU (two fit, handed out in turn) have about the same work together
+    const int h = logical / a.n_items;
+    const int item = (h & 1) ? logical % a.n_items : a.n_items - 1 - logical % a.n_items;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, g = lane >> 4;
     const int kvh = h / (a.nh / a.nkv);
