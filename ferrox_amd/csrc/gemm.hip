@@ -14,6 +14,7 @@
 // Dual mode: two weight matrices (gate, up) are multiplied at once and the
 // epilogue stores silu(gate) * up  (ferrox-moe/src/lib.rs:655-658).
 #include "common.h"
+#include <type_traits>
 #include <utility>
 
 FX_DEFINE_LAST_ERROR()
@@ -544,15 +545,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 // W is the A operand: the accumulator of lane (m = lane%16, g) holds
 // C[m][n0 + 4g + r], r = 0..3.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ uint4 load16(const bf16* row, int k, int K) {
-    return (row && k < K) ? *(const uint4*)(row + k) : make_uint4(0, 0, 0, 0);
-}
-// the same from weights stored in slabs of 64 k (kb_stride elements apart; 0: plain rows)
-__device__ __forceinline__ uint4 load16w(const bf16* row, int k, int K, long kb_stride) {
-    if (!row || k >= K) return make_uint4(0, 0, 0, 0);
-    return kb_stride ? *(const uint4*)(row + (size_t)(k >> 6) * kb_stride + (k & 63)) : *(const uint4*)(row + k);
-}
-
 // NORM: the rows of A are float32 and are normed on the way in, y = x * rsqrt(mean(x^2) + eps) * w
 // (ferrox-core/src/matmul.rs:62-69): x * w is rounded to bfloat16 and multiplied, the sums of
 // squares that the waves gather over their parts of K are added up, and the product is scaled by
@@ -596,18 +588,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     for (int a = 0; a < NW; ++a) {
         const int n = DUAL ? n0 + (a >> 1) * 16 + li : n0 + a * 16 + li;
         const bool up = DUAL && (a & 1);
+        // rows past the end repeat the last one: their columns are never stored
+        const int nc = min(n, g.N - 1);
         if (g.kb_stride)
-            wrow[a] = (n < g.N) ? Wbase + ((size_t)n + (up ? g.up_offset / g.K : 0)) * 64 : nullptr;
+            wrow[a] = Wbase + ((size_t)nc + (up ? g.up_offset / g.K : 0)) * 64;
         else
-            wrow[a] = (n < g.N) ? Wbase + (size_t)n * g.K + (up ? g.up_offset : 0) : nullptr;
+            wrow[a] = Wbase + (size_t)nc * g.K + (up ? g.up_offset : 0);
     }
+    const size_t slab = g.kb_stride ? (size_t)g.kb_stride : 64;     // element (row, k) is at row + (k / 64) * slab + k % 64
     const bf16* xrow[MT];       // NORM: float rows, kept under the same name
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = r0 + mt * 16 + li;
         const bool live = pairs ? pair_a >= 0 : m < r_end;
         const size_t off = !live ? 0 : (size_t)(pairs ? pair_a : (g.a_rows ? g.a_rows[m] : m)) * g.lda;
-        xrow[mt] = live ? (NORM ? (const bf16*)((const float*)g.A + off) : (const bf16*)g.A + off) : nullptr;
+        // a dead row reads the first row of A instead: its products land in rows that are never stored
+        xrow[mt] = NORM ? (live ? (const bf16*)((const float*)g.A + off) : nullptr) : (const bf16*)g.A + off;
     }
     f32x4_t acc[MT][NW];
 #pragma unroll
@@ -618,57 +614,94 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     const int n_super = (g.K + 127) / 128;
     const int per = (n_super + WAVES - 1) / WAVES;
     const int s_end = min(n_super, (wave + 1) * per);
-    constexpr int UN = (MT * NW <= 4 && !NORM) ? 2 : 1;     // pieces whose loads are issued together
-    for (int s = wave * per; s < s_end; s += UN) {
-        uint4 w[UN][NW][4], x[UN][MT][4];
+    // One piece: its loads (four per set of weight rows and per row tile), then its products.  FULL: the piece
+    // lies inside K, so every load is unconditional and the compiler can count the loads in flight.
+    auto load_piece = [&](auto full, int sp, uint4 (&w)[NW][4], uint4 (&x)[MT][4]) {
+        constexpr bool FULL = decltype(full)::value;
+        const int kb = sp * 128 + grp * 8;     // load u of this lane: k = kb + 32u .. +7
 #pragma unroll
-        for (int p = 0; p < UN; ++p) {
-            const int kb = (s + p) * 128 + grp * 8;     // load u of this lane: k = kb + 32u .. +7
-            const bool live = s + p < s_end;
+        for (int u = 0; u < 4; ++u) {
+            const int k = kb + 32 * u;
+            const bool kin = FULL || k < g.K;
+            const size_t woff = (size_t)(k >> 6) * slab + (k & 63);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-#pragma unroll
-                for (int a = 0; a < NW; ++a) w[p][a][u] = load16w(live ? wrow[a] : nullptr, kb + 32 * u, g.K, g.kb_stride);
-                if constexpr (NORM) {
-                    const int k = kb + 32 * u;
-                    const bool kin = live && k < g.K;
-                    float gv[8];
-                    if (g.norm_dtype == FX_F32) {
-                        load8f((const float*)g.norm_w + k, kin, gv);
-                    } else {
-                        const uint4 gw = kin ? *(const uint4*)((const bf16*)g.norm_w + k) : make_uint4(0, 0, 0, 0);
-                        gv[0] = __uint_as_float(gw.x << 16); gv[1] = __uint_as_float(gw.x & 0xffff0000u);
-                        gv[2] = __uint_as_float(gw.y << 16); gv[3] = __uint_as_float(gw.y & 0xffff0000u);
-                        gv[4] = __uint_as_float(gw.z << 16); gv[5] = __uint_as_float(gw.z & 0xffff0000u);
-                        gv[6] = __uint_as_float(gw.w << 16); gv[7] = __uint_as_float(gw.w & 0xffff0000u);
-                    }
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        float xv[8];
-                        load8f((const float*)xrow[mt] + k, kin && xrow[mt], xv);
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) ss[mt] += xv[i] * xv[i];
-                        x[p][mt][u] = make_uint4(pack_bf16(xv[0] * gv[0], xv[1] * gv[1]), pack_bf16(xv[2] * gv[2], xv[3] * gv[3]),
-                                                 pack_bf16(xv[4] * gv[4], xv[5] * gv[5]), pack_bf16(xv[6] * gv[6], xv[7] * gv[7]));
-                    }
+            for (int a = 0; a < NW; ++a) w[a][u] = kin ? *(const uint4*)(wrow[a] + woff) : make_uint4(0, 0, 0, 0);
+            if constexpr (NORM) {
+                float gv[8];
+                if (g.norm_dtype == FX_F32) {
+                    load8f((const float*)g.norm_w + k, kin, gv);
                 } else {
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) x[p][mt][u] = load16(live ? xrow[mt] : nullptr, kb + 32 * u, g.K);
+                    const uint4 gw = kin ? *(const uint4*)((const bf16*)g.norm_w + k) : make_uint4(0, 0, 0, 0);
+                    gv[0] = __uint_as_float(gw.x << 16); gv[1] = __uint_as_float(gw.x & 0xffff0000u);
+                    gv[2] = __uint_as_float(gw.y << 16); gv[3] = __uint_as_float(gw.y & 0xffff0000u);
+                    gv[4] = __uint_as_float(gw.z << 16); gv[5] = __uint_as_float(gw.z & 0xffff0000u);
+                    gv[6] = __uint_as_float(gw.w << 16); gv[7] = __uint_as_float(gw.w & 0xffff0000u);
                 }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    float xv[8];
+                    load8f((const float*)xrow[mt] + k, kin && xrow[mt], xv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) ss[mt] += xv[i] * xv[i];
+                    x[mt][u] = make_uint4(pack_bf16(xv[0] * gv[0], xv[1] * gv[1]), pack_bf16(xv[2] * gv[2], xv[3] * gv[3]),
+                                          pack_bf16(xv[4] * gv[4], xv[5] * gv[5]), pack_bf16(xv[6] * gv[6], xv[7] * gv[7]));
+                }
+            } else {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) x[mt][u] = kin ? *(const uint4*)(xrow[mt] + k) : make_uint4(0, 0, 0, 0);
             }
         }
+    };
+    auto multiply_piece = [&](const uint4 (&w)[NW][4], const uint4 (&x)[MT][4]) {
 #pragma unroll
-        for (int p = 0; p < UN; ++p)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int u = 0; u < 4; ++u) {
+                const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[mt][u]);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[p][mt][u]);
-#pragma unroll
-                    for (int a = 0; a < NW; ++a)
-                        acc[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[p][a][u]), xb,
-                                                                            acc[mt][a], 0, 0, 0);
-                }
+                for (int a = 0; a < NW; ++a)
+                    acc[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[a][u]), xb, acc[mt][a], 0, 0, 0);
+            }
+    };
+    constexpr std::true_type whole{};
+    constexpr std::false_type masked{};
+    const int s_whole = min(s_end, g.K / 128);       // pieces before this one lie inside K
+    int sp = wave * per;
+    // Few accumulators leave registers for two pieces: the loads of the next piece are then issued before the
+    // products of this one, so a wave always has a piece on its way from memory.  Each product follows the
+    // loads issued after its own in straight-line code.
+    constexpr bool TWO = MT * NW <= 4 && !NORM;
+    if constexpr (TWO) {
+        if (sp < s_whole) {
+            uint4 w0[NW][4], x0[MT][4], w1[NW][4], x1[MT][4];
+            load_piece(whole, sp, w0, x0);
+            for (; sp + 2 < s_whole; sp += 2) {
+                load_piece(whole, sp + 1, w1, x1);
+                multiply_piece(w0, x0);
+                load_piece(whole, sp + 2, w0, x0);
+                multiply_piece(w1, x1);
+            }
+            if (sp + 1 < s_whole) {
+                load_piece(whole, sp + 1, w1, x1);
+                multiply_piece(w0, x0);
+                multiply_piece(w1, x1);
+                sp += 2;
+            } else {
+                multiply_piece(w0, x0);
+                sp += 1;
+            }
+        }
+    } else {
+        for (; sp < s_whole; ++sp) {
+            uint4 w[NW][4], x[MT][4];
+            load_piece(whole, sp, w, x);
+            multiply_piece(w, x);
+        }
+    }
+    for (; sp < s_end; ++sp) {          // the piece that K ends in
+        uint4 w[NW][4], x[MT][4];
+        load_piece(masked, sp, w, x);
+        multiply_piece(w, x);
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
