@@ -869,8 +869,10 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 #undef FX_TILED
 }
 
-static int g_skinny_four = 1024;   // blocks that four-set tiles must still give; 0: never four sets (measurement)
+static int g_skinny_four = 0;      // blocks that four-set tiles must still give; 0: never four sets (two leave registers for more waves)
 FX_API void fx_gemm_set_skinny_four(int blocks) { g_skinny_four = blocks; }
+static int g_skinny_nw = 0, g_skinny_eight = -1;        // measurement only: sets per wave (1, 2, 4) and waves (0: four, 1: eight) whatever the sizes
+FX_API void fx_gemm_set_skinny(int nw, int eight) { g_skinny_nw = nw; g_skinny_eight = eight; }
 static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
 static int g_wide_force = 0;   // measurement only: 256, 192, 128 or 64 picks that wide tile whatever the sizes
 FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; g_wide_force = on > 1 ? on : 0; }
@@ -989,13 +991,15 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16 + n_always
                                      : M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
         const bool dual = epi == EPI_SILU_MUL;
-        // two sets of weight rows per wave share the activations they multiply: worth it when
-        // there are blocks enough either way
-        int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 2048) ? 2 : 1;
-        // four sets when even then there are blocks enough: a block's fixed work is spread over more weights
+        // two sets of weight rows per wave share the activations they multiply and halve the blocks' fixed
+        // work; one set when that would leave too few blocks to keep the memory busy, or when a row or two meet
+        // so many weight rows that the blocks are plenty either way (measured on the sizes of the engine)
+        int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 160) ? 2 : 1;
+        if (!dual && (norm_w || (M <= 2 && (long)ceil_div(N, 16) * m_tiles >= 4096))) nw = 1;
+        // four sets: measurement only (they leave registers for two waves per SIMD, which streams less)
         if (mt == 1 && !norm_w && g_skinny_four && (long)ceil_div(N, dual ? 32 : 64) * m_tiles >= g_skinny_four) nw = 4;
-        const long blocks = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles;
-        const bool eight = blocks < 1024 && mt * nw <= 4 && K >= 2048;
+        if (g_skinny_nw && !norm_w && (g_skinny_nw < 4 || mt == 1) && !(dual && g_skinny_nw == 1)) nw = g_skinny_nw;
+        const bool eight = g_skinny_eight > 0 && mt * nw <= 4;      // measurement only: four waves stream as well
         launch_skinny(g, epi, mt, eight, nw, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;

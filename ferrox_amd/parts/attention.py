@@ -93,8 +93,9 @@ class PagedAttention(Mixer):
                 "v": (self.n_kv_heads, self.head_dim, block_size)}
 
     def forward_from_residual(self, norm, ctx, cache, residual) -> bool:
-        """Few tokens: the norm is applied inside the q/k/v product."""
-        if (ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm"
+        """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
+        more, every block's reading and norming of all rows costs more than the norm kernel)."""
+        if (ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm" or residual.shape[0] > 16
                 or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
         qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=(norm.weight, norm.eps))
