@@ -347,6 +347,38 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
         close(out2[last], ref[last], dtype, f"decode attention chunk {chunk}")
 
 
+@pytest.mark.parametrize("hd,bs,window", [(64, 16, 0), (64, 64, 0), (128, 64, 40000), (32, 16, 9000)])
+def test_attention_over_more_pages_than_a_block_copies(hd, bs, window):
+    """A sequence of more than 1024 pages (the kernels copy that many page ids into LDS and read the rest of
+    the table from memory): its last 64 tokens as a block of queries, and its last token alone."""
+    from ferrox_amd import ops
+    nh, nkv, dtype = 2, 1, torch.bfloat16
+    L = bs * 1030 + 5
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, [L], 1e6, hd, 1040)
+    scale = 1.0 / math.sqrt(hd)
+    kp, vp, tab = k_pages.double().cpu(), v_pages.double().cpu(), table.cpu()[0].long()
+    ks = kp[tab].permute(0, 2, 1, 3).reshape(-1, nkv, hd)[:L]                  # [L, nkv, hd]
+    vs = vp[tab].permute(0, 3, 1, 2).reshape(-1, nkv, hd)[:L]
+    qs = q_rot[L - 64:].double().cpu().reshape(64, nh, hd)
+    ref = torch.zeros(64, nh, hd, dtype=torch.float64)
+    for i in range(64):
+        p = L - 64 + i
+        lo = max(0, p - window + 1) if window else 0
+        for h in range(nh):
+            sc = (ks[lo:p + 1, 0] @ qs[i, h]) * scale
+            ref[i, h] = torch.softmax(sc, 0) @ vs[lo:p + 1, 0]
+    ref = ref.reshape(64, nh * hd)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    out = torch.zeros(L, nh * hd, dtype=dtype, device=DEV)
+    ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32([0]), i32([L - 64]), i32([64]), nh, nkv, hd, bs, window, scale)
+    close(out[L - 64:], ref, dtype, "tiled attention, last block")
+    out2 = torch.zeros(L, nh * hd, dtype=dtype, device=DEV)
+    for chunk in (None, 4096):
+        ops.attention_decode(q_rot, out2, k_pages, v_pages, table, pos, i32([0]), i32([L - 1]), nh, nkv, hd, bs, window, scale,
+                             max_kv_len=L, chunk=chunk)
+        close(out2[L - 1], ref[63], dtype, f"decode attention chunk {chunk}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,H,E,k,renorm", [(1, 64, 8, 2, False), (7, 96, 6, 3, True), (33, 200, 60, 4, False),
                                              (5, 128, 130, 8, True), (4, 72, 5, 5, False)])
