@@ -275,28 +275,56 @@ FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, 
 // in ascending j, the selection order (ferrox-moe/src/lib.rs:735-745).
 // y is float32 [T*k, H].
 // ---------------------------------------------------------------------------
+// xg != nullptr: the new rows are also written as xg = round(h * norm_w) (no scale yet) with each block's sum
+// of squares of its 256 columns in ss[t * gridDim.y + blockIdx.y]: the product that reads xg scales its
+// rows by rsqrt(sum / H + eps), which is RMSNorm with the rounding of the norm that a product applies itself.
+template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
                                                           const float* __restrict__ shared, const float* __restrict__ gate,
-                                                          int H, int k, int slabs) {
-    const int t = blockIdx.x, T = gridDim.x;
+                                                          int H, int k, int slabs, const void* __restrict__ norm_w,
+                                                          int norm_dtype, T* __restrict__ xg, float* __restrict__ ss) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, n_tok = gridDim.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
-    if (c >= H) return;
-    float acc = 0.f;
-    for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
-    if (shared) {      // routed first, then shared (lib.rs:746-750); the shared output may come as `slabs` partial sums [slab][T][H]
-        float sh = 0.f;
-        for (int s = 0; s < slabs; ++s) sh += shared[((size_t)s * T + t) * H + c];
-        acc += (gate ? gate[t] : 1.f) * sh;
+    float v = 0.f;
+    if (c < H) {
+        float acc = 0.f;
+        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
+        if (shared) {      // routed first, then shared (lib.rs:746-750); the shared output may come as `slabs` partial sums [slab][T][H]
+            float sh = 0.f;
+            for (int s = 0; s < slabs; ++s) sh += shared[((size_t)s * n_tok + t) * H + c];
+            acc += (gate ? gate[t] : 1.f) * sh;
+        }
+        v = h[(size_t)t * H + c] + acc;
+        h[(size_t)t * H + c] = v;
     }
-    h[(size_t)t * H + c] += acc;
+    if (!xg) return;
+    if (c < H) from_float(xg + (size_t)t * H + c, v * load_as_float(norm_w, norm_dtype, c));
+    const float total = block_sum<4>(v * v, red);
+    if (threadIdx.x == 0) ss[t * gridDim.y + blockIdx.y] = total;
 }
 
+// norm_w != nullptr: x_out = round(h * norm_w) of the new rows, in out_dtype, and ss[t][b] = the sum of squares of
+// columns [256 b, 256 b + 256) of row t.
 FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv, const float* w,
-                          const float* shared, const float* gate, int T, int H, int k, int slabs) {
+                          const float* shared, const float* gate, int T, int H, int k, int slabs,
+                          const void* norm_w, int norm_dtype, void* x_out, int out_dtype, float* ss) {
     FX_REQUIRE(T >= 0 && H > 0 && k > 0 && slabs >= 1, "moe_combine: bad sizes");
     if (T == 0) return 0;
-    moe_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, (hipStream_t)stream>>>(h, y, inv, w, shared, gate, H, k, slabs);
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T, (H + 255) / 256);
+    if (norm_w) {
+        FX_REQUIRE(x_out && ss, "moe_combine: the rows for the norm need places to write");
+        FX_REQUIRE(norm_dtype == FX_F32 || norm_dtype == FX_BF16, "moe_combine: unknown norm weight dtype %d", norm_dtype);
+        FX_REQUIRE(out_dtype == FX_F32 || out_dtype == FX_BF16, "moe_combine: unknown output dtype %d", out_dtype);
+        if (out_dtype == FX_F32)
+            moe_combine_kernel<float><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, (float*)x_out, ss);
+        else
+            moe_combine_kernel<bf16><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, (bf16*)x_out, ss);
+    } else {
+        moe_combine_kernel<float><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, nullptr, 0, nullptr, nullptr);
+    }
     FX_CHECK_LAUNCH("moe_combine");
     return 0;
 }

@@ -46,6 +46,8 @@ struct GemmArgs {
     const void* norm_w;  // skinny bf16 kernel only: A is the float32 residual stream and RMSNorm with these weights
     int norm_dtype;      //   is applied on the way in; norm_w is [K]
     float norm_eps;
+    const float* row_ss; // skinny bf16 kernel only: row m of the product is scaled by rsqrt(sum(row_ss[m][0..row_ss_n)) / K + norm_eps)
+    int row_ss_n;        //   (the rows of A are x * w of an RMSNorm whose scale is still to come)
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
@@ -727,6 +729,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         if (pairs ? ml < 0 : ml >= r_end) continue;
         const int m = (g.c_rows && !pairs) ? g.c_rows[ml] : ml;
         float rstd = 1.f;
+        if (!NORM && g.row_ss) {
+            float total = 0.f;
+            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)m * g.row_ss_n + b];
+            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+        }
         if constexpr (NORM) {
             float total = 0.f;
 #pragma unroll
@@ -934,7 +941,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
-                   const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows) {
+                   const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows,
+                   const float* row_ss, int row_ss_n) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -955,6 +963,10 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     }
     GemmArgs g;
     g.norm_w = norm_w; g.norm_dtype = norm_dtype; g.norm_eps = norm_eps;
+    g.row_ss = row_ss; g.row_ss_n = row_ss_n;
+    FX_REQUIRE(!row_ss || (row_ss_n >= 1 && !norm_w && !expert_offsets && !pair_ids && !a_rows && !c_rows && dtype == FX_BF16 &&
+                           epi == EPI_STORE && M <= 64 && K % 8 == 0 && lda % 8 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0)),
+               "gemm: a row scale from sums of squares goes with a plain stored bfloat16 product of up to 64 aligned rows");
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;

@@ -95,8 +95,19 @@ class Model:
     # ---- forward ---------------------------------------------------------
     def forward(self, ctx: StepContext, caches: list):
         h = self.embedding.forward(ctx.token_ids)
+        # blocks that chain their norms: the block before may already have applied this block's first norm
+        # to the rows it finished (in the kernel that finished them)
+        normed = None
         for i, e in enumerate(self.schedule):
-            self.blocks[e.layer].forward(h, ctx, caches[i])
+            block = self.blocks[e.layer]
+            if getattr(block, "chains_norms", False):
+                nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+                then = (nxt.first_norm, nxt.takes_scale_later(ctx.act_dtype)) \
+                    if nxt is not None and getattr(nxt, "chains_norms", False) else None
+                normed = block.forward(h, ctx, caches[i], normed=normed, then=then)
+            else:
+                block.forward(h, ctx, caches[i])
+                normed = None
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
         x = self.final_norm.forward(h, ctx, rows=ctx.logit_rows)

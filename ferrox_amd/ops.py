@@ -52,11 +52,11 @@ _sigs = {
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                        c_int, c_int, c_int, c_int],
+                                        c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -172,10 +172,21 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
     _call("elementwise", "fx_fill_u32", _stream(), _p(t), value, t.element_size() * t.numel() // 4)
 
 
-def moe_combine(h, y_sorted, inv, weights, top_k, shared=None, gate=None) -> None:
+class ScaleLater:
+    """Rows x = round(h * w) of an RMSNorm whose scale is still to come: `ss` [T, n] holds sums of squares of
+    parts of each row of h, and row t is to be scaled by rsqrt(sum(ss[t]) / width + eps).  `gemm(..., row_ss=)`
+    applies the scale to its product, which is the rounding of the norm that `gemm(..., norm=)` applies itself."""
+    __slots__ = ("x", "ss", "eps")
+
+    def __init__(self, x, ss, eps):
+        self.x, self.ss, self.eps = x, ss, eps
+
+
+def moe_combine(h, y_sorted, inv, weights, top_k, shared=None, gate=None, scale_later=None):
     """h[t] += sum_j weights[t, j] * y_sorted[inv[t*k + j]] (inv None: y is in pair order t*k + j)
     + gate[t] * shared[t] if the float32 output of a shared expert is given; `shared` may also be
-    [S, T, H], partial outputs that are summed first."""
+    [S, T, H], partial outputs that are summed first.
+    `scale_later` = (norm weight, eps, dtype): also returns the new rows as a ScaleLater for that RMSNorm."""
     T, H = h.shape
     if y_sorted.dtype != torch.float32 or h.dtype != torch.float32:
         raise KernelError("moe_combine works on float32")
@@ -184,8 +195,17 @@ def moe_combine(h, y_sorted, inv, weights, top_k, shared=None, gate=None) -> Non
         if shared.dtype != torch.float32 or not shared.is_contiguous() or shared.shape[-2:] != h.shape or shared.dim() > 3:
             raise KernelError("moe_combine: the shared expert's output must be float32 [T, H] or [S, T, H]")
         slabs = shared.shape[0] if shared.dim() == 3 else 1
+    x, nw, eps, code, ss = None, None, 0.0, 0, None
+    if scale_later is not None:
+        nw, eps, dt = scale_later
+        if nw.numel() != H or not nw.is_contiguous() or not h.is_contiguous():
+            raise KernelError(f"moe_combine: norm weight of {nw.numel()} elements for width {H}")
+        x, code = torch.empty((T, H), dtype=dt, device=h.device), dtype_code(dt)
+        ss = torch.empty((T, (H + 255) // 256), dtype=torch.float32, device=h.device)
     _call("elementwise", "fx_moe_combine", _stream(), _p(h), _p(y_sorted), _p(_i32(inv, "inv")), _p(weights),
-          _p(shared), _p(gate), T, H, top_k, slabs)
+          _p(shared), _p(gate), T, H, top_k, slabs, _p(nw), dtype_code(nw.dtype) if nw is not None else 0,
+          _p(x), code, _p(ss))
+    return ScaleLater(x, ss, float(eps)) if ss is not None else None
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: torch.Tensor | None = None,
@@ -194,7 +214,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
          norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
-         always: tuple | None = None, w_kblocked: bool = False) -> torch.Tensor:
+         always: tuple | None = None, w_kblocked: bool = False, row_ss: tuple | None = None) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -212,7 +232,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     `w_kblocked`: `w` is stored as `to_kblocked` makes it, [.., K/64, N, 64] (bfloat16, K % 64 == 0).
     `norm` = (weight [K], eps): `a` is the float32 residual stream and RMSNorm is applied on the way
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
+    `row_ss` = (ss [M, n] float32, eps): row m of the product is scaled by rsqrt(sum(ss[m]) / K + eps)
+    before the bias is added (the rows of `a` are a ScaleLater's; plain stored bfloat16 product, M <= 64).
     """
+    if row_ss is not None:
+        ss = row_ss[0]
+        if ss.dtype != torch.float32 or ss.dim() != 2 or not ss.is_contiguous() or ss.shape[0] != a.shape[0]:
+            raise KernelError("gemm: row_ss must be a contiguous float32 [rows, parts]")
     if norm is not None:
         if a.dtype != torch.float32 or w.dtype != torch.bfloat16 or epilogue != EPI_STORE:
             raise KernelError("gemm: the fused norm reads float32 rows for a stored bfloat16 product")
@@ -270,8 +296,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
           _p(_i32(expert_offsets, "expert_offsets")), E, M, N, K,
           _p(norm[0]) if norm is not None else None, dtype_code(norm[0].dtype) if norm is not None else 0,
-          float(norm[1]) if norm is not None else 0.0, _p(_i32(pair_ids, "pair_ids")), int(pair_div),
-          n_always, always_rows, always_from_a, n_w if w_kblocked else 0)
+          float(norm[1]) if norm is not None else (float(row_ss[1]) if row_ss is not None else 0.0),
+          _p(_i32(pair_ids, "pair_ids")), int(pair_div),
+          n_always, always_rows, always_from_a, n_w if w_kblocked else 0,
+          _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0)
     return out
 
 

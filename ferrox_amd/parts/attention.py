@@ -102,9 +102,17 @@ class PagedAttention(Mixer):
         self.forward(None, ctx, cache, residual, qkv=qkv)
         return True
 
+    def takes_scale_later(self, act_dtype) -> bool:
+        """Whether forward takes an ops.ScaleLater as x (the block before then leaves its rows that way)."""
+        w = self.qkv.weight
+        return act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0
+
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         if qkv is None:
-            qkv = self.qkv(x)
+            if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
+                qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
+            else:
+                qkv = self.qkv(x)
         q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]

@@ -141,6 +141,7 @@ class StepContext:
     block_tables: dict                 # group key -> int32 [n_seqs, max_blocks]
     block_size: int
     logit_rows: torch.Tensor | None = None   # int32 [R] token indices whose logits are wanted
+    carry: object = None               # what a feed-forward hands on to the next block (its rows, normed), see PreNormBlock
     _memo: dict = field(default_factory=dict)
 
     def memo(self, key, make: Callable):
@@ -228,7 +229,12 @@ class FeedForward(Part):
 
 
 class Block(Part):
+    """A block that sets `chains_norms = True` also has a `first_norm` and takes
+    forward(h, ctx, cache, normed=None, then=None): `normed` is first_norm(h) if the block before has made it,
+    `then` is (the first norm of the block after, that block's takes_scale_later(dtype)); it returns the
+    rows normed by that norm if one of its kernels has made them, else None."""
     mixer: Mixer
+    chains_norms = False
 
     def forward(self, h, ctx: StepContext, cache: LayerCache) -> None:
         raise NotImplementedError

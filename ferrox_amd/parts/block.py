@@ -16,12 +16,33 @@ class PreNormBlock(Block):
     def children(self):
         return [(self._prefixes[s], getattr(self, s)) for s in ("norm1", "mixer", "norm2", "ffn")]
 
-    def forward(self, h, ctx, cache) -> None:
+    chains_norms = True     # forward takes `normed` and `then` and returns what the next block may take as `normed`
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def takes_scale_later(self, act_dtype) -> bool:
+        f = getattr(self.mixer, "takes_scale_later", None)
+        return bool(f and f(act_dtype))
+
+    def forward(self, h, ctx, cache, normed=None, then=None):
+        """`normed`: norm1(h), if the block before has already made it (a tensor, or an ops.ScaleLater if this
+        block's mixer takes one).  `then`: (the norm that the next block applies first, whether its mixer
+        takes an ops.ScaleLater); a feed-forward that says `norms_after` may apply that norm to the rows it
+        has just finished and leave the result in ctx.carry, which is returned (else None)."""
         # a part may offer `forward_from_residual(norm, ...)`: it then applies the norm itself, fused
         # into its first kernel, and says False when it cannot for this step
-        fused = getattr(self.mixer, "forward_from_residual", None)
-        if fused is None or not fused(self.norm1, ctx, cache, h):
-            self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
+        if normed is not None:
+            self.mixer.forward(normed, ctx, cache, h)
+        else:
+            fused = getattr(self.mixer, "forward_from_residual", None)
+            if fused is None or not fused(self.norm1, ctx, cache, h):
+                self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
+        ctx.carry = None
+        more = {"then_norm": then} if then is not None and getattr(self.ffn, "norms_after", False) else {}
         fused = getattr(self.ffn, "forward_from_residual", None)
-        if fused is None or not fused(self.norm2, ctx, h):
-            self.ffn.forward(self.norm2.forward(h, ctx), ctx, h)
+        if fused is None or not fused(self.norm2, ctx, h, **more):
+            self.ffn.forward(self.norm2.forward(h, ctx), ctx, h, **more)
+        out, ctx.carry = ctx.carry, None
+        return out

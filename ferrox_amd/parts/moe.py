@@ -33,6 +33,7 @@ def side_stream(device) -> torch.cuda.Stream:
 class SparseMoE(FeedForward):
     kernel_libraries = ("elementwise", "gemm", "moe")
     record = None      # a list here collects every call's expert ids (measurement only)
+    norms_after = True   # forward(..., then_norm=norm) may leave norm(residual) in ctx.carry for the next layer
 
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
                  norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
@@ -96,7 +97,20 @@ class SparseMoE(FeedForward):
             router = torch.cat(same_dtype([router, fetch("shared_expert_gate.weight").reshape(1, -1)]), dim=0)
         self.router = router.contiguous()
 
-    def forward_from_residual(self, norm, ctx, residual) -> bool:
+    @staticmethod
+    def _then(then_norm, ctx, n_tokens) -> dict:
+        """How the combine prepares the new rows for the next block's norm: `then_norm` is (norm, whether the
+        block takes an ops.ScaleLater).  For few rows the combine also writes them times the norm's weight,
+        with sums of squares, and the product that follows applies the scale: the norm costs no launch.
+        (For many rows a norm kernel of its own is as fast.)"""
+        if then_norm is None or getattr(then_norm[0], "kind", None) != "rmsnorm":
+            return {}
+        norm, later_ok = then_norm
+        if n_tokens <= 16 and later_ok and ctx.act_dtype == torch.bfloat16:
+            return dict(scale_later=(norm.weight, norm.eps, ctx.act_dtype))
+        return {}
+
+    def forward_from_residual(self, norm, ctx, residual, then_norm=None) -> bool:
         """Few tokens: the norm and the router are one launch, and the expert products group the
         (token, slot) pairs themselves instead of reading a sorted layout."""
         T = residual.shape[0]
@@ -109,13 +123,15 @@ class SparseMoE(FeedForward):
         x, ids, weights, gate = front
         aligned = self.hidden_size % 8 == 0 and self.expert_intermediate_size % 8 == 0
         if T <= 16 and ids.numel() <= 64 and aligned:       # the expert products take the pairs unsorted
-            self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None))
+            self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None), then_norm=then_norm)
         else:
-            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts))
+            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts),
+                         then_norm=then_norm)
         return True
 
-    def forward(self, x, ctx, residual, routed=None) -> None:
+    def forward(self, x, ctx, residual, routed=None, then_norm=None) -> None:
         T = x.shape[0]
+        then = self._then(then_norm, ctx, T)
         if routed is not None and routed[3] is None and self.shared_pieces and x.dtype == self.w_gate_up_all.dtype:
             # few tokens, unsorted pairs, shared expert as pieces: two launches do all experts
             ids, weights, gate = routed[:3]
@@ -126,7 +142,7 @@ class SparseMoE(FeedForward):
                            always=(S, T, True), w_kblocked=self.kblocked)
             y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False),
                          w_kblocked=self.kblocked)
-            ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate)
+            ctx.carry = ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate, **then)
             return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
         if overlap:
@@ -164,8 +180,9 @@ class SparseMoE(FeedForward):
         if overlap:
             main.wait_event(join)
             shared_out.record_stream(main)
-            ops.moe_combine(residual, y, None, weights, self.top_k, shared=shared_out, gate=gate)
+            ctx.carry = ops.moe_combine(residual, y, None, weights, self.top_k, shared=shared_out, gate=gate, **then)
+        elif self.shared is None:
+            ctx.carry = ops.moe_combine(residual, y, None, weights, self.top_k, **then)
         else:
             ops.moe_combine(residual, y, None, weights, self.top_k)
-            if self.shared is not None:
-                self.shared.forward(x, ctx, residual, row_scale=gate)
+            self.shared.forward(x, ctx, residual, row_scale=gate)

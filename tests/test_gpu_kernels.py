@@ -44,6 +44,29 @@ def test_gemm_plain_and_epilogues(dtype, M, N, K):
     close(h, h0.double() + ref * scale.double()[:, None], dtype, "residual")
 
 
+@pytest.mark.parametrize("T,H,N,k,S", [(1, 2048, 6144, 4, 4), (8, 2048, 6144, 4, 4), (16, 264, 100, 3, 0), (5, 520, 72, 1, 2)])
+def test_combine_that_leaves_the_scale_to_the_product(T, H, N, k, S):
+    """combine -> rows times the norm's weight and sums of squares -> product that scales its rows,
+    against combine -> norm kernel -> product and against the plain formulas"""
+    from ferrox_amd import ops
+    h = rnd(T, H, scale=2.0)
+    y, wts = rnd(T * k, H, seed=1), torch.rand(T, k, generator=torch.Generator().manual_seed(2)).to(DEV)
+    shared = rnd(S, T, H, seed=3) if S else None
+    gate = torch.rand(T, generator=torch.Generator().manual_seed(4)).to(DEV) if S else None
+    gamma = (1.0 + rnd(H, seed=5, scale=0.2)).to(torch.bfloat16)
+    w, bias = rnd(N, H, dtype=torch.bfloat16, seed=6, scale=0.05), rnd(N, dtype=torch.bfloat16, seed=7)
+    h1, h2 = h.clone(), h.clone()
+    ops.moe_combine(h1, y, None, wts, k, shared=shared, gate=gate)
+    two = ops.gemm(ops.rmsnorm(h1, gamma, 1e-6, torch.bfloat16), w, bias=bias)
+    later = ops.moe_combine(h2, y, None, wts, k, shared=shared, gate=gate, scale_later=(gamma, 1e-6, torch.bfloat16))
+    assert isinstance(later, ops.ScaleLater) and torch.equal(h1, h2)
+    close(later.ss.sum(1), (h1.double() ** 2).sum(1), torch.float32, "sums of squares")
+    got = ops.gemm(later.x, w, bias=bias, row_ss=(later.ss, later.eps))
+    want = plain.rms_norm(h1.double().cpu(), gamma.double().cpu(), 1e-6) @ w.double().cpu().T + bias.double().cpu()
+    close(got, want, torch.bfloat16, "product with the scale applied afterwards")
+    close(two, want, torch.bfloat16, "norm, then product")
+
+
 @pytest.mark.parametrize("tile", [256, 192, 128, 64])
 @pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
 def test_gemm_every_wide_tile(tile, M, N, K):
