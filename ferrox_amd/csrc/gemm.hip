@@ -876,10 +876,8 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 #undef FX_TILED
 }
 
-static int g_skinny_four = 0;      // blocks that four-set tiles must still give; 0: never four sets (two leave registers for more waves)
-FX_API void fx_gemm_set_skinny_four(int blocks) { g_skinny_four = blocks; }
-static int g_skinny_nw = 0, g_skinny_eight = -1;        // measurement only: sets per wave (1, 2, 4) and waves (0: four, 1: eight) whatever the sizes
-FX_API void fx_gemm_set_skinny(int nw, int eight) { g_skinny_nw = nw; g_skinny_eight = eight; }
+static int g_skinny_nw = 0;        // measurement only: 1 or 2 sets of weight rows per wave whatever the sizes
+FX_API void fx_gemm_set_skinny(int nw) { g_skinny_nw = nw; }
 static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
 static int g_wide_force = 0;   // measurement only: 256, 192, 128 or 64 picks that wide tile whatever the sizes
 FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; g_wide_force = on > 1 ? on : 0; }
@@ -918,19 +916,17 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
     }
 }
 
-// mt: row tiles per block (1, 2, 4); eight: 8 waves split K instead of 4; nw: 16-row weight sets per wave
-static void launch_skinny(const GemmArgs& g, int epi, int mt, bool eight, int nw, int m_tiles, hipStream_t s) {
+// mt: row tiles per block (1, 2, 4); nw: 16-row weight sets per wave.  Four waves split K (eight stream no faster).
+static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int m_tiles, hipStream_t s) {
 #define FX_SK(MT_, W_, NW_) launch_skinny_cfg<MT_, W_, NW_>(g, epi, m_tiles, s)
-    if (nw == 4) {
-        FX_SK(1, 4, 4);
-    } else if (nw == 2) {
-        if (mt == 1) { if (eight) FX_SK(1, 8, 2); else FX_SK(1, 4, 2); }
-        else if (mt == 2) { if (eight) FX_SK(2, 8, 2); else FX_SK(2, 4, 2); }
+    if (nw == 2) {
+        if (mt == 1) FX_SK(1, 4, 2);
+        else if (mt == 2) FX_SK(2, 4, 2);
         else FX_SK(4, 4, 2);
     } else {
-        if (mt == 1) { if (eight) FX_SK(1, 8, 1); else FX_SK(1, 4, 1); }
-        else if (mt == 2) { if (eight) FX_SK(2, 8, 1); else FX_SK(2, 4, 1); }
-        else { if (eight) FX_SK(4, 8, 1); else FX_SK(4, 4, 1); }
+        if (mt == 1) FX_SK(1, 4, 1);
+        else if (mt == 2) FX_SK(2, 4, 1);
+        else FX_SK(4, 4, 1);
     }
 #undef FX_SK
 }
@@ -1008,11 +1004,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         // so many weight rows that the blocks are plenty either way (measured on the sizes of the engine)
         int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 160) ? 2 : 1;
         if (!dual && (norm_w || (M <= 2 && (long)ceil_div(N, 16) * m_tiles >= 4096))) nw = 1;
-        // four sets: measurement only (they leave registers for two waves per SIMD, which streams less)
-        if (mt == 1 && !norm_w && g_skinny_four && (long)ceil_div(N, dual ? 32 : 64) * m_tiles >= g_skinny_four) nw = 4;
-        if (g_skinny_nw && !norm_w && (g_skinny_nw < 4 || mt == 1) && !(dual && g_skinny_nw == 1)) nw = g_skinny_nw;
-        const bool eight = g_skinny_eight > 0 && mt * nw <= 4;      // measurement only: four waves stream as well
-        launch_skinny(g, epi, mt, eight, nw, m_tiles, s);
+        if ((g_skinny_nw == 1 && !dual) || (g_skinny_nw == 2 && !norm_w)) nw = g_skinny_nw;
+        launch_skinny(g, epi, mt, nw, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }
