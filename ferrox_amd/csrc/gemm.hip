@@ -334,8 +334,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 // chunk they fetch, so that the 16 rows an MFMA operand reads fall on distinct
 // banks without padding.  Waves form a 2 x 4 grid: a wave owns TN/4 weight rows
 // and every second block of 16 rows (so a tile with few rows, an expert's share,
-// still spreads over both halves); row blocks past the tile's rows are not
-// multiplied.
+// still spreads over both halves, and the two waves of a SIMD are one of each
+// half); row blocks past the tile's rows are not multiplied.  The rows' ring may
+// be shallower than the weights' (NSA < NS): weights come from memory and are
+// read once, so more of them are kept on their way.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(1))) const void* fx_global_ptr;
 typedef __attribute__((address_space(3))) void* fx_lds_ptr;
@@ -538,9 +540,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 
 // ---------------------------------------------------------------------------
 // Few rows (decode): the weights are streamed once from memory straight into
-// MFMA operands, no LDS staging.  A block owns 16 output columns (16 rows of W)
-// and up to 16*MT logical rows; its WAVES waves split K between them in pieces
-// of 128 and their partial sums are added in wave order through LDS.  In each
+// MFMA operands, no LDS staging.  A block owns NW sets of 16 rows of W and up
+// to 16*MT logical rows; its WAVES waves split K between them in pieces of 128
+// (with few accumulators, the next piece's loads are issued before this piece's
+// products) and their partial sums are added in wave order through LDS.  In each
 // of the four loads of a piece the lanes (i = lane%16, g = lane/16) of a row
 // read 64 contiguous bytes of W row n0+i; the activations use the same
 // k -> lane assignment, which is all the MFMA needs to be right.
