@@ -200,7 +200,7 @@ def main() -> int:
     log(f"decode batch {args.batch}: {dt * 1e3:.3f} ms/step, {tok_s:.1f} tok/s, {distinct:.1f} experts/layer, "
         f"{achieved / 1e9:.0f} GB/s")
     out = {
-        "metric": "decode tok/s (batch 8, 2,048-token prompts)", "value": round(tok_s, 2), "unit": "tokens/s",
+        "metric": f"decode tok/s (batch {args.batch}, {args.ctx:,}-token prompts)", "value": round(tok_s, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: seeded random token ids, seeded random N(0,0.02) weights",
