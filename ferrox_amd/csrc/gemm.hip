@@ -48,6 +48,19 @@ struct GemmArgs {
     float norm_eps;
     const float* row_ss; // skinny bf16 kernel only: row m of the product is scaled by rsqrt(sum(row_ss[m][0..row_ss_n)) / K + norm_eps)
     int row_ss_n;        //   (the rows of A are x * w of an RMSNorm whose scale is still to come)
+    // skinny bf16 kernel, rope epilogue: C is [M, (nh + 2 nkv) * hd], queries | keys | values of token m at position
+    // positions[m] of sequence token_seq[m].  Queries are rotated and stored in C; keys are rotated and stored in their
+    // page, values in theirs (transposed), nothing of either in C.  Split-half pairs (i, i + rot/2), angle
+    // pos * theta^(-2i/rot) (ferrox-core/src/attention.rs:20-32); the product is rounded to bfloat16 before it is
+    // rotated, as when the rotation is a kernel of its own.
+    const int* rope_positions;
+    const int* rope_token_seq;
+    const int* rope_table;
+    int rope_max_blocks;
+    void* rope_k_pages;     // null: nothing is written to pages (a layer that reads another's cache)
+    void* rope_v_pages;
+    int rope_nh, rope_nkv, rope_hd, rope_bs, rope_rot;
+    float rope_theta;
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
@@ -565,9 +578,10 @@ __device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
 
 // NW: sets of 16 weight rows per wave; in dual mode set a is the gate (a even) or up (a odd) rows of
 // column group a / 2.
-template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false>
+template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
     static_assert(!DUAL || NW % 2 == 0, "dual mode multiplies two matrices");
+    static_assert(!ROPE || (MT == 1 && NW == 2 && !DUAL && !NORM && EPI == EPI_STORE), "the rope epilogue pairs two sets of columns of one row tile");
     static_assert(!NORM || (!DUAL && EPI == EPI_STORE), "the fused norm feeds a plain product");
     __shared__ float red_ss[NORM ? WAVES : 1][MT][64];
     float ss[MT];
@@ -588,10 +602,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, grp = lane >> 4;
     const bf16* Wbase = (const bf16*)g.W + (size_t)expert * g.w_stride;
+    // rope epilogue: a block takes 16 + 16 columns of one head, (16 j .. , rot/2 + 16 j ..) while they are rotated,
+    // two neighbouring sets of 16 after that
+    int rope_head = 0, rope_j = 0, rope_c0 = 0, rope_c1 = 0;
+    bool rope_rotated = false;
+    if constexpr (ROPE) {
+        const int per_head = g.rope_hd >> 5;
+        rope_head = blockIdx.x / per_head;
+        rope_j = blockIdx.x - rope_head * per_head;
+        const bool is_v = rope_head >= g.rope_nh + g.rope_nkv;
+        const int n_rot = is_v ? 0 : g.rope_rot >> 5;          // blocks of this head whose columns are rotated
+        rope_rotated = rope_j < n_rot;
+        rope_c0 = rope_rotated ? 16 * rope_j : (is_v ? 32 * rope_j : g.rope_rot + 32 * (rope_j - n_rot));
+        rope_c1 = rope_rotated ? rope_c0 + (g.rope_rot >> 1) : rope_c0 + 16;
+    }
     const bf16* wrow[NW];
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
-        const int n = DUAL ? n0 + (a >> 1) * 16 + li : n0 + a * 16 + li;
+        const int n = ROPE ? rope_head * g.rope_hd + (a ? rope_c1 : rope_c0) + li
+                           : (DUAL ? n0 + (a >> 1) * 16 + li : n0 + a * 16 + li);
         const bool up = DUAL && (a & 1);
         // rows past the end repeat the last one: their columns are never stored
         const int nc = min(n, g.N - 1);
@@ -717,6 +746,62 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         for (int mt = 0; mt < MT; ++mt) red_ss[wave][mt][lane] = ss[mt];
     }
     __syncthreads();
+    if constexpr (ROPE) {
+        static_assert(!ROPE || WAVES == 4, "a wave per accumulator row");
+        const int L = lane, r = wave;
+        const int ml = r0 + (L & 15);
+        if (ml >= r_end) return;
+        f32x4_t v0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v1 = v0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            v0 += red[w][0][L];
+            v1 += red[w][1][L];
+        }
+        float rstd = 1.f;
+        if (g.row_ss) {
+            float total = 0.f;
+            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
+            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+        }
+        const int hd = g.rope_hd, cc = (L >> 4) * 4 + r;
+        const int d0 = rope_c0 + cc, d1 = rope_c1 + cc;
+        float o0 = v0[r] * rstd, o1 = v1[r] * rstd;
+        if (g.bias) {
+            o0 += load_as_float(g.bias, g.bias_dtype, rope_head * hd + d0);
+            o1 += load_as_float(g.bias, g.bias_dtype, rope_head * hd + d1);
+        }
+        const float a = bf16_to_float(float_to_bf16(o0)), b = bf16_to_float(float_to_bf16(o1));
+        float y0 = a, y1 = b;
+        const int pos = g.rope_positions[ml];
+        if (rope_rotated) {
+            const int p = 16 * rope_j + cc;
+            const float freq = 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot);
+            float sn, cs;
+            sincosf((float)pos * freq, &sn, &cs);
+            y0 = a * cs - b * sn;
+            y1 = a * sn + b * cs;
+        }
+        if (rope_head < g.rope_nh) {
+            bf16* dst = (bf16*)g.C + (size_t)ml * g.ldc + (size_t)rope_head * hd;
+            from_float(dst + d0, y0);
+            from_float(dst + d1, y1);
+            return;
+        }
+        if (!g.rope_k_pages) return;
+        const int bs = g.rope_bs;
+        const size_t page = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / bs];
+        const int slot = pos % bs;
+        if (rope_head < g.rope_nh + g.rope_nkv) {
+            bf16* dst = (bf16*)g.rope_k_pages + ((page * g.rope_nkv + (rope_head - g.rope_nh)) * bs + slot) * hd;
+            from_float(dst + d0, y0);
+            from_float(dst + d1, y1);
+        } else {
+            bf16* dst = (bf16*)g.rope_v_pages + (page * g.rope_nkv + (rope_head - g.rope_nh - g.rope_nkv)) * hd * bs + slot;
+            from_float(dst + (size_t)d0 * bs, y0);
+            from_float(dst + (size_t)d1 * bs, y1);
+        }
+        return;
+    }
     constexpr int SETS = DUAL ? NW / 2 : NW;      // column groups of a block
     constexpr int OUTS = MT * SETS;               // accumulator tiles (dual: pairs of them) that become output tiles
     for (int idx = tid; idx < OUTS * 64; idx += WAVES * 64) {
@@ -934,6 +1019,36 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int m_tile
 #undef FX_SK
 }
 
+// The q/k/v product of up to 16 tokens with the rotation and the cache write in its epilogue (see GemmArgs):
+// bfloat16, C [M, (nh + 2 nkv) hd], bias [N] or null, row_ss as in fx_gemm.  head_dim and the rotary dimension
+// are multiples of 32.  k_pages [pages][nkv][bs][hd] and v_pages [pages][nkv][hd][bs], or both null.
+FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, long kb_rows, const void* bias, int bias_dtype,
+                       void* C, long ldc, int M, int K, const float* row_ss, int row_ss_n, float eps,
+                       const int* positions, const int* token_seq, const int* table, int max_blocks,
+                       void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, float theta) {
+    FX_REQUIRE(M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K, "qkv_rope: 1..16 rows of a multiple of 8 elements");
+    FX_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 32 == 0 && rot >= 0 && rot <= hd && rot % 32 == 0 && bs > 0,
+               "qkv_rope: head_dim %d and rotary dimension %d must be multiples of 32", hd, rot);
+    const int N = (nh + 2 * nkv) * hd;
+    FX_REQUIRE(ldc >= N && (((uintptr_t)A | (uintptr_t)W) % 16) == 0, "qkv_rope: output rows too short or operands not aligned");
+    FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "qkv_rope: key and value pages must come together");
+    FX_REQUIRE(positions && token_seq && (!k_pages || (table && max_blocks > 0)), "qkv_rope: positions, sequences and block table");
+    FX_REQUIRE(!bias || bias_dtype == FX_F32 || bias_dtype == FX_BF16, "qkv_rope: unknown bias dtype %d", bias_dtype);
+    FX_REQUIRE(kb_rows == 0 || (kb_rows == N && K % 64 == 0), "qkv_rope: weights in slabs of 64 k hold all %d rows", N);
+    FX_REQUIRE(!row_ss || row_ss_n >= 1, "qkv_rope: sums of squares without their count");
+    GemmArgs g = {};
+    g.A = A; g.lda = lda; g.W = W; g.kb_stride = kb_rows * 64; g.bias = bias; g.bias_dtype = bias_dtype;
+    g.C = C; g.ldc = ldc; g.M = M; g.N = N; g.K = K; g.vec_ok = 1;
+    g.row_ss = row_ss; g.row_ss_n = row_ss_n; g.norm_eps = eps;
+    g.rope_positions = positions; g.rope_token_seq = token_seq; g.rope_table = table; g.rope_max_blocks = max_blocks;
+    g.rope_k_pages = k_pages; g.rope_v_pages = v_pages;
+    g.rope_nh = nh; g.rope_nkv = nkv; g.rope_hd = hd; g.rope_bs = bs; g.rope_rot = rot; g.rope_theta = theta;
+    dim3 grid((nh + 2 * nkv) * (hd / 32), 1);
+    gemm_bf16_skinny_kernel<1, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
+    FX_CHECK_LAUNCH("qkv_rope");
+    return 0;
+}
+
 // dtype: type of A and W.  C is: T for EPI_STORE and EPI_SILU_MUL, float32 otherwise.
 // rows_hint: in grouped mode, the expected number of rows per expert (chooses the tile).
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
@@ -960,7 +1075,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                        (((uintptr_t)A | (uintptr_t)W | (uintptr_t)norm_w) % 16 == 0),
                    "gemm: the fused norm takes up to 32 rows per group, K a multiple of 8 and 16-byte aligned rows");
     }
-    GemmArgs g;
+    GemmArgs g = {};
     g.norm_w = norm_w; g.norm_dtype = norm_dtype; g.norm_eps = norm_eps;
     g.row_ss = row_ss; g.row_ss_n = row_ss_n;
     FX_REQUIRE(!row_ss || (row_ss_n >= 1 && !norm_w && !expert_offsets && !pair_ids && !a_rows && !c_rows && dtype == FX_BF16 &&

@@ -57,6 +57,9 @@ _sigs = {
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
+    ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
+                              c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                              c_int, c_int, c_int, c_int, c_int, c_float],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -300,6 +303,46 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(_i32(pair_ids, "pair_ids")), int(pair_div),
           n_always, always_rows, always_from_a, n_w if w_kblocked else 0,
           _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0)
+    return out
+
+
+def can_qkv_rope(x, w, n_rows: int, head_dim: int, rotary_dim: int, interleaved: bool) -> bool:
+    """Whether qkv_rope takes these operands: up to 16 rows of bfloat16 (or a ScaleLater of them), split-half
+    rotation, head and rotary dimensions that are multiples of 32, aligned rows."""
+    xt = x.x if isinstance(x, ScaleLater) else x
+    return (n_rows <= 16 and not interleaved and head_dim % 32 == 0 and rotary_dim % 32 == 0
+            and xt.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+            and xt.dim() == 2 and xt.stride(1) == 1 and xt.stride(0) % 8 == 0 and xt.shape[1] % 8 == 0
+            and xt.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def qkv_rope(x, w, bias, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads, head_dim,
+             block_size, rotary_dim, theta) -> torch.Tensor:
+    """The q/k/v product of few tokens with the rotation and the cache write in its epilogue: returns
+    [T, (n_heads + 2 n_kv_heads) head_dim] whose query columns are rotated (the others are not written); rotated
+    keys and the values go into their pages (k_pages None: nowhere).  The bits are those of `gemm` followed by
+    `rope_kv_write`.  `x` may be a ScaleLater."""
+    later = x if isinstance(x, ScaleLater) else None
+    xt = later.x if later else x
+    T, K = xt.shape
+    N = (n_heads + 2 * n_kv_heads) * head_dim
+    if w.shape != (N, K):
+        raise KernelError(f"qkv_rope: weights {tuple(w.shape)} for [{N}, {K}]")
+    if bias is not None and bias.numel() != N:
+        raise KernelError(f"qkv_rope: bias has {bias.numel()} elements for {N} columns")
+    if k_pages is not None:
+        if k_pages.dtype != xt.dtype or v_pages.dtype != xt.dtype:
+            raise KernelError("cache pages and activations differ in dtype")
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (n_kv_heads, head_dim, block_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_pages.shape)}, {tuple(v_pages.shape)}")
+    out = torch.empty((T, N), dtype=xt.dtype, device=xt.device)
+    _call("gemm", "fx_qkv_rope", _stream(), _p(xt), xt.stride(0), _p(w), 0, _p(bias),
+          dtype_code(bias.dtype) if bias is not None else 0, _p(out), out.stride(0), T, K,
+          _p(later.ss) if later else None, later.ss.shape[1] if later else 0, float(later.eps) if later else 0.0,
+          _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")), _p(_i32(block_table, "block_table")),
+          block_table.shape[1] if block_table is not None else 0, _p(k_pages), _p(v_pages),
+          n_heads, n_kv_heads, head_dim, block_size, rotary_dim, float(theta))
     return out
 
 

@@ -108,21 +108,29 @@ class PagedAttention(Mixer):
         return act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0
 
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
-        if qkv is None:
-            if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
-                qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
-            else:
-                qkv = self.qkv(x)
-        q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
-        if rot is None:
-            self.position.apply(q, k, ctx)
-            rot = (0, 1.0, False)
-        ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
-                          k_pages if cache.writes else None, v_pages if cache.writes else None,
-                          self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1], rot[2])
+        if (qkv is None and rot is not None
+                and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot[0], rot[2])):
+            # few tokens: rotation and cache write happen in the product's epilogue
+            qkv = ops.qkv_rope(x, self.qkv.weight, self.qkv.bias, ctx.positions, ctx.token_seq, table,
+                               k_pages if cache.writes else None, v_pages if cache.writes else None,
+                               self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1])
+            q = qkv[:, :self.qw]
+        else:
+            if qkv is None:
+                if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
+                    qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
+                else:
+                    qkv = self.qkv(x)
+            q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
+            if rot is None:
+                self.position.apply(q, k, ctx)
+                rot = (0, 1.0, False)
+            ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
+                              k_pages if cache.writes else None, v_pages if cache.writes else None,
+                              self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1], rot[2])
         out = torch.empty((ctx.n_tokens, self.qw), dtype=qkv.dtype, device=qkv.device)
         items = ctx.memo("attention_items", lambda: attention_items(ctx))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)

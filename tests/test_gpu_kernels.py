@@ -327,6 +327,48 @@ def test_rope_and_cache_write(dtype, nh, nkv, hd, bs, rot, theta):
         assert torch.equal(v_pages[page, :, :, p % bs].reshape(-1), v[t]), f"v page token {t}"
 
 
+@pytest.mark.parametrize("later", [False, True])
+@pytest.mark.parametrize("T,H,nh,nkv,hd,bs,rot,bias", [(1, 2048, 16, 16, 128, 64, 128, True), (8, 2048, 16, 16, 128, 64, 128, True),
+                                                       (16, 264, 6, 2, 64, 16, 32, True), (5, 520, 3, 1, 32, 8, 0, False),
+                                                       (7, 128, 4, 2, 96, 32, 64, True)])
+def test_qkv_product_that_rotates_and_writes_the_cache(later, T, H, nh, nkv, hd, bs, rot, bias):
+    """The q/k/v product with rotation and cache write in its epilogue gives the bits of the product followed
+    by rope_kv_write: rotated queries, key pages and value pages; also from rows whose norm's scale is applied
+    by the product."""
+    from ferrox_amd import ops
+    N = (nh + 2 * nkv) * hd
+    w = rnd(N, H, dtype=torch.bfloat16, seed=1, scale=0.05)
+    b = rnd(N, dtype=torch.bfloat16, seed=2) if bias else None
+    x = rnd(T, H, dtype=torch.bfloat16, seed=3)
+    if later:
+        ss = (torch.rand(T, (H + 255) // 256, generator=torch.Generator().manual_seed(4)) * 40 + 1).to(DEV)
+        x = ops.ScaleLater(x, ss, 1e-6)
+    g = torch.Generator().manual_seed(5)
+    n_seq = 3
+    seq = torch.randint(0, n_seq, (T,), generator=g)
+    pos = torch.zeros(T, dtype=torch.long)
+    for s_ in range(n_seq):                       # distinct positions inside a sequence
+        idx = (seq == s_).nonzero().flatten()
+        pos[idx] = torch.randperm(5 * bs, generator=g)[:idx.numel()]
+    table = torch.randperm(n_seq * 5, generator=g).reshape(n_seq, 5).to(torch.int32).to(DEV)
+    pos_d, seq_d = pos.to(torch.int32).to(DEV), seq.to(torch.int32).to(DEV)
+    pages = lambda: (torch.zeros(n_seq * 5, nkv, bs, hd, dtype=torch.bfloat16, device=DEV),
+                     torch.zeros(n_seq * 5, nkv, hd, bs, dtype=torch.bfloat16, device=DEV))
+    assert ops.can_qkv_rope(x, w, T, hd, rot, False)
+    k1, v1 = pages()
+    got = ops.qkv_rope(x, w, b, pos_d, seq_d, table, k1, v1, nh, nkv, hd, bs, rot, 1e6)
+    k2, v2 = pages()
+    ref = ops.gemm(x.x, w, bias=b, row_ss=(x.ss, x.eps)) if later else ops.gemm(x, w, bias=b)
+    qw, kvw = nh * hd, nkv * hd
+    ops.rope_kv_write(ref[:, :qw], ref[:, qw:qw + kvw], ref[:, qw + kvw:], pos_d, seq_d, table, k2, v2, nh, nkv, hd, bs, rot, 1e6)
+    assert torch.equal(got[:, :qw], ref[:, :qw]), "rotated queries"
+    assert torch.equal(k1, k2), "key pages"
+    assert torch.equal(v1, v2), "value pages"
+    got2 = ops.qkv_rope(x, w, b, pos_d, seq_d, table, None, None, nh, nkv, hd, bs, rot, 1e6)     # no pages: queries only
+    assert torch.equal(got2[:, :qw], ref[:, :qw])
+    assert not ops.can_qkv_rope(x, w, 17, hd, rot, False) and not ops.can_qkv_rope(x, w, T, hd, rot, True)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,hd,bs,window", [(4, 4, 16, 16, 0), (3, 1, 32, 8, 16), (6, 3, 48, 4, 40), (2, 2, 128, 64, 0),
                                                  (8, 2, 80, 16, 7), (4, 1, 256, 32, 100), (4, 2, 64, 64, 50), (3, 1, 128, 128, 90),
