@@ -639,6 +639,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         // a dead row reads the first row of A instead: its products land in rows that are never stored
         xrow[mt] = NORM ? (live ? (const bf16*)((const float*)g.A + off) : nullptr) : (const bf16*)g.A + off;
     }
+    // rope epilogue: what thread (lane, wave) needs for its pair of outputs, row lane % 16, column 4 (lane / 16) + wave
+    // of the two sets, is fetched and worked out here, while the weights are on their way
+    float rope_sn = 0.f, rope_cs = 1.f, rope_rstd = 1.f, rope_b0 = 0.f, rope_b1 = 0.f;
+    size_t rope_page = 0;
+    int rope_slot = 0;
+    if constexpr (ROPE) {
+        const int ml = min(r0 + li, r_end - 1), cc = grp * 4 + wave;
+        const int pos = g.rope_positions[ml];
+        if (g.row_ss) {
+            float total = 0.f;
+            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
+            rope_rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+        }
+        if (g.bias) {
+            rope_b0 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c0 + cc);
+            rope_b1 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c1 + cc);
+        }
+        if (rope_rotated) {
+            const int p = 16 * rope_j + cc;
+            const float freq = 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot);
+            sincosf((float)pos * freq, &rope_sn, &rope_cs);
+        }
+        if (rope_head >= g.rope_nh && g.rope_k_pages) {
+            rope_page = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / g.rope_bs];
+            rope_slot = pos % g.rope_bs;
+        }
+    }
     f32x4_t acc[MT][NW];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -757,29 +784,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             v0 += red[w][0][L];
             v1 += red[w][1][L];
         }
-        float rstd = 1.f;
-        if (g.row_ss) {
-            float total = 0.f;
-            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
-            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
-        }
         const int hd = g.rope_hd, cc = (L >> 4) * 4 + r;
         const int d0 = rope_c0 + cc, d1 = rope_c1 + cc;
-        float o0 = v0[r] * rstd, o1 = v1[r] * rstd;
+        float o0 = v0[r] * rope_rstd, o1 = v1[r] * rope_rstd;
         if (g.bias) {
-            o0 += load_as_float(g.bias, g.bias_dtype, rope_head * hd + d0);
-            o1 += load_as_float(g.bias, g.bias_dtype, rope_head * hd + d1);
+            o0 += rope_b0;
+            o1 += rope_b1;
         }
         const float a = bf16_to_float(float_to_bf16(o0)), b = bf16_to_float(float_to_bf16(o1));
         float y0 = a, y1 = b;
-        const int pos = g.rope_positions[ml];
         if (rope_rotated) {
-            const int p = 16 * rope_j + cc;
-            const float freq = 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot);
-            float sn, cs;
-            sincosf((float)pos * freq, &sn, &cs);
-            y0 = a * cs - b * sn;
-            y1 = a * sn + b * cs;
+            y0 = a * rope_cs - b * rope_sn;
+            y1 = a * rope_sn + b * rope_cs;
         }
         if (rope_head < g.rope_nh) {
             bf16* dst = (bf16*)g.C + (size_t)ml * g.ldc + (size_t)rope_head * hd;
@@ -789,14 +805,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         }
         if (!g.rope_k_pages) return;
         const int bs = g.rope_bs;
-        const size_t page = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / bs];
-        const int slot = pos % bs;
         if (rope_head < g.rope_nh + g.rope_nkv) {
-            bf16* dst = (bf16*)g.rope_k_pages + ((page * g.rope_nkv + (rope_head - g.rope_nh)) * bs + slot) * hd;
+            bf16* dst = (bf16*)g.rope_k_pages + ((rope_page * g.rope_nkv + (rope_head - g.rope_nh)) * bs + rope_slot) * hd;
             from_float(dst + d0, y0);
             from_float(dst + d1, y1);
         } else {
-            bf16* dst = (bf16*)g.rope_v_pages + (page * g.rope_nkv + (rope_head - g.rope_nh - g.rope_nkv)) * hd * bs + slot;
+            bf16* dst = (bf16*)g.rope_v_pages + (rope_page * g.rope_nkv + (rope_head - g.rope_nh - g.rope_nkv)) * hd * bs + rope_slot;
             from_float(dst + (size_t)d0 * bs, y0);
             from_float(dst + (size_t)d1 * bs, y1);
         }
