@@ -234,6 +234,104 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
     align_block(ids, n, k, E, per_row, lds, lds + E + 1, expert_offsets, sorted_token, sorted_pair, inv);
 }
 
+// Many pairs: the same sort by many blocks, in two launches.  First every wave counts the experts of its
+// group of 64 pairs into gcnt[group][expert].  Then every block adds up, per expert, the counts of all groups
+// (the offsets) and of the groups before its own (the pairs that come earlier), and its waves place their
+// groups' pairs; block 0 also writes the offsets out.  The order inside an expert is the order of the pairs.
+#define SORT_WAVES 4
+__global__ __launch_bounds__(SORT_WAVES * 64) void moe_count_kernel(const int* __restrict__ ids, int n, int E,
+                                                                    int* __restrict__ gcnt) {
+    extern __shared__ int lds[];                    // SORT_WAVES rows of E counts
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = blockIdx.x * SORT_WAVES + wave;
+    if (g * 64 >= n) return;
+    int* row = lds + wave * E;
+    int bits = 0;
+    while ((1 << bits) < E) ++bits;
+    for (int e = lane; e < E; e += 64) row[e] = 0;
+    __builtin_amdgcn_wave_barrier();
+    const int i = g * 64 + lane;
+    int e = i < n ? ids[i] : -1;
+    if (e >= E) e = -1;
+    const unsigned long long same = same_expert_lanes(e, bits);
+    if (e >= 0 && lane == __ffsll((long long)same) - 1) row[e] = __popcll(same);
+    __builtin_amdgcn_wave_barrier();
+    for (int x = lane; x < E; x += 64) gcnt[(size_t)g * E + x] = row[x];
+}
+
+__global__ __launch_bounds__(SORT_WAVES * 64) void moe_place_kernel(const int* __restrict__ ids, int n, int k, int E,
+                                                                    const int* __restrict__ gcnt,
+                                                                    int* __restrict__ expert_offsets,
+                                                                    int* __restrict__ sorted_token,
+                                                                    int* __restrict__ sorted_pair, int* __restrict__ inv) {
+    extern __shared__ int lds[];
+    int* offs = lds;                                // E + 1: first sorted row of each expert
+    int* before = lds + E + 1;                      // E: pairs of the expert in groups before this block's
+    int* part = before + E;                         // SORT_WAVES x 2 x E partial sums
+    const int th = threadIdx.x, lane = th & 63, wave = th >> 6;
+    const int G = (n + 63) >> 6, g0 = blockIdx.x * SORT_WAVES;
+    int bits = 0;
+    while ((1 << bits) < E) ++bits;
+    // wave w adds the groups w, w + SORT_WAVES, ...: all of them, and those before g0
+    for (int e = lane; e < E; e += 64) {
+        int all = 0, early = 0;
+        for (int g = wave; g < G; g += SORT_WAVES) {
+            const int c = gcnt[(size_t)g * E + e];
+            all += c;
+            if (g < g0) early += c;
+        }
+        part[(wave * 2) * E + e] = all;
+        part[(wave * 2 + 1) * E + e] = early;
+    }
+    __syncthreads();
+    for (int e = th; e < E; e += SORT_WAVES * 64) {
+        int all = 0, early = 0;
+#pragma unroll
+        for (int w = 0; w < SORT_WAVES; ++w) {
+            all += part[(w * 2) * E + e];
+            early += part[(w * 2 + 1) * E + e];
+        }
+        offs[e + 1] = all;
+        before[e] = early;
+    }
+    __syncthreads();
+    if (th < 64) {   // inclusive scan of the totals by the first wave, 64 experts at a time
+        int carry = 0;
+        if (lane == 0) offs[0] = 0;
+        for (int base = 0; base < E; base += 64) {
+            const int e = base + lane;
+            int v = e < E ? offs[e + 1] : 0;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int u = __shfl_up(v, o, 64);
+                if (lane >= o) v += u;
+            }
+            if (e < E) offs[e + 1] = carry + v;
+            carry += __shfl(v, 63, 64);
+        }
+    }
+    __syncthreads();
+    if (blockIdx.x == 0)
+        for (int e = th; e <= E; e += SORT_WAVES * 64) expert_offsets[e] = offs[e];
+    const int g = g0 + wave;
+    if (g >= G) return;
+    const int i = g * 64 + lane;
+    int e = i < n ? ids[i] : -1;
+    if (e >= E) e = -1;
+    if (e < 0) return;                              // (ballots below are taken by the lanes that have a pair)
+    int earlier = before[e];
+    for (int w = 0; w < wave; ++w) earlier += gcnt[(size_t)(g0 + w) * E + e];     // this block's groups before mine
+    unsigned long long same = __ballot(1);
+    for (int b = 0; b < bits; ++b) {
+        const unsigned long long set = __ballot((e >> b) & 1);
+        same &= ((e >> b) & 1) ? set : ~set;
+    }
+    const int dst = offs[e] + earlier + __popcll(same & ((1ull << lane) - 1ull));
+    sorted_token[dst] = i / k;
+    if (sorted_pair) sorted_pair[dst] = i;
+    if (inv) inv[i] = dst;
+}
+
 // few tokens: selection (a wave per token) and the sort in one block of 16 waves
 __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* __restrict__ logits, long ld, int T, int E,
                                                                   int k, int renorm, int gating, int* __restrict__ ids,
@@ -371,11 +469,21 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
     return 0;
 }
 
+// gcnt: room for ceil(n / 64) * E ints (or null: one block does it all, whatever n)
 FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
-                        int* sorted_token, int* sorted_pair, int* inv) {
+                        int* sorted_token, int* sorted_pair, int* inv, int* gcnt) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
     FX_REQUIRE(E >= 1, "moe_align: E=%d", E);
     FX_REQUIRE(E <= 4096, "moe_align: %d experts are more than this kernel's 4096", E);
+    if (gcnt && n > 2048 && (size_t)(E + 1 + E + 2 * SORT_WAVES * E) * 4 <= 60 * 1024) {
+        const int G = (n + 63) / 64, blocks = (G + SORT_WAVES - 1) / SORT_WAVES;
+        moe_count_kernel<<<blocks, SORT_WAVES * 64, (size_t)SORT_WAVES * E * 4, (hipStream_t)stream>>>(ids, n, E, gcnt);
+        FX_CHECK_LAUNCH("moe_count");
+        moe_place_kernel<<<blocks, SORT_WAVES * 64, (size_t)(E + 1 + E + 2 * SORT_WAVES * E) * 4, (hipStream_t)stream>>>(
+            ids, n, k, E, gcnt, expert_offsets, sorted_token, sorted_pair, inv);
+        FX_CHECK_LAUNCH("moe_place");
+        return 0;
+    }
     size_t shm;
     const int per_row = align_groups_per_row(n, E, 60 * 1024, &shm);
     const int nt = n > 4096 ? 1024 : (n > 256 ? 512 : 256);

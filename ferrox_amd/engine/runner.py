@@ -11,6 +11,8 @@ the step, by whoever schedules it.
 """
 from __future__ import annotations
 
+import gc
+
 from dataclasses import dataclass, field
 
 import torch
@@ -83,8 +85,17 @@ class DecodeGraph:
             model.forward(self._context(), caches)              # once eagerly: loads the kernels
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = model.forward(self._context(), caches)
+            # no garbage collection while the stream is recording: a tensor of an earlier step that is freed
+            # then makes the allocator query events, which a recording stream does not allow
+            collecting = gc.isenabled()
+            gc.collect()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = model.forward(self._context(), caches)
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         return self.logits

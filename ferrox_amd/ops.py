@@ -73,7 +73,7 @@ _sigs = {
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
                               c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 5,
-    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
@@ -489,8 +489,10 @@ def moe_align(ids: torch.Tensor, n_experts: int):
     dev = ids.device
     offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
     buf = torch.empty((3, n), dtype=torch.int32, device=dev)
+    # many pairs are sorted by many blocks, which hand each other the counts of every group of 64 pairs
+    gcnt = torch.empty((-(-n // 64), n_experts), dtype=torch.int32, device=dev) if n > 2048 else None
     _call("moe", "fx_moe_align", _stream(), _p(_i32(ids, "ids")), n, k, n_experts, _p(offsets), _p(buf[0]), _p(buf[1]),
-          _p(buf[2]))
+          _p(buf[2]), _p(gcnt))
     return offsets, buf[0], buf[1], buf[2]
 
 

@@ -570,7 +570,7 @@ def test_moe_front(T, H, E, k, renorm, has_gate):
     assert ops.moe_front(rnd(65, H), gamma, eps, router, E, k, renorm, has_gate=has_gate) is None     # too many rows
 
 
-@pytest.mark.parametrize("T,E,k", [(5000, 60, 4), (3000, 700, 2), (1, 3, 1), (130, 1, 1)])
+@pytest.mark.parametrize("T,E,k", [(5000, 60, 4), (3000, 700, 2), (1, 3, 1), (130, 1, 1), (2048, 60, 4), (701, 7, 3), (683, 5, 3)])
 def test_sort_by_expert_at_large_sizes(T, E, k):
     """more pairs than one round of counters holds: rows of several groups; against a stable sort"""
     from ferrox_amd import ops
