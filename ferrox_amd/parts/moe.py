@@ -100,13 +100,13 @@ class SparseMoE(FeedForward):
     @staticmethod
     def _then(then_norm, ctx, n_tokens) -> dict:
         """How the combine prepares the new rows for the next block's norm: `then_norm` is (norm, whether the
-        block takes an ops.ScaleLater).  For few rows the combine also writes them times the norm's weight,
-        with sums of squares, and the product that follows applies the scale: the norm costs no launch.
-        (For many rows a norm kernel of its own is as fast.)"""
+        block takes an ops.ScaleLater).  For up to 64 rows (what the product for few rows takes) the combine also
+        writes them times the norm's weight, with sums of squares, and the product that follows applies the
+        scale: the norm costs no launch.  (For many rows a norm kernel of its own is as fast.)"""
         if then_norm is None or getattr(then_norm[0], "kind", None) != "rmsnorm":
             return {}
         norm, later_ok = then_norm
-        if n_tokens <= 16 and later_ok and ctx.act_dtype == torch.bfloat16:
+        if n_tokens <= 64 and later_ok and ctx.act_dtype == torch.bfloat16:
             return dict(scale_later=(norm.weight, norm.eps, ctx.act_dtype))
         return {}
 
