@@ -563,6 +563,12 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 // W is the A operand: the accumulator of lane (m = lane%16, g) holds
 // C[m][n0 + 4g + r], r = 0..3.
 // ---------------------------------------------------------------------------
+// rsqrt(mean of squares + eps) of a row from the sum of its squares, every step rounded by itself, so that
+// every epilogue that scales its rows gets the same bits whatever the compiler does around it
+__device__ __forceinline__ float row_rstd(float total, int K, float eps) {
+    return __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)K), eps)));
+}
+
 // NORM: the rows of A are float32 and are normed on the way in, y = x * rsqrt(mean(x^2) + eps) * w
 // (ferrox-core/src/matmul.rs:62-69): x * w is rounded to bfloat16 and multiplied, the sums of
 // squares that the waves gather over their parts of K are added up, and the product is scaled by
@@ -581,7 +587,7 @@ __device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
 template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g) {
     static_assert(!DUAL || NW % 2 == 0, "dual mode multiplies two matrices");
-    static_assert(!ROPE || (MT == 1 && NW == 2 && !DUAL && !NORM && EPI == EPI_STORE), "the rope epilogue pairs two sets of columns of one row tile");
+    static_assert(!ROPE || (NW == 2 && !DUAL && !NORM && EPI == EPI_STORE), "the rope epilogue pairs two sets of columns");
     static_assert(!NORM || (!DUAL && EPI == EPI_STORE), "the fused norm feeds a plain product");
     __shared__ float red_ss[NORM ? WAVES : 1][MT][64];
     float ss[MT];
@@ -639,31 +645,38 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         // a dead row reads the first row of A instead: its products land in rows that are never stored
         xrow[mt] = NORM ? (live ? (const bf16*)((const float*)g.A + off) : nullptr) : (const bf16*)g.A + off;
     }
-    // rope epilogue: what thread (lane, wave) needs for its pair of outputs, row lane % 16, column 4 (lane / 16) + wave
-    // of the two sets, is fetched and worked out here, while the weights are on their way
-    float rope_sn = 0.f, rope_cs = 1.f, rope_rstd = 1.f, rope_b0 = 0.f, rope_b1 = 0.f;
-    size_t rope_page = 0;
-    int rope_slot = 0;
+    // rope epilogue: what thread (lane, wave) needs for its pairs of outputs, rows 16 mt + lane % 16, column
+    // 4 (lane / 16) + wave of the two sets, is fetched and worked out here, while the weights are on their way
+    float rope_sn[MT], rope_cs[MT], rope_rstd[MT], rope_b0 = 0.f, rope_b1 = 0.f;
+    size_t rope_page[MT];
+    int rope_slot[MT];
     if constexpr (ROPE) {
-        const int ml = min(r0 + li, r_end - 1), cc = grp * 4 + wave;
-        const int pos = g.rope_positions[ml];
-        if (g.row_ss) {
-            float total = 0.f;
-            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
-            rope_rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
-        }
+        const int cc = grp * 4 + wave;
         if (g.bias) {
             rope_b0 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c0 + cc);
             rope_b1 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c1 + cc);
         }
-        if (rope_rotated) {
-            const int p = 16 * rope_j + cc;
-            const float freq = 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot);
-            sincosf((float)pos * freq, &rope_sn, &rope_cs);
-        }
-        if (rope_head >= g.rope_nh && g.rope_k_pages) {
-            rope_page = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / g.rope_bs];
-            rope_slot = pos % g.rope_bs;
+        const int p = 16 * rope_j + cc;
+        const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int ml = min(r0 + 16 * mt + li, r_end - 1);
+            const int pos = g.rope_positions[ml];
+            rope_rstd[mt] = 1.f;
+            if (g.row_ss) {
+                float total = 0.f;
+                for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
+                rope_rstd[mt] = row_rstd(total, g.K, g.norm_eps);
+            }
+            rope_sn[mt] = 0.f;
+            rope_cs[mt] = 1.f;
+            if (rope_rotated) sincosf((float)pos * freq, &rope_sn[mt], &rope_cs[mt]);
+            rope_page[mt] = 0;
+            rope_slot[mt] = 0;
+            if (rope_head >= g.rope_nh && g.rope_k_pages) {
+                rope_page[mt] = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / g.rope_bs];
+                rope_slot[mt] = pos % g.rope_bs;
+            }
         }
     }
     f32x4_t acc[MT][NW];
@@ -776,43 +789,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     if constexpr (ROPE) {
         static_assert(!ROPE || WAVES == 4, "a wave per accumulator row");
         const int L = lane, r = wave;
-        const int ml = r0 + (L & 15);
-        if (ml >= r_end) return;
-        f32x4_t v0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v1 = v0;
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
-            v0 += red[w][0][L];
-            v1 += red[w][1][L];
-        }
-        const int hd = g.rope_hd, cc = (L >> 4) * 4 + r;
+        const int hd = g.rope_hd, bs = g.rope_bs, cc = (L >> 4) * 4 + r;
         const int d0 = rope_c0 + cc, d1 = rope_c1 + cc;
-        float o0 = v0[r] * rope_rstd, o1 = v1[r] * rope_rstd;
-        if (g.bias) {
-            o0 += rope_b0;
-            o1 += rope_b1;
-        }
-        const float a = bf16_to_float(float_to_bf16(o0)), b = bf16_to_float(float_to_bf16(o1));
-        float y0 = a, y1 = b;
-        if (rope_rotated) {
-            y0 = a * rope_cs - b * rope_sn;
-            y1 = a * rope_sn + b * rope_cs;
-        }
-        if (rope_head < g.rope_nh) {
-            bf16* dst = (bf16*)g.C + (size_t)ml * g.ldc + (size_t)rope_head * hd;
-            from_float(dst + d0, y0);
-            from_float(dst + d1, y1);
-            return;
-        }
-        if (!g.rope_k_pages) return;
-        const int bs = g.rope_bs;
-        if (rope_head < g.rope_nh + g.rope_nkv) {
-            bf16* dst = (bf16*)g.rope_k_pages + ((rope_page * g.rope_nkv + (rope_head - g.rope_nh)) * bs + rope_slot) * hd;
-            from_float(dst + d0, y0);
-            from_float(dst + d1, y1);
-        } else {
-            bf16* dst = (bf16*)g.rope_v_pages + (rope_page * g.rope_nkv + (rope_head - g.rope_nh - g.rope_nkv)) * hd * bs + rope_slot;
-            from_float(dst + (size_t)d0 * bs, y0);
-            from_float(dst + (size_t)d1 * bs, y1);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int ml = r0 + 16 * mt + (L & 15);
+            if (ml >= r_end) continue;
+            f32x4_t v0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v1 = v0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                v0 += red[w][mt * NW][L];
+                v1 += red[w][mt * NW + 1][L];
+            }
+            // product times scale is rounded before the bias is added, as in the plain epilogue (whose bias sits
+            // behind a branch); the empty statement keeps the compiler from fusing the two here
+            float o0 = v0[r] * rope_rstd[mt], o1 = v1[r] * rope_rstd[mt];
+            asm volatile("" : "+v"(o0), "+v"(o1));
+            if (g.bias) {
+                o0 += rope_b0;
+                o1 += rope_b1;
+            }
+            const float a = bf16_to_float(float_to_bf16(o0)), b = bf16_to_float(float_to_bf16(o1));
+            float y0 = a, y1 = b;
+            if (rope_rotated) {
+                y0 = a * rope_cs[mt] - b * rope_sn[mt];
+                y1 = a * rope_sn[mt] + b * rope_cs[mt];
+            }
+            if (rope_head < g.rope_nh) {
+                bf16* dst = (bf16*)g.C + (size_t)ml * g.ldc + (size_t)rope_head * hd;
+                from_float(dst + d0, y0);
+                from_float(dst + d1, y1);
+            } else if (g.rope_k_pages) {
+                if (rope_head < g.rope_nh + g.rope_nkv) {
+                    bf16* dst = (bf16*)g.rope_k_pages + ((rope_page[mt] * g.rope_nkv + (rope_head - g.rope_nh)) * bs + rope_slot[mt]) * hd;
+                    from_float(dst + d0, y0);
+                    from_float(dst + d1, y1);
+                } else {
+                    bf16* dst = (bf16*)g.rope_v_pages + (rope_page[mt] * g.rope_nkv + (rope_head - g.rope_nh - g.rope_nkv)) * hd * bs + rope_slot[mt];
+                    from_float(dst + (size_t)d0 * bs, y0);
+                    from_float(dst + (size_t)d1 * bs, y1);
+                }
+            }
         }
         return;
     }
@@ -834,7 +851,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         if (!NORM && g.row_ss) {
             float total = 0.f;
             for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)m * g.row_ss_n + b];
-            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+            rstd = row_rstd(total, g.K, g.norm_eps);
         }
         if constexpr (NORM) {
             float total = 0.f;
@@ -842,7 +859,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             for (int w = 0; w < WAVES; ++w)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) total += red_ss[w][mt][(L & 15) + 16 * q];
-            rstd = 1.0f / sqrtf(total / (float)g.K + g.norm_eps);
+            rstd = row_rstd(total, g.K, g.norm_eps);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -1033,14 +1050,14 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int m_tile
 #undef FX_SK
 }
 
-// The q/k/v product of up to 16 tokens with the rotation and the cache write in its epilogue (see GemmArgs):
+// The q/k/v product of up to 64 tokens with the rotation and the cache write in its epilogue (see GemmArgs):
 // bfloat16, C [M, (nh + 2 nkv) hd], bias [N] or null, row_ss as in fx_gemm.  head_dim and the rotary dimension
 // are multiples of 32.  k_pages [pages][nkv][bs][hd] and v_pages [pages][nkv][hd][bs], or both null.
 FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, long kb_rows, const void* bias, int bias_dtype,
                        void* C, long ldc, int M, int K, const float* row_ss, int row_ss_n, float eps,
                        const int* positions, const int* token_seq, const int* table, int max_blocks,
                        void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, float theta) {
-    FX_REQUIRE(M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K, "qkv_rope: 1..16 rows of a multiple of 8 elements");
+    FX_REQUIRE(M >= 1 && M <= 64 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K, "qkv_rope: 1..64 rows of a multiple of 8 elements");
     FX_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 32 == 0 && rot >= 0 && rot <= hd && rot % 32 == 0 && bs > 0,
                "qkv_rope: head_dim %d and rotary dimension %d must be multiples of 32", hd, rot);
     const int N = (nh + 2 * nkv) * hd;
@@ -1058,7 +1075,9 @@ FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, lon
     g.rope_k_pages = k_pages; g.rope_v_pages = v_pages;
     g.rope_nh = nh; g.rope_nkv = nkv; g.rope_hd = hd; g.rope_bs = bs; g.rope_rot = rot; g.rope_theta = theta;
     dim3 grid((nh + 2 * nkv) * (hd / 32), 1);
-    gemm_bf16_skinny_kernel<1, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
+    if (M <= 16) gemm_bf16_skinny_kernel<1, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
+    else if (M <= 32) gemm_bf16_skinny_kernel<2, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
+    else gemm_bf16_skinny_kernel<4, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
     FX_CHECK_LAUNCH("qkv_rope");
     return 0;
 }

@@ -307,10 +307,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
 
 
 def can_qkv_rope(x, w, n_rows: int, head_dim: int, rotary_dim: int, interleaved: bool) -> bool:
-    """Whether qkv_rope takes these operands: up to 16 rows of bfloat16 (or a ScaleLater of them), split-half
+    """Whether qkv_rope takes these operands: up to 64 rows of bfloat16 (or a ScaleLater of them), split-half
     rotation, head and rotary dimensions that are multiples of 32, aligned rows."""
     xt = x.x if isinstance(x, ScaleLater) else x
-    return (n_rows <= 16 and not interleaved and head_dim % 32 == 0 and rotary_dim % 32 == 0
+    return (n_rows <= 64 and not interleaved and head_dim % 32 == 0 and rotary_dim % 32 == 0
             and xt.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
             and xt.dim() == 2 and xt.stride(1) == 1 and xt.stride(0) % 8 == 0 and xt.shape[1] % 8 == 0
             and xt.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)

@@ -330,7 +330,8 @@ def test_rope_and_cache_write(dtype, nh, nkv, hd, bs, rot, theta):
 @pytest.mark.parametrize("later", [False, True])
 @pytest.mark.parametrize("T,H,nh,nkv,hd,bs,rot,bias", [(1, 2048, 16, 16, 128, 64, 128, True), (8, 2048, 16, 16, 128, 64, 128, True),
                                                        (16, 264, 6, 2, 64, 16, 32, True), (5, 520, 3, 1, 32, 8, 0, False),
-                                                       (7, 128, 4, 2, 96, 32, 64, True)])
+                                                       (7, 128, 4, 2, 96, 32, 64, True), (30, 264, 6, 2, 64, 16, 64, True),
+                                                       (64, 2048, 16, 16, 128, 64, 128, True), (50, 128, 4, 2, 96, 32, 64, False)])
 def test_qkv_product_that_rotates_and_writes_the_cache(later, T, H, nh, nkv, hd, bs, rot, bias):
     """The q/k/v product with rotation and cache write in its epilogue gives the bits of the product followed
     by rope_kv_write: rotated queries, key pages and value pages; also from rows whose norm's scale is applied
@@ -366,7 +367,7 @@ def test_qkv_product_that_rotates_and_writes_the_cache(later, T, H, nh, nkv, hd,
     assert torch.equal(v1, v2), "value pages"
     got2 = ops.qkv_rope(x, w, b, pos_d, seq_d, table, None, None, nh, nkv, hd, bs, rot, 1e6)     # no pages: queries only
     assert torch.equal(got2[:, :qw], ref[:, :qw])
-    assert not ops.can_qkv_rope(x, w, 17, hd, rot, False) and not ops.can_qkv_rope(x, w, T, hd, rot, True)
+    assert not ops.can_qkv_rope(x, w, 65, hd, rot, False) and not ops.can_qkv_rope(x, w, T, hd, rot, True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
