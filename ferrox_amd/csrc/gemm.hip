@@ -1145,7 +1145,11 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                 (((uintptr_t)A | (uintptr_t)W) % 16 == 0));
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
     FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
-    if (g.vec_ok && (per_group <= 64 || pair_ids)) {
+    // 33..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights faster
+    // than four row tiles per block of the kernel for few rows
+    const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > 32 && K % 64 == 0 &&
+                              !g_no_wide && ceil_div(N, 128) >= 512;
+    if (g.vec_ok && (per_group <= 64 || pair_ids) && !many_columns) {
         const int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
         const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16 + n_always
                                      : M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
@@ -1162,7 +1166,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     }
     const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
     FX_REQUIRE(!g.kb_stride || (per_group > 64 && wide_ok), "gemm: no kernel for weights in slabs of 64 k at these sizes");
-    if (per_group <= 64) {
+    if (per_group <= 64 && !many_columns) {
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else if (g.vec_ok && K % 64 == 0 && !g_no_wide) {
@@ -1173,7 +1177,9 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         };
         auto score = [&](int tm, int tn, double quality) {
             const long t = tiles(tm, tn);
-            return quality * (double)t / (double)(ceil_div(t, 256) * 256L);
+            // plain rows: the share of a tile's rows that exist (an expert's missing row blocks are skipped)
+            const double rows = expert_offsets ? 1.0 : (double)M / (double)((long)ceil_div(M, tm) * tm);
+            return quality * rows * (double)t / (double)(ceil_div(t, 256) * 256L);
         };
         double s256 = score(256, 256, 1.0), s192 = dual ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
                s64 = score(128, 128, 0.7);

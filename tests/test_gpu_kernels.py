@@ -28,7 +28,8 @@ def close(got, want, dtype, what, k=1):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 100, 96), (16, 256, 128), (17, 257, 200), (33, 72, 40),
                                     (64, 64, 64), (130, 300, 520), (257, 129, 1032), (3, 50, 100),
-                                    (130, 300, 512), (257, 129, 1024), (300, 520, 64), (513, 72, 128), (65, 16, 192)])
+                                    (130, 300, 512), (257, 129, 1024), (300, 520, 64), (513, 72, 128), (65, 16, 192),
+                                    (40, 65600, 64), (64, 65536, 128)])
 def test_gemm_plain_and_epilogues(dtype, M, N, K):
     from ferrox_amd import ops
     a, w = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1)
