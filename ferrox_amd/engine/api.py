@@ -33,7 +33,7 @@ class Completion:
 class Engine:
     def __init__(self, model_dir: str | None = None, *, config=None, random_weights: int | None = None,
                  dtype="bfloat16", device="cuda:0", block_size: int = 64, num_pages: int | None = None,
-                 max_seqs: int = 64, max_tokens_per_step: int = 2048, prefill_chunk: int = 512,
+                 max_seqs: int = 64, max_tokens_per_step: int = 2048, prefill_chunk: int = 2048,
                  ctx_size: int = 0):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
