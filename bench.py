@@ -40,6 +40,11 @@ A27B = {
     "max_window_layers": 21, "tie_word_embeddings": False, "qkv_bias": True,
 }
 FULL_LAYERS = 24
+# the other shape of the family (not the default run): Qwen2-57B-A14B
+A14B = dict(A27B, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+            num_experts=64, num_experts_per_tok=8, moe_intermediate_size=2560, shared_expert_intermediate_size=20480,
+            intermediate_size=18944, max_position_embeddings=32768)
+SHAPES = {"a2.7b": ("Qwen1.5-MoE-A2.7B shape", A27B), "57b-a14b": ("Qwen2-57B-A14B shape", A14B)}
 
 
 def log(*a):
@@ -47,12 +52,13 @@ def log(*a):
 
 
 class Bench:
-    def __init__(self, layers: int, dtype: str, block_size: int, max_batch: int, ctx: int, new_tokens: int):
+    def __init__(self, layers: int, dtype: str, block_size: int, max_batch: int, ctx: int, new_tokens: int,
+                 shape: dict = A27B):
         import torch
         from ferrox_amd.engine.loading import random_model
         from ferrox_amd.engine.runner import ModelRunner
         self.torch = torch
-        cfg = dict(A27B)
+        cfg = dict(shape)
         cfg["num_hidden_layers"] = layers
         t0 = time.time()
         self.model = random_model(cfg, seed=0, dtype=dtype, device="cuda:0")
@@ -168,7 +174,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--ctx", type=int, default=2048, help="prompt length of the decode runs")
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (both are reported)")
+    ap.add_argument("--shape", default="a2.7b", choices=sorted(SHAPES), help="layer sizes (the default run is a2.7b)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (both are reported); 0 = all")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode runs")
@@ -182,7 +189,9 @@ def main() -> int:
 
     new_tokens = args.steps + args.warmup + 2
     max_batch = 1 if args.only_prefill else max(args.batch, 1 if args.no_points else 64)
-    b = Bench(args.layers, args.dtype, args.block_size, max_batch, args.ctx, max(new_tokens, 64))
+    shape_name, shape = SHAPES[args.shape]
+    full_layers = shape["num_hidden_layers"]
+    b = Bench(args.layers or full_layers, args.dtype, args.block_size, max_batch, args.ctx, max(new_tokens, 64), shape)
     c = b.cfg
     if args.no_graphs:
         b.runner.use_graphs = False
@@ -205,7 +214,7 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: seeded random token ids, seeded random N(0,0.02) weights",
         "config": {
-            "model": "Qwen1.5-MoE-A2.7B shape", "layers": c.num_hidden_layers, "layers_of_model": FULL_LAYERS,
+            "model": shape_name, "layers": c.num_hidden_layers, "layers_of_model": full_layers,
             "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
             "head_dim": c.head_dim, "experts": c.num_experts, "top_k": c.num_experts_per_tok,
             "moe_intermediate": c.moe_intermediate_size, "shared_intermediate": c.shared_expert_intermediate_size,
