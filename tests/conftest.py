@@ -73,7 +73,19 @@ ODD_F = {
     "rms_norm_eps": 1e-5, "max_position_embeddings": 512, "use_sliding_window": False, "sliding_window": 64,
     "max_window_layers": 2, "tie_word_embeddings": False,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5)}
+# the larger model's layer sizes with few experts: 7 query heads per kv head, eight experts per token, a shared
+# expert eight times as wide as an expert
+WIDE_G = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 1, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "num_experts": 10, "num_experts_per_tok": 8, "norm_topk_prob": False, "moe_intermediate_size": 2560,
+    "shared_expert_intermediate_size": 20480, "intermediate_size": 18944, "decoder_sparse_step": 1,
+    "mlp_only_layers": [], "vocab_size": 500, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 8192, "use_sliding_window": False, "sliding_window": 4096,
+    "max_window_layers": 1, "tie_word_embeddings": False,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5),
+        "G": (WIDE_G, 6)}
 
 
 @pytest.fixture(scope="session")

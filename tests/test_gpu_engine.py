@@ -15,7 +15,7 @@ from conftest import ROOT, TINY
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [1, 7, 16, 33, 70, 45], "B": [3, 17, 40, 64, 90, 120], "C": [2, 35, 66, 130, 51],
-           "D": [40, 75], "E": [150, 260], "F": [5, 70, 33, 150]}
+           "D": [40, 75], "E": [150, 260], "F": [5, 70, 33, 150], "G": [30, 70]}
 # Bounds on |engine - plain| per logit: (absolute, relative to |plain|, relative to the standard
 # deviation of the position's logits).
 # float32: the engine differs from a float64 computation by float32 rounding only.
@@ -304,9 +304,9 @@ def test_preemption_and_seeded_sampling_through_the_entry_point(model_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["D", "E", "F"])
+@pytest.mark.parametrize("name", ["D", "E", "F", "G"])
 def test_production_layer_sizes(model_folders, name, dtype):
-    """one or two layers of the sizes the engine is built for (D, E) and of widths that allow no
+    """one or two layers of the sizes the engine is built for (D, E, G) and of widths that allow no
     16-byte loads (F), pages of 64: whole prompts (tiled matrix kernels, MFMA prefill attention),
     then mixed portions and single tokens (streaming kernels, split decode attention, recorded
     decode steps)"""
