@@ -74,6 +74,23 @@ __device__ __forceinline__ float load_as_float(const void* p, int dtype, size_t 
     return dtype == FX_F32 ? ((const float*)p)[i] : bf16_to_float(((const bf16*)p)[i]);
 }
 
+// N elements first, first + STRIDE, ... (zero from `limit` on) of such a tensor.  The branch on the type
+// is taken once around all N loads, so that they are on their way together: taken per element it makes
+// every load wait for the one before.
+template <typename WT, int N, int STRIDE>
+__device__ __forceinline__ void load_strided_typed(const WT* p, int first, int limit, float (&out)[N]) {
+    WT raw[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) raw[i] = p[min(first + i * STRIDE, limit - 1)];
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = first + i * STRIDE < limit ? to_float(raw[i]) : 0.f;
+}
+template <int N, int STRIDE>
+__device__ __forceinline__ void load_strided_as_float(const void* p, int dtype, int first, int limit, float (&out)[N]) {
+    if (dtype == FX_F32) load_strided_typed<float, N, STRIDE>((const float*)p, first, limit, out);
+    else load_strided_typed<bf16, N, STRIDE>((const bf16*)p, first, limit, out);
+}
+
 // ---- wave (64 lanes) and block reductions in a fixed order ------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

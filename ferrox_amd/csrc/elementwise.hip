@@ -58,8 +58,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
         for (int i = 0; i < 16; ++i) {
             const int c = threadIdx.x + i * 256;
             xv[i] = c < H ? x[c] : 0.f;
-            wv[i] = c < H ? load_as_float(w, w_dtype, c) : 0.f;
         }
+        load_strided_as_float<16, 256>(w, w_dtype, threadIdx.x, H, wv);
 #pragma unroll
         for (int i = 0; i < 16; ++i) ss += xv[i] * xv[i];
         ss = block_sum<4>(ss, red);
@@ -287,20 +287,44 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h,
     __shared__ float red[4];
     const int t = blockIdx.x, n_tok = gridDim.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
-    float v = 0.f;
+    float v = 0.f, nw = 0.f;
     if (c < H) {
+        // the loads of eight terms are asked for together and added in order: the sums are those of a plain loop
+        const float h_old = h[(size_t)t * H + c];
         float acc = 0.f;
-        for (int j = 0; j < k; ++j) acc += w[t * k + j] * y[(size_t)(inv ? inv[t * k + j] : t * k + j) * H + c];
+        for (int j0 = 0; j0 < k; j0 += 8) {
+            float wv[8], yv[8];
+            int from[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int j = min(j0 + u, k - 1);
+                from[u] = inv ? inv[t * k + j] : t * k + j;
+                wv[u] = w[t * k + j];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) yv[u] = y[(size_t)from[u] * H + c];
+            if (j0 == 0 && xg) nw = load_as_float(norm_w, norm_dtype, c);     // (waits for its load: after the others have left)
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (j0 + u < k) acc += wv[u] * yv[u];
+        }
         if (shared) {      // routed first, then shared (lib.rs:746-750); the shared output may come as `slabs` partial sums [slab][T][H]
             float sh = 0.f;
-            for (int s = 0; s < slabs; ++s) sh += shared[((size_t)s * n_tok + t) * H + c];
+            for (int s0 = 0; s0 < slabs; s0 += 8) {
+                float sv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) sv[u] = shared[((size_t)min(s0 + u, slabs - 1) * n_tok + t) * H + c];
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (s0 + u < slabs) sh += sv[u];
+            }
             acc += (gate ? gate[t] : 1.f) * sh;
         }
-        v = h[(size_t)t * H + c] + acc;
+        v = h_old + acc;
         h[(size_t)t * H + c] = v;
     }
     if (!xg) return;
-    if (c < H) from_float(xg + (size_t)t * H + c, v * load_as_float(norm_w, norm_dtype, c));
+    if (c < H) from_float(xg + (size_t)t * H + c, v * nw);
     const float total = block_sum<4>(v * v, red);
     if (threadIdx.x == 0) ss[t * gridDim.y + blockIdx.y] = total;
 }

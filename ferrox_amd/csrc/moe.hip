@@ -388,44 +388,88 @@ __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
     const int t = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_rows = E + has_gate, chunks = H >> 3;
 
-    // this wave's two router rows: their first loads leave before the norm is done
+    // this wave's two router rows
     const int e_a = blockIdx.x * FRONT_ROWS + wave, e_b = e_a + FRONT_WAVES;
     const bf16* wa = e_a < n_rows ? W + (size_t)e_a * H : nullptr;
     const bf16* wb = e_b < n_rows ? W + (size_t)e_b * H : nullptr;
-    uint4 pa = make_uint4(0, 0, 0, 0), pb = pa;
-    if (lane < chunks) {
-        if (wa) pa = *(const uint4*)(wa + lane * 8);
-        if (wb) pb = *(const uint4*)(wb + lane * 8);
-    }
-
     const float* row = h + (size_t)t * ldh;
-    float ss = 0.f;
-    for (int c = tid; c < H; c += FRONT_THREADS) {
-        const float v = row[c];
-        xs[c] = v;
-        ss += v * v;
-    }
-    ss = block_sum<FRONT_WAVES>(ss, red);
-    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
-    for (int c = tid; c < H; c += FRONT_THREADS) {
-        const bf16 b = float_to_bf16(xs[c] * scale * load_as_float(gamma, gamma_dtype, c));
-        if (blockIdx.x == 0) x_out[(size_t)t * H + c] = b;
-        xs[c] = bf16_to_float(b);
-    }
-    __syncthreads();
-
     float acc_a = 0.f, acc_b = 0.f;
-    for (int c = lane; c < chunks; c += 64) {
-        const int cn = c + 64;
-        uint4 na = make_uint4(0, 0, 0, 0), nb = na;
-        if (cn < chunks) {
-            if (wa) na = *(const uint4*)(wa + cn * 8);
-            if (wb) nb = *(const uint4*)(wb + cn * 8);
+
+    if (H <= FRONT_THREADS * 16) {
+        // Usual widths: everything this thread reads from memory (its part of the router's rows, of the
+        // residual row and of the norm's weights) is asked for at once, so that the kernel waits for memory
+        // once.  Elements go to threads and are summed as in rmsnorm_kernel: the same bits.
+        constexpr int NC = FRONT_THREADS * 16 / 8 / 64;      // 16-byte pieces of a router row per lane
+        uint4 pa[NC], pb[NC];
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int c = lane + 64 * i;
+            pa[i] = (wa && c < chunks) ? *(const uint4*)(wa + c * 8) : make_uint4(0, 0, 0, 0);
+            pb[i] = (wb && c < chunks) ? *(const uint4*)(wb + c * 8) : make_uint4(0, 0, 0, 0);
         }
-        acc_a += dot8(pa, xs + c * 8);
-        acc_b += dot8(pb, xs + c * 8);
-        pa = na;
-        pb = nb;
+        float xv[16], gv[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = tid + i * FRONT_THREADS;
+            xv[i] = c < H ? row[c] : 0.f;
+        }
+        load_strided_as_float<16, FRONT_THREADS>(gamma, gamma_dtype, tid, H, gv);
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ss += xv[i] * xv[i];
+        ss = block_sum<FRONT_WAVES>(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = tid + i * FRONT_THREADS;
+            if (c < H) {
+                const bf16 b = float_to_bf16(xv[i] * scale * gv[i]);
+                if (blockIdx.x == 0) x_out[(size_t)t * H + c] = b;
+                xs[c] = bf16_to_float(b);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {          // k in the order of the loop below
+            const int c = lane + 64 * i;
+            if (c < chunks) {
+                acc_a += dot8(pa[i], xs + c * 8);
+                acc_b += dot8(pb[i], xs + c * 8);
+            }
+        }
+    } else {
+        // their first loads leave before the norm is done
+        uint4 pa = make_uint4(0, 0, 0, 0), pb = pa;
+        if (lane < chunks) {
+            if (wa) pa = *(const uint4*)(wa + lane * 8);
+            if (wb) pb = *(const uint4*)(wb + lane * 8);
+        }
+        float ss = 0.f;
+        for (int c = tid; c < H; c += FRONT_THREADS) {
+            const float v = row[c];
+            xs[c] = v;
+            ss += v * v;
+        }
+        ss = block_sum<FRONT_WAVES>(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+        for (int c = tid; c < H; c += FRONT_THREADS) {
+            const bf16 b = float_to_bf16(xs[c] * scale * load_as_float(gamma, gamma_dtype, c));
+            if (blockIdx.x == 0) x_out[(size_t)t * H + c] = b;
+            xs[c] = bf16_to_float(b);
+        }
+        __syncthreads();
+        for (int c = lane; c < chunks; c += 64) {
+            const int cn = c + 64;
+            uint4 na = make_uint4(0, 0, 0, 0), nb = na;
+            if (cn < chunks) {
+                if (wa) na = *(const uint4*)(wa + cn * 8);
+                if (wb) nb = *(const uint4*)(wb + cn * 8);
+            }
+            acc_a += dot8(pa, xs + c * 8);
+            acc_b += dot8(pb, xs + c * 8);
+            pa = na;
+            pb = nb;
+        }
     }
     acc_a = wave_sum(acc_a);
     acc_b = wave_sum(acc_b);
