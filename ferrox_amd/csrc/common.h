@@ -70,8 +70,33 @@ __device__ __forceinline__ void from_float(float* p, float v) { *p = v; }
 __device__ __forceinline__ void from_float(bf16* p, float v) { *p = float_to_bf16(v); }
 
 // load one element of a tensor whose element type is only known at run time
+// Without a branch: two 16-bit loads (the halves of a float, or the same bfloat16 twice).  A branch on the
+// type around a load makes the compiler wait for that load before the paths join, so a thread that
+// loads several such values would wait for each in turn.  In two steps, so that a caller can ask for
+// its other loads between the fetch and the first use.
+struct RawElement {
+    unsigned lo, hi, shift, keep_hi;
+};
+__device__ __forceinline__ RawElement fetch_element(const void* p, int dtype, size_t i) {
+    const unsigned short* q = (const unsigned short*)p;
+    const bool f32 = dtype == FX_F32;
+    const size_t e = f32 ? 2 * i : i;
+    // float: lo | hi << 16; bfloat16: lo << 16.  The three constants pass through an empty statement so that
+    // the compiler cannot tell the cases apart and bring the branch back.
+    int second = f32 ? 1 : 0;
+    RawElement r;
+    r.shift = f32 ? 0u : 16u;
+    r.keep_hi = f32 ? 0xffff0000u : 0u;
+    asm volatile("" : "+v"(second), "+v"(r.shift), "+v"(r.keep_hi));
+    r.lo = q[e];
+    r.hi = q[e + second];
+    return r;
+}
+__device__ __forceinline__ float element_as_float(const RawElement& r) {
+    return __uint_as_float((r.lo << r.shift) | ((r.hi << 16) & r.keep_hi));
+}
 __device__ __forceinline__ float load_as_float(const void* p, int dtype, size_t i) {
-    return dtype == FX_F32 ? ((const float*)p)[i] : bf16_to_float(((const bf16*)p)[i]);
+    return element_as_float(fetch_element(p, dtype, i));
 }
 
 // N elements first, first + STRIDE, ... (zero from `limit` on) of such a tensor.  The branch on the type

@@ -301,6 +301,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 #undef FX_MULTIPLY
 
     // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
+    float bias_v[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) bias_v[j] = 0.f;
+    if (!DUAL && g.bias) load_strided_as_float<NT, 16>(g.bias, g.bias_dtype, n0 + wn * WN + (lane & 15), g.N, bias_v);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -321,7 +325,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                     const int n = n0 + wn * WN + j * 16 + (lane & 15);
                     if (n >= g.N) continue;
                     float v = acc[i][j][r];
-                    if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
+                    if (g.bias) v += bias_v[j];
                     if (EPI == EPI_STORE) {
                         from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
                     } else if (EPI == EPI_STORE_F32) {
@@ -516,13 +520,40 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 #undef FX_LOOP
 
     // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
+    float bias_v[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) bias_v[j] = 0.f;
+    if (!DUAL && g.bias) load_strided_as_float<NT, 16>(g.bias, g.bias_dtype, n0 + wn * WN + (lane & 15), g.N, bias_v);
+    // Where each of this lane's rows goes (and its scale) is fetched for all rows at once, and so are the old
+    // values that a row block adds to: a load inside the loops below would be waited for before the next leaves.
+    int m_of[MT][4];
+    float scale_of[MT][4];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
+            const int safe = (ml < r_end && ml < r0 + TM) ? ml : r0;
+            m_of[i][r] = g.c_rows ? g.c_rows[safe] : safe;
+            scale_of[i][r] = (EPI == EPI_RESID && g.row_scale) ? g.row_scale[safe] : 1.f;
+        }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
+        float old[4][NT];
+        if (EPI == EPI_RESID) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const int n = min(n0 + wn * WN + j * 16 + (lane & 15), g.N - 1);
+                    old[r][j] = ((const float*)g.C)[(size_t)m_of[i][r] * g.ldc + n];
+                }
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
             if (ml >= r_end || ml >= r0 + TM) continue;
-            const int m = g.c_rows ? g.c_rows[ml] : ml;
+            const int m = m_of[i][r];
             if (DUAL) {
 #pragma unroll
                 for (int j = 0; j < NT; j += 2) {
@@ -536,14 +567,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
                     const int n = n0 + wn * WN + j * 16 + (lane & 15);
                     if (n >= g.N) continue;
                     float v = acc[i][j][r];
-                    if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
+                    if (g.bias) v += bias_v[j];
                     if (EPI == EPI_STORE) {
                         from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
                     } else if (EPI == EPI_STORE_F32) {
                         ((float*)g.C)[(size_t)m * g.ldc + n] = v;
                     } else {
-                        if (g.row_scale) v *= g.row_scale[ml];
-                        ((float*)g.C)[(size_t)m * g.ldc + n] += v;
+                        if (g.row_scale) {
+                            v *= scale_of[i][r];
+                            asm volatile("" : "+v"(v));      // rounded before it is added (no fused multiply-add)
+                        }
+                        ((float*)g.C)[(size_t)m * g.ldc + n] = old[r][j] + v;
                     }
                 }
             }
@@ -563,10 +597,27 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 // W is the A operand: the accumulator of lane (m = lane%16, g) holds
 // C[m][n0 + 4g + r], r = 0..3.
 // ---------------------------------------------------------------------------
-// rsqrt(mean of squares + eps) of a row from the sum of its squares, every step rounded by itself, so that
-// every epilogue that scales its rows gets the same bits whatever the compiler does around it
+// rsqrt(mean of squares + eps) of a row from the sum of its squares.  Division and sqrtf are the correctly
+// rounded ones (the compiler's default for HIP; __fsqrt_rn is NOT: it is the approximate instruction, whose
+// result the compiler refines in some kernels and not in others), so every epilogue that scales its rows
+// gets the same bits.
 __device__ __forceinline__ float row_rstd(float total, int K, float eps) {
-    return __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)K), eps)));
+    const float mean = total / (float)K;
+    return 1.0f / sqrtf(mean + eps);
+}
+
+// p[0] + p[1] + ... in that order; eight loads leave together (a plain loop would wait for each in turn)
+__device__ __forceinline__ float sum_in_order(const float* p, int n) {
+    float total = 0.f;
+    for (int b0 = 0; b0 < n; b0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[min(b0 + u, n - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (b0 + u < n) total += v[u];
+    }
+    return total;
 }
 
 // NORM: the rows of A are float32 and are normed on the way in, y = x * rsqrt(mean(x^2) + eps) * w
@@ -652,31 +703,43 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     int rope_slot[MT];
     if constexpr (ROPE) {
         const int cc = grp * 4 + wave;
-        if (g.bias) {
-            rope_b0 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c0 + cc);
-            rope_b1 = load_as_float(g.bias, g.bias_dtype, rope_head * g.rope_hd + rope_c1 + cc);
+        const bool to_pages = rope_head >= g.rope_nh && g.rope_k_pages;
+        // first every load that depends on nothing, then the page ids, which need position and sequence
+        int row_of[MT], pos[MT], seq[MT];
+        float total[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            row_of[mt] = min(r0 + 16 * mt + li, r_end - 1);
+            pos[mt] = g.rope_positions[row_of[mt]];
+            seq[mt] = to_pages ? g.rope_token_seq[row_of[mt]] : 0;
         }
+        // (without a bias the same loads read the positions instead: a branch around them would wait for them)
+        const void* bias_or = g.bias ? g.bias : (const void*)g.rope_positions;
+        const int bias_dt = g.bias ? g.bias_dtype : FX_F32;
+        const RawElement e0 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c0 + cc : 0);
+        const RawElement e1 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c1 + cc : 0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            total[mt] = g.row_ss ? sum_in_order(g.row_ss + (size_t)row_of[mt] * g.row_ss_n, g.row_ss_n) : 0.f;
+        rope_b0 = element_as_float(e0);
+        rope_b1 = element_as_float(e1);
         const int p = 16 * rope_j + cc;
         const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const int ml = min(r0 + 16 * mt + li, r_end - 1);
-            const int pos = g.rope_positions[ml];
-            rope_rstd[mt] = 1.f;
-            if (g.row_ss) {
-                float total = 0.f;
-                for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)ml * g.row_ss_n + b];
-                rope_rstd[mt] = row_rstd(total, g.K, g.norm_eps);
-            }
-            rope_sn[mt] = 0.f;
-            rope_cs[mt] = 1.f;
-            if (rope_rotated) sincosf((float)pos * freq, &rope_sn[mt], &rope_cs[mt]);
             rope_page[mt] = 0;
             rope_slot[mt] = 0;
-            if (rope_head >= g.rope_nh && g.rope_k_pages) {
-                rope_page[mt] = (size_t)g.rope_table[(size_t)g.rope_token_seq[ml] * g.rope_max_blocks + pos / g.rope_bs];
-                rope_slot[mt] = pos % g.rope_bs;
+            if (to_pages) {
+                rope_page[mt] = (size_t)g.rope_table[(size_t)seq[mt] * g.rope_max_blocks + pos[mt] / g.rope_bs];
+                rope_slot[mt] = pos[mt] % g.rope_bs;
             }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            rope_rstd[mt] = g.row_ss ? row_rstd(total[mt], g.K, g.norm_eps) : 1.f;
+            rope_sn[mt] = 0.f;
+            rope_cs[mt] = 1.f;
+            if (rope_rotated) sincosf((float)pos[mt] * freq, &rope_sn[mt], &rope_cs[mt]);
         }
     }
     f32x4_t acc[MT][NW];
@@ -848,11 +911,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         if (pairs ? ml < 0 : ml >= r_end) continue;
         const int m = (g.c_rows && !pairs) ? g.c_rows[ml] : ml;
         float rstd = 1.f;
-        if (!NORM && g.row_ss) {
-            float total = 0.f;
-            for (int b = 0; b < g.row_ss_n; ++b) total += g.row_ss[(size_t)m * g.row_ss_n + b];
-            rstd = row_rstd(total, g.K, g.norm_eps);
-        }
+        float bias_v[4] = {0.f, 0.f, 0.f, 0.f};          // of columns n0 + 16 a + 4 (L / 16) + 0..3
+        if (!DUAL && g.bias) load_strided_as_float<4, 1>(g.bias, g.bias_dtype, n0 + a * 16 + (L >> 4) * 4, g.N, bias_v);
+        if (!NORM && g.row_ss) rstd = row_rstd(sum_in_order(g.row_ss + (size_t)m * g.row_ss_n, g.row_ss_n), g.K, g.norm_eps);
         if constexpr (NORM) {
             float total = 0.f;
 #pragma unroll
@@ -861,23 +922,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
                 for (int q = 0; q < 4; ++q) total += red_ss[w][mt][(L & 15) + 16 * q];
             rstd = row_rstd(total, g.K, g.norm_eps);
         }
+        // what a row block adds to, and its scale: fetched together, ahead of the stores
+        float old[4] = {0.f, 0.f, 0.f, 0.f}, row_scale = 1.f;
+        if (EPI == EPI_RESID) {
+            if (g.row_scale) row_scale = g.row_scale[ml];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                old[r] = ((const float*)g.C)[(size_t)m * g.ldc + min(n0 + a * 16 + (L >> 4) * 4 + r, g.N - 1)];
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n0 + a * 16 + (L >> 4) * 4 + r;
             if (n >= g.N) continue;
             float o = v[r] * rstd;
+            asm volatile("" : "+v"(o));          // the product is rounded before the bias is added (no fused multiply-add)
             if (DUAL) {
                 from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(o) * v2[r]);
                 continue;
             }
-            if (g.bias) o += load_as_float(g.bias, g.bias_dtype, n);
+            if (g.bias) o += bias_v[r];
             if (EPI == EPI_STORE) {
                 from_float((bf16*)g.C + (size_t)m * g.ldc + n, o);
             } else if (EPI == EPI_STORE_F32) {
                 ((float*)g.C)[(size_t)m * g.ldc + n] = o;
             } else {
-                if (g.row_scale) o *= g.row_scale[ml];
-                ((float*)g.C)[(size_t)m * g.ldc + n] += o;
+                if (g.row_scale) {
+                    o *= row_scale;
+                    asm volatile("" : "+v"(o));
+                }
+                ((float*)g.C)[(size_t)m * g.ldc + n] = old[r] + o;
             }
         }
     }
