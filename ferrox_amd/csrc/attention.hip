@@ -384,6 +384,16 @@ __device__ __forceinline__ uint4 keep_keys(uint4 v, int first_key, int kv_begin,
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// All ones if `ok`, else zero, as a value the compiler knows nothing about: data that is loaded and then
+// ANDed with it is loaded always.  With a plain `ok ? x : 0` the compiler loads only where ok holds, behind a
+// branch, and waits for that load before it goes on: a tile's loads would then leave one at a time.
+__device__ __forceinline__ uint32_t opaque_mask(bool ok) {
+    uint32_t m = ok ? 0xffffffffu : 0u;
+    asm volatile("" : "+v"(m));
+    return m;
+}
+__device__ __forceinline__ uint4 and_mask(uint4 x, uint32_t m) { return make_uint4(x.x & m, x.y & m, x.z & m, x.w & m); }
+
 template <int HD>   // compile-time bound of head_dim (a.hd <= HD)
 struct WaveAttn {
     static constexpr int KS = HD / 32;   // k-steps of S^T = K Q^T
@@ -423,34 +433,44 @@ struct WaveAttn {
         const int vkey = vlive ? kg : safe_group;
         int vblk, vslot;
         page_slot(a, vkey, vblk, vslot);
-        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)pl.page(vblk) * a.nkv + kvh) * hd * bs + vslot;
+        // every page id of the tile is looked up before the first load leaves: a lookup that stands between two
+        // groups of loads makes the second group wait for the first
+        const int vpage = pl.page(vblk);
+        int kpage[4], kslots[4];
+        bool klives[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            const int key0 = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
+            klives[kb] = key0 >= kv_begin && key0 < kv_end;
+            int kblk;
+            page_slot(a, klives[kb] ? key0 : safe_group, kblk, kslots[kb]);
+            kpage[kb] = pl.page(kblk);
+        }
+        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)vpage * a.nkv + kvh) * hd * bs + vslot;
         uint4 vv[EARLY_V ? CB : 1][2];
+        const uint32_t vmask = opaque_mask(vlive);
         if (EARLY_V) {
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const int d = 16 * cb + li;
                 const bf16* vr = vbase + (size_t)(d < hd ? d : 0) * bs;
                 const uint4 x0 = *(const uint4*)vr, x1 = *(const uint4*)(vr + 8);
-                const bool ok = vlive && d < hd;
-                vv[cb][0] = ok ? x0 : make_uint4(0, 0, 0, 0);
-                vv[cb][1] = ok ? x1 : make_uint4(0, 0, 0, 0);
+                const uint32_t ok = vmask & opaque_mask(d < hd);
+                vv[cb][0] = and_mask(x0, ok);
+                vv[cb][1] = and_mask(x1, ok);
             }
         }
         f32x4_t sc[4];
         uint4 kf[4][KS];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-            const int key0 = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
-            const bool klive = key0 >= kv_begin && key0 < kv_end;
-            const int key = klive ? key0 : safe_group;
-            int kblk, kslot;
-            page_slot(a, key, kblk, kslot);
-            const bf16* kr = (const bf16*)a.k_pages + (((size_t)pl.page(kblk) * a.nkv + kvh) * bs + kslot) * hd;
+            const bf16* kr = (const bf16*)a.k_pages + (((size_t)kpage[kb] * a.nkv + kvh) * bs + kslots[kb]) * hd;
+            const uint32_t kmask = opaque_mask(klives[kb]);
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
                 const int d = 32 * u + 8 * g;
                 const uint4 x = *(const uint4*)(kr + (d < hd ? d : 0));
-                kf[kb][u] = (klive && d < hd) ? x : make_uint4(0, 0, 0, 0);
+                kf[kb][u] = and_mask(x, kmask & opaque_mask(d < hd));
             }
         }
 #pragma unroll
@@ -479,9 +499,9 @@ struct WaveAttn {
                 const int d = 16 * cb + li;
                 const bf16* vr = vbase + (size_t)(d < hd ? d : 0) * bs;
                 const uint4 x0 = *(const uint4*)vr, x1 = *(const uint4*)(vr + 8);
-                const bool ok = vlive && d < hd;
-                v0 = ok ? x0 : make_uint4(0, 0, 0, 0);
-                v1 = ok ? x1 : make_uint4(0, 0, 0, 0);
+                const uint32_t ok = vmask & opaque_mask(d < hd);
+                v0 = and_mask(x0, ok);
+                v1 = and_mask(x1, ok);
             }
             if (edge) {
                 v0 = keep_keys(v0, kg, kv_begin, kv_end);
