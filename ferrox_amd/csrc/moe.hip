@@ -275,10 +275,16 @@ __global__ __launch_bounds__(SORT_WAVES * 64) void moe_place_kernel(const int* _
     // wave w adds the groups w, w + SORT_WAVES, ...: all of them, and those before g0
     for (int e = lane; e < E; e += 64) {
         int all = 0, early = 0;
-        for (int g = wave; g < G; g += SORT_WAVES) {
-            const int c = gcnt[(size_t)g * E + e];
-            all += c;
-            if (g < g0) early += c;
+        for (int gb = wave; gb < G; gb += 8 * SORT_WAVES) {       // eight counts are fetched together
+            int c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) c[u] = gcnt[(size_t)min(gb + u * SORT_WAVES, G - 1) * E + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int g = gb + u * SORT_WAVES;
+                if (g < G) all += c[u];
+                if (g < G && g < g0) early += c[u];
+            }
         }
         part[(wave * 2) * E + e] = all;
         part[(wave * 2 + 1) * E + e] = early;
