@@ -34,6 +34,49 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
                                              float* __restrict__ gate_out, int* ids_copy, long es = 1) {
     const int lane = threadIdx.x & 63;
     if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E * es]));
+    if (E <= 64) {
+        // a lane per expert: the same sums and comparisons as below (whose loops then run once), with the scores
+        // in registers, so that no round waits for LDS or for the store of the round before
+        const bool mine = lane < E;
+        const float x = mine ? row[lane * es] : 0.f;
+        float sc;
+        if (gating == GATE_SOFTMAX) {
+            const float mx = wave_max(mine ? x : NEG_INFINITY_F);
+            const float ex = mine ? expf(x - mx) : 0.f;
+            const float sum = wave_sum(ex);
+            sc = ex / sum;
+        } else {
+            sc = 1.0f / (1.0f + expf(-x));
+        }
+        if (!mine) sc = -1.f;           // below every score, like the loop's start value
+        float wsum = 0.f, my_w = 0.f;
+        int my_id = 0;
+        for (int j = 0; j < k; ++j) {
+            float best = sc;
+            int bi = mine ? lane : 0x7fffffff;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, 64);
+                const int oi = __shfl_xor(bi, o, 64);
+                if (ob > best || (ob == best && oi < bi)) {
+                    best = ob;
+                    bi = oi;
+                }
+            }
+            if (lane == j) {
+                my_w = best;
+                my_id = bi;
+            }
+            if (lane == bi) sc = -2.f;  // scores are >= 0; taken out of the race
+            wsum += best;
+        }
+        if (lane < k) {
+            ids[t * k + lane] = my_id;
+            if (ids_copy) ids_copy[t * k + lane] = my_id;
+            weights[t * k + lane] = renorm ? my_w / wsum : my_w;
+        }
+        return;
+    }
     if (gating == GATE_SOFTMAX) {
         float mx = NEG_INFINITY_F;
         for (int e = lane; e < E; e += 64) mx = fmaxf(mx, row[e * es]);
