@@ -278,7 +278,9 @@ FX_API int fx_cast(void* stream, int src_dtype, const void* src, int dst_dtype, 
 // xg != nullptr: the new rows are also written as xg = round(h * norm_w) (no scale yet) with each block's sum
 // of squares of its 256 columns in ss[t * gridDim.y + blockIdx.y]: the product that reads xg scales its
 // rows by rsqrt(sum / H + eps), which is RMSNorm with the rounding of the norm that a product applies itself.
-template <typename T>
+// VEC = 4: a thread takes four neighbouring columns with 16-byte loads (H % 4 == 0, aligned rows); a block then
+// covers 1024 columns, and each of its waves one group of 256 for the sums of squares.
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                                           const int* __restrict__ inv, const float* __restrict__ w,
                                                           const float* __restrict__ shared, const float* __restrict__ gate,
@@ -286,14 +288,26 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h,
                                                           int norm_dtype, T* __restrict__ xg, float* __restrict__ ss) {
     __shared__ float red[4];
     const int t = blockIdx.x, n_tok = gridDim.x;
-    const int c = blockIdx.y * 256 + threadIdx.x;
-    float v = 0.f, nw = 0.f;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * VEC;
+    auto load = [&](const float* p, float (&out)[VEC]) {
+        if constexpr (VEC == 4) {
+            const float4 q = *(const float4*)p;
+            out[0] = q.x; out[1] = q.y; out[2] = q.z; out[3] = q.w;
+        } else {
+            out[0] = *p;
+        }
+    };
+    float v[VEC], nw[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = nw[i] = 0.f;
     if (c < H) {
         // the loads of eight terms are asked for together and added in order: the sums are those of a plain loop
-        const float h_old = h[(size_t)t * H + c];
-        float acc = 0.f;
+        float h_old[VEC], acc[VEC];
+        load(h + (size_t)t * H + c, h_old);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
         for (int j0 = 0; j0 < k; j0 += 8) {
-            float wv[8], yv[8];
+            float wv[8], yv[8][VEC];
             int from[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -302,31 +316,59 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ h,
                 wv[u] = w[t * k + j];
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) yv[u] = y[(size_t)from[u] * H + c];
-            if (j0 == 0 && xg) nw = load_as_float(norm_w, norm_dtype, c);     // (waits for its load: after the others have left)
+            for (int u = 0; u < 8; ++u) load(y + (size_t)from[u] * H + c, yv[u]);
+            if (j0 == 0 && xg) {     // (waits for its load: after the others have left)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) nw[i] = load_as_float(norm_w, norm_dtype, c + i);
+            }
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (j0 + u < k) acc += wv[u] * yv[u];
+                if (j0 + u < k) {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) acc[i] = fmaf(wv[u], yv[u][i], acc[i]);
+                }
         }
         if (shared) {      // routed first, then shared (lib.rs:746-750); the shared output may come as `slabs` partial sums [slab][T][H]
-            float sh = 0.f;
-            for (int s0 = 0; s0 < slabs; s0 += 8) {
-                float sv[8];
+            float sh[VEC];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) sv[u] = shared[((size_t)min(s0 + u, slabs - 1) * n_tok + t) * H + c];
+            for (int i = 0; i < VEC; ++i) sh[i] = 0.f;
+            for (int s0 = 0; s0 < slabs; s0 += 8) {
+                float sv[8][VEC];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) load(shared + ((size_t)min(s0 + u, slabs - 1) * n_tok + t) * H + c, sv[u]);
 #pragma unroll
                 for (int u = 0; u < 8; ++u)
-                    if (s0 + u < slabs) sh += sv[u];
+                    if (s0 + u < slabs) {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) sh[i] += sv[u][i];
+                    }
             }
-            acc += (gate ? gate[t] : 1.f) * sh;
+            const float gt = gate ? gate[t] : 1.f;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(gt, sh[i], acc[i]);
         }
-        v = h_old + acc;
-        h[(size_t)t * H + c] = v;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = h_old[i] + acc[i];
+        if constexpr (VEC == 4) *(float4*)(h + (size_t)t * H + c) = make_float4(v[0], v[1], v[2], v[3]);
+        else h[(size_t)t * H + c] = v[0];
     }
     if (!xg) return;
-    if (c < H) from_float(xg + (size_t)t * H + c, v * nw);
-    const float total = block_sum<4>(v * v, red);
-    if (threadIdx.x == 0) ss[t * gridDim.y + blockIdx.y] = total;
+    if (c < H) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) from_float(xg + (size_t)t * H + c + i, v[i] * nw[i]);
+    }
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sq = fmaf(v[i], v[i], sq);
+    const int n_groups = (H + 255) / 256;
+    if constexpr (VEC == 4) {
+        const float total = wave_sum(sq);
+        const int group = blockIdx.y * 4 + (threadIdx.x >> 6);
+        if ((threadIdx.x & 63) == 0 && group < n_groups) ss[t * n_groups + group] = total;
+    } else {
+        const float total = block_sum<4>(sq, red);
+        if (threadIdx.x == 0) ss[t * n_groups + blockIdx.y] = total;
+    }
 }
 
 // norm_w != nullptr: x_out = round(h * norm_w) of the new rows, in out_dtype, and ss[t][b] = the sum of squares of
@@ -337,18 +379,27 @@ FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv
     FX_REQUIRE(T >= 0 && H > 0 && k > 0 && slabs >= 1, "moe_combine: bad sizes");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(T, (H + 255) / 256);
+    // few rows: a thread per column spreads the row's loads over more waves, which is what counts then
+    const bool vec = (long)T * H >= (1L << 18) && H % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                     (!shared || ((uintptr_t)shared % 16) == 0);
+    const dim3 grid(T, vec ? (H + 1023) / 1024 : (H + 255) / 256);
+#define FX_COMBINE(TYPE, XOUT) \
+    do { \
+        if (vec) moe_combine_kernel<TYPE, 4><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, XOUT, ss); \
+        else moe_combine_kernel<TYPE, 1><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, XOUT, ss); \
+    } while (0)
     if (norm_w) {
         FX_REQUIRE(x_out && ss, "moe_combine: the rows for the norm need places to write");
         FX_REQUIRE(norm_dtype == FX_F32 || norm_dtype == FX_BF16, "moe_combine: unknown norm weight dtype %d", norm_dtype);
         FX_REQUIRE(out_dtype == FX_F32 || out_dtype == FX_BF16, "moe_combine: unknown output dtype %d", out_dtype);
-        if (out_dtype == FX_F32)
-            moe_combine_kernel<float><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, (float*)x_out, ss);
-        else
-            moe_combine_kernel<bf16><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, norm_w, norm_dtype, (bf16*)x_out, ss);
+        if (out_dtype == FX_F32) FX_COMBINE(float, (float*)x_out);
+        else FX_COMBINE(bf16, (bf16*)x_out);
     } else {
-        moe_combine_kernel<float><<<grid, 256, 0, s>>>(h, y, inv, w, shared, gate, H, k, slabs, nullptr, 0, nullptr, nullptr);
+        norm_w = nullptr;
+        ss = nullptr;
+        FX_COMBINE(float, (float*)nullptr);
     }
+#undef FX_COMBINE
     FX_CHECK_LAUNCH("moe_combine");
     return 0;
 }

@@ -68,6 +68,35 @@ def test_combine_that_leaves_the_scale_to_the_product(T, H, N, k, S):
     close(two, want, torch.bfloat16, "norm, then product")
 
 
+@pytest.mark.parametrize("T,H,k,S,sorted_rows", [(130, 2048, 4, 4, False), (300, 1000, 3, 0, True), (140, 2052, 2, 1, True)])
+def test_combine_of_many_rows_equals_that_of_few(T, H, k, S, sorted_rows):
+    """Many rows go four columns to a thread, few rows one: the same bits in the residual stream and in the rows
+    for the next norm, the same sums of squares up to the order of their terms."""
+    from ferrox_amd import ops
+    assert T * H >= 1 << 18 and (T // 2 + 1) * H < 1 << 18
+    h = rnd(T, H, scale=2.0)
+    y, wts = rnd(T * k, H, seed=1), torch.rand(T, k, generator=torch.Generator().manual_seed(2)).to(DEV)
+    inv = torch.randperm(T * k, generator=torch.Generator().manual_seed(3)).to(torch.int32).to(DEV) if sorted_rows else None
+    shared = rnd(S, T, H, seed=3) if S else None
+    gate = torch.rand(T, generator=torch.Generator().manual_seed(4)).to(DEV) if S else None
+    gamma = (1.0 + rnd(H, seed=5, scale=0.2)).to(torch.bfloat16)
+    h_all = h.clone()
+    all_rows = ops.moe_combine(h_all, y, inv, wts, k, shared=shared, gate=gate, scale_later=(gamma, 1e-6, torch.bfloat16))
+    cut = T // 2
+    for lo, hi in ((0, cut), (cut, T)):
+        h_part = h[lo:hi].clone()
+        part = ops.moe_combine(h_part, y if inv is not None else y[lo * k:hi * k], inv[lo * k:hi * k] if inv is not None else None,
+                               wts[lo:hi].contiguous(), k, shared=shared[:, lo:hi].contiguous() if S else None,
+                               gate=gate[lo:hi].contiguous() if S else None, scale_later=(gamma, 1e-6, torch.bfloat16))
+        assert torch.equal(h_all[lo:hi], h_part), "residual stream"
+        assert torch.equal(all_rows.x[lo:hi], part.x), "rows for the next norm"
+        close(all_rows.ss[lo:hi], part.ss, torch.float32, "sums of squares per 256 columns")
+    want = h.double().cpu() + (wts.double().cpu()[:, :, None] * (y.double().cpu()[inv.long().cpu()] if inv is not None else y.double().cpu()).view(T, k, H)).sum(1)
+    if S:
+        want = want + gate.double().cpu()[:, None] * shared.double().cpu().sum(0)
+    close(h_all, want, torch.float32, "combined rows")
+
+
 @pytest.mark.parametrize("tile", [256, 192, 128, 64])
 @pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
 def test_gemm_every_wide_tile(tile, M, N, K):
