@@ -116,6 +116,14 @@ __device__ __forceinline__ void load_strided_as_float(const void* p, int dtype, 
     else load_strided_typed<bf16, N, STRIDE>((const bf16*)p, first, limit, out);
 }
 
+// The rotation of one pair by an angle, (a, b) -> (a cos - b sin, a sin + b cos), with its roundings spelled
+// out (one product rounded, then a fused multiply-add), so that every kernel that rotates gets the same bits
+// whatever the compiler would have made of the plain expression.
+__device__ __forceinline__ void rotate_pair(float a, float b, float cs, float sn, float& y0, float& y1) {
+    y0 = fmaf(a, cs, -(b * sn));
+    y1 = fmaf(a, sn, b * cs);
+}
+
 // ---- wave (64 lanes) and block reductions in a fixed order ------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta) {
+    int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta, int vec8) {
     __shared__ float cs[128], sn[128];     // rot / 2 <= 128
     const int tid = threadIdx.x;
     const int half = rot >> 1;
@@ -135,15 +135,45 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
             k_dst = k_pages + ((size_t)page * nkv * bs + pos % bs) * hd;      // + kv head * bs * hd
         }
         const int heads = nh + (k_pages ? nkv : 0);
-        for (int i = part * 256 + tid; i < heads * half; i += step) {
-            const int head = i / half, p = i - head * half;
-            const int ia = interleaved ? 2 * p : p;
-            const int ib = interleaved ? 2 * p + 1 : p + half;
-            const T* src = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)(head - nh) * hd;
-            T* dst = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k_dst + (size_t)(head - nh) * bs * hd;
-            const float a = to_float(src[ia]), b = to_float(src[ib]);
-            from_float(dst + ia, a * cs[p] - b * sn[p]);
-            from_float(dst + ib, a * sn[p] + b * cs[p]);
+        if (vec8) {
+            // bfloat16, split halves, everything a multiple of eight: eight neighbouring pairs to a thread, 16 bytes
+            // per load and store
+            const int h8 = half >> 3;
+            for (int i = part * 256 + tid; i < heads * h8; i += step) {
+                const int head = i / h8, p = (i - head * h8) * 8;
+                const T* src = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)(head - nh) * hd;
+                T* dst = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k_dst + (size_t)(head - nh) * bs * hd;
+                const uint4 ua = *(const uint4*)(src + p), ub = *(const uint4*)(src + p + half);
+                const uint32_t wa[4] = {ua.x, ua.y, ua.z, ua.w}, wb[4] = {ub.x, ub.y, ub.z, ub.w};
+                uint32_t oa[4], ob[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float y0[2], y1[2];
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh) {
+                        const float a = __uint_as_float(hh ? wa[e] & 0xffff0000u : wa[e] << 16);
+                        const float b = __uint_as_float(hh ? wb[e] & 0xffff0000u : wb[e] << 16);
+                        rotate_pair(a, b, cs[p + 2 * e + hh], sn[p + 2 * e + hh], y0[hh], y1[hh]);
+                    }
+                    oa[e] = pack_bf16(y0[0], y0[1]);
+                    ob[e] = pack_bf16(y1[0], y1[1]);
+                }
+                *(uint4*)(dst + p) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
+                *(uint4*)(dst + p + half) = make_uint4(ob[0], ob[1], ob[2], ob[3]);
+            }
+        } else {
+            for (int i = part * 256 + tid; i < heads * half; i += step) {
+                const int head = i / half, p = i - head * half;
+                const int ia = interleaved ? 2 * p : p;
+                const int ib = interleaved ? 2 * p + 1 : p + half;
+                const T* src = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)(head - nh) * hd;
+                T* dst = head < nh ? q + (size_t)t * ldq + (size_t)head * hd : k_dst + (size_t)(head - nh) * bs * hd;
+                const float a = to_float(src[ia]), b = to_float(src[ib]);
+                float y0, y1;
+                rotate_pair(a, b, cs[p], sn[p], y0, y1);
+                from_float(dst + ia, y0);
+                from_float(dst + ib, y1);
+            }
         }
         if (k_pages && rot < hd) {         // beyond the rotated dimensions
             const int rest = hd - rot;
@@ -199,16 +229,18 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
     const long n_blocks = (long)T * split + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
     FX_REQUIRE(n_blocks < (1L << 31), "rope_kv_write: too many tokens and heads for one launch");
     const unsigned blocks = (unsigned)n_blocks;
+    const int vec8 = dtype == FX_BF16 && !interleaved && rot % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 && ldk % 8 == 0 &&
+                     ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && (!k_pages || ((uintptr_t)k_pages % 16) == 0);
     if (dtype == FX_F32)
         rope_kv_write_kernel<float><<<blocks, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
                                                            positions, token_seq, block_table, max_blocks,
                                                            (float*)k_pages, (float*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                           interleaved, theta);
+                                                           interleaved, theta, 0);
     else if (dtype == FX_BF16)
         rope_kv_write_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
                                                           positions, token_seq, block_table, max_blocks,
                                                           (bf16*)k_pages, (bf16*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                          interleaved, theta);
+                                                          interleaved, theta, vec8);
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("rope_kv_write");

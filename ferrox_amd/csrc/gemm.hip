@@ -874,10 +874,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             }
             const float a = bf16_to_float(float_to_bf16(o0)), b = bf16_to_float(float_to_bf16(o1));
             float y0 = a, y1 = b;
-            if (rope_rotated) {
-                y0 = a * rope_cs[mt] - b * rope_sn[mt];
-                y1 = a * rope_sn[mt] + b * rope_cs[mt];
-            }
+            if (rope_rotated) rotate_pair(a, b, rope_cs[mt], rope_sn[mt], y0, y1);
             if (rope_head < g.rope_nh) {
                 bf16* dst = (bf16*)g.C + (size_t)ml * g.ldc + (size_t)rope_head * hd;
                 from_float(dst + d0, y0);

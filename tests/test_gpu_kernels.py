@@ -357,6 +357,44 @@ def test_rope_and_cache_write(dtype, nh, nkv, hd, bs, rot, theta):
         assert torch.equal(v_pages[page, :, :, p % bs].reshape(-1), v[t]), f"v page token {t}"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,bs,rot,seq_lens", [(4, 2, 128, 64, 128, [300, 7, 330]), (3, 1, 80, 64, 48, [640, 5]),
+                                                       (2, 2, 64, 16, 64, [530, 40]), (2, 1, 96, 128, 96, [520])])
+def test_rope_and_cache_write_of_long_prompts(dtype, nh, nkv, hd, bs, rot, seq_lens):
+    """Many tokens, eight pairs to a thread: pages that begin or end inside a sequence, page sizes other than 64,
+    tokens of another sequence between."""
+    theta = 1e6
+    n_pages = sum(-(-L // bs) for L in seq_lens) + 2
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, seq_lens, theta, rot, n_pages)
+    assert len(toks) >= 512
+    T = len(toks)
+    p = pos.double().cpu()
+    freq = 1.0 / theta ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot)
+    ang = p[:, None] * freq[None, :]                                   # plain.rope_neox, all tokens at once
+    def rotated(x, heads):
+        x = x.double().cpu().reshape(T, heads, hd)
+        a, b = x[..., :rot // 2], x[..., rot // 2:rot]
+        c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        return torch.cat([a * c - b * s_, a * s_ + b * c, x[..., rot:]], dim=-1)
+    assert torch.allclose(plain.rope_neox(q[5].double().cpu().reshape(nh, hd)[:, :rot], int(pos[5]), theta),
+                          rotated(q, nh)[5, :, :rot])                  # the formula above is the plain one
+    # the angle is position x frequency in float32 (ferrox-core/src/attention.rs:20-32): at position p it is known to
+    # about p x 2^-23, and so are the rotated values (times their size); bfloat16 rounds coarser than that anyway
+    def near(got, want, what):
+        got, want = got.double().cpu(), want.double().cpu()
+        bound = float(want.abs().max()) * ((1e-5 if dtype == torch.float32 else 1e-2) + float(p.max()) * 2.0 ** -22)
+        err = float((got - want).abs().max())
+        assert err <= bound, f"{what}: max error {err:.3e} > {bound:.3e}"
+    near(q_rot.reshape(T, nh, hd), rotated(q, nh), "rotated queries")
+    page_of = table.cpu()[seq.cpu().long(), (pos.cpu() // bs).long()].long()
+    slot = (pos.cpu() % bs).long()
+    near(k_pages.cpu()[page_of, :, slot, :], rotated(k, nkv), "key pages")
+    assert torch.equal(v_pages.cpu()[page_of, :, :, slot], v.cpu().reshape(T, nkv, hd)), "value pages"
+    used = torch.zeros(n_pages, bs, dtype=torch.bool)
+    used[page_of, slot] = True
+    assert bool(torch.isnan(v_pages.cpu().float().permute(0, 3, 1, 2)[~used]).all()), "slots past the sequences stay untouched"
+
+
 @pytest.mark.parametrize("later", [False, True])
 @pytest.mark.parametrize("T,H,nh,nkv,hd,bs,rot,bias", [(1, 2048, 16, 16, 128, 64, 128, True), (8, 2048, 16, 16, 128, 64, 128, True),
                                                        (16, 264, 6, 2, 64, 16, 32, True), (5, 520, 3, 1, 32, 8, 0, False),
