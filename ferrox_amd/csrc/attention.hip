@@ -564,18 +564,20 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int p = a.positions[tok];
+    // the page ids of the whole chunk are copied, whatever part of it the position and the window leave: the copy
+    // then does not wait for the position to arrive (entries past the sequence's pages are read and never used)
+    __shared__ int page_copy[PAGE_COPY];
+    int first_blk, last_blk, unused;
+    page_slot(a, split * a.chunk, first_blk, unused);
+    page_slot(a, (split + 1) * a.chunk - 1, last_blk, unused);
+    first_blk = min(first_blk, a.max_blocks - 1);
+    last_blk = min(last_blk, a.max_blocks - 1);
+    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
     const int kv_begin = max(a.window > 0 ? max(0, p - a.window + 1) : 0, split * a.chunk);
     const int kv_end = min(p + 1, (split + 1) * a.chunk);
     const int n = min(16, group - hb * 16);        // query heads in this block
     const int h0 = kvh * group + hb * 16;
     const bool empty = kv_begin >= kv_end;
-    __shared__ int page_copy[PAGE_COPY];
-    int first_blk = 0, last_blk = -1, unused;
-    if (!empty) {
-        page_slot(a, kv_begin, first_blk, unused);
-        page_slot(a, kv_end - 1, last_blk, unused);
-    }
-    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
     WaveAttn<HD> w;
     const bool row_ok = li < n;
     w.init(row_ok && !empty ? (const bf16*)a.q + (size_t)tok * a.ldq + (size_t)(h0 + li) * hd : nullptr, hd);
