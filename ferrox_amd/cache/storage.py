@@ -14,14 +14,13 @@ from ..parts.base import LayerCache
 
 class CacheStorage:
     def __init__(self, model, manager, dtype: torch.dtype, device):
-        from ..engine.model import group_key
         self.caches: list[LayerCache] = []
         self.bytes = 0
         bs = manager.block_size
         for i, e in enumerate(model.schedule):
             mixer = model.blocks[e.layer].mixer
             shapes = mixer.page_shapes(bs)
-            key = group_key(mixer) if shapes else None
+            key = mixer.cache_group()[0] if shapes else None
             state = {}
             for name, (shape, sdtype) in mixer.state_shapes().items():
                 state[name] = torch.zeros((manager.slots.n_slots, *shape), dtype=sdtype or dtype, device=device)

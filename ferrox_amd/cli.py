@@ -91,23 +91,31 @@ def main(argv=None) -> int:
     if args.verbose_prompt:
         print("prompt tokens:", prompt_ids, file=sys.stderr)
 
+    import torch
+    if not torch.cuda.is_available():
+        print("error: no GPU is visible; this engine has no CPU path", file=sys.stderr)
+        return 2
+    from .csrc.build import KernelBuildError
     from .engine.api import Engine
     from .sampling.sampler import SamplingParams
 
-    t0 = time.time()
-    engine = Engine(args.model, dtype=args.dtype, device=args.device, block_size=args.block_size,
-                    num_pages=args.num_pages or None, max_seqs=4, ctx_size=args.ctx_size,
-                    max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk)
-    print(f"load time: {time.time() - t0:.2f} s", file=sys.stderr)
-    if engine.model.config.defaulted_keys:
-        print("config keys defaulted: " + ", ".join(engine.model.config.defaulted_keys), file=sys.stderr)
-    seed = args.seed if args.seed >= 0 else (time.time_ns() & 0x7FFFFFFFFFFFFFFF)       # run.rs:462-471
-    params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
-                            args.presence_penalty, args.frequency_penalty, seed)
-    t1 = time.time()
+    # everything that can be wrong with the folder, the configuration, the weights or the request ends the
+    # program with one message and exit code 2 (the reference bails the same way, run.rs:598-607)
     try:
+        t0 = time.time()
+        engine = Engine(args.model, dtype=args.dtype, device=args.device, block_size=args.block_size,
+                        num_pages=args.num_pages or None, max_seqs=4, ctx_size=args.ctx_size,
+                        max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk)
+        print(f"load time: {time.time() - t0:.2f} s", file=sys.stderr)
+        defaulted = getattr(getattr(engine.model, "config", None), "defaulted_keys", ())
+        if defaulted:                                                                    # run.rs:520-528
+            print("config keys defaulted: " + ", ".join(defaulted), file=sys.stderr)
+        seed = args.seed if args.seed >= 0 else (time.time_ns() & 0x7FFFFFFFFFFFFFFF)       # run.rs:462-471
+        params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
+                                args.presence_penalty, args.frequency_penalty, seed)
+        t1 = time.time()
         out = engine.generate_detailed([prompt_ids], args.n_predict, params, ignore_eos=args.ignore_eos)[0]
-    except ValueError as e:
+    except (ValueError, OSError, KernelBuildError) as e:     # ConfigError, CheckpointError, SafetensorsError are ValueErrors
         print(f"error: {e}", file=sys.stderr)
         return 2
     dt = time.time() - t1

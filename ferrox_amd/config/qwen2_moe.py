@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+from .. import limits
 from .base import ConfigError, ConfigReader
 
 
@@ -118,6 +119,14 @@ class Qwen2MoeConfig:
             bad(f"head_dim {self.head_dim} must be even for rotary pairs")
         if self.num_experts and not 1 <= self.num_experts_per_tok <= self.num_experts:
             bad(f"num_experts_per_tok {self.num_experts_per_tok} must lie in 1..num_experts {self.num_experts}")
+        if self.num_experts > limits.MOE_MAX_EXPERTS:
+            bad(f"num_experts {self.num_experts} is more than the routing kernels take ({limits.MOE_MAX_EXPERTS})")
+        if self.num_experts_per_tok > limits.MOE_MAX_TOP_K:
+            bad(f"num_experts_per_tok {self.num_experts_per_tok} is more than the routing kernels take "
+                f"({limits.MOE_MAX_TOP_K})")
+        if self.head_dim % limits.HEAD_DIM_STEP or self.head_dim > limits.HEAD_DIM_MAX:
+            bad(f"head_dim {self.head_dim}: the attention kernels take multiples of {limits.HEAD_DIM_STEP} "
+                f"up to {limits.HEAD_DIM_MAX}")
         for l in self.mlp_only_layers:
             if not 0 <= l < self.num_hidden_layers:
                 bad(f"mlp_only_layers names layer {l}, the model has {self.num_hidden_layers}")

@@ -924,7 +924,7 @@ __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
                 if (kt0 + key < kv_begin || kt0 + key >= kv_end)
                     st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
             }
-            __builtin_amdgcn_s_barrier();
+            lds_barrier();      // the zeros are in LDS (a bare s_barrier does not wait for this wave's stores) before any wave reads values
         }
         if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;           // nothing in this tile for this wave's rows
         f32x4_t sc[4];
@@ -966,8 +966,13 @@ __global__ __launch_bounds__(256) void attn_mfma_direct_kernel(AttnArgs a) {
     }
 }
 
-static int g_direct = 2;     // measurement only: 0 keeps prefill on the kernel that stages tiles through registers; 2, 3: stages
-FX_API void fx_attn_set_direct(int stages) { g_direct = stages; }
+// Switch for tests and measurement (ferrox_amd/debug.py is its one caller); the product path never sets it.
+static int g_direct = 2;     // "direct_stages": 0 keeps prefill on the kernel that stages tiles through registers; 2 (default), 3: stages
+FX_API int fx_debug_set(const char* key, int value) {
+    if (!strcmp(key, "direct_stages")) { g_direct = value; return 0; }
+    FX_REQUIRE(false, "attention: no debug switch '%s' (direct_stages)", key);
+    return 1;
+}
 
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
     return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
@@ -1018,15 +1023,11 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
 
 // Single queries.  part_o has n_items*nh*splits*hd floats, part_ml n_items*nh*splits*2;
 // splits * chunk must cover every position + 1.
-FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
-                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
-                          const int* positions, const int* item_seq, const int* item_tok, int n_items,
-                          int nh, int nkv, int hd, int bs, int window, float scale,
-                          float* part_o, float* part_ml, int splits, int chunk, int waves) {
-    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window)) return 1;
-    FX_REQUIRE(splits > 0 && chunk > 0 && chunk % 64 == 0, "attn_decode: chunk %d must be a positive multiple of 64", chunk);
-    FX_REQUIRE(splits <= 8192, "attn_decode: %d chunks are more than the merge kernel takes (8192)", splits);
-    if (n_items <= 0) return 0;
+static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
+                              const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
+                              const int* positions, const int* item_seq, const int* item_tok, int n_items,
+                              int nh, int nkv, int hd, int bs, int window, float scale,
+                              float* part_o, float* part_ml, int splits, int chunk, int waves) {
     AttnArgs a = {};
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
@@ -1065,4 +1066,23 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     }
     FX_CHECK_LAUNCH("attn_decode");
     return 0;
+}
+
+static int attn_decode_check(int dtype, int nh, int nkv, int hd, int bs, int window, int splits, int chunk) {
+    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window)) return 1;
+    FX_REQUIRE(splits > 0 && chunk > 0 && chunk % 64 == 0, "attn_decode: chunk %d must be a positive multiple of 64", chunk);
+    FX_REQUIRE(splits <= 8192, "attn_decode: %d chunks are more than the merge kernel takes (8192)", splits);
+    return 0;
+}
+
+FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
+                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
+                          const int* positions, const int* item_seq, const int* item_tok, int n_items,
+                          int nh, int nkv, int hd, int bs, int window, float scale,
+                          float* part_o, float* part_ml, int splits, int chunk, int waves) {
+    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, splits, chunk)) return 1;
+    if (n_items <= 0) return 0;
+    return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
+                              item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
+                              chunk, waves);
 }

@@ -27,7 +27,7 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
 HOST_LIBRARIES = ("host_runtime",)
-LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling") + HOST_LIBRARIES
+LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling", "probe") + HOST_LIBRARIES
 HEADERS = ("common.h",)
 
 _loaded: dict[str, ctypes.CDLL] = {}

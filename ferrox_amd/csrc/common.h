@@ -10,6 +10,7 @@
 #include <stdio.h>
 #include <stdarg.h>
 #include <math.h>
+#include <string.h>
 
 #define FX_API extern "C" __attribute__((visibility("default")))
 

@@ -61,6 +61,7 @@ struct GemmArgs {
     void* rope_v_pages;
     int rope_nh, rope_nkv, rope_hd, rope_bs, rope_rot;
     float rope_theta;
+    const float* rope_freq_factors;   // rot/2 floats or null: the angle of pair i is divided by rope_freq_factors[i]
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
@@ -725,6 +726,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         rope_b1 = element_as_float(e1);
         const int p = 16 * rope_j + cc;
         const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
+        const float freq_div = rope_rotated && g.rope_freq_factors ? g.rope_freq_factors[p] : 1.f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             rope_page[mt] = 0;
@@ -739,7 +741,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             rope_rstd[mt] = g.row_ss ? row_rstd(total[mt], g.K, g.norm_eps) : 1.f;
             rope_sn[mt] = 0.f;
             rope_cs[mt] = 1.f;
-            if (rope_rotated) sincosf((float)pos[mt] * freq, &rope_sn[mt], &rope_cs[mt]);
+            if (rope_rotated) {
+                float angle = (float)pos[mt] * freq;
+                if (g.rope_freq_factors) angle = angle / freq_div;
+                sincosf(angle, &rope_sn[mt], &rope_cs[mt]);
+            }
         }
     }
     f32x4_t acc[MT][NW];
@@ -1065,11 +1071,17 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 #undef FX_TILED
 }
 
-static int g_skinny_nw = 0;        // measurement only: 1 or 2 sets of weight rows per wave whatever the sizes
-FX_API void fx_gemm_set_skinny(int nw) { g_skinny_nw = nw; }
-static int g_no_wide = 0;   // measurement only: 1 sends many-row products to the older tiled kernel
-static int g_wide_force = 0;   // measurement only: 256, 192, 128 or 64 picks that wide tile whatever the sizes
-FX_API void fx_gemm_set_wide(int on) { g_no_wide = !on; g_wide_force = on > 1 ? on : 0; }
+// Switches for tests and measurement (ferrox_amd/debug.py is their one caller): they pick, whatever the sizes,
+// a kernel variant that the sizes would otherwise choose.  The product path never sets them.
+static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per wave of the product for few rows (0: by the sizes)
+static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
+static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
+FX_API int fx_debug_set(const char* key, int value) {
+    if (!strcmp(key, "skinny_sets")) { g_skinny_nw = value; return 0; }
+    if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
+    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, wide)", key);
+    return 1;
+}
 
 template <int TMB, int TN, int NS, int NSA = NS>
 static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
@@ -1126,7 +1138,8 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int m_tile
 FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, long kb_rows, const void* bias, int bias_dtype,
                        void* C, long ldc, int M, int K, const float* row_ss, int row_ss_n, float eps,
                        const int* positions, const int* token_seq, const int* table, int max_blocks,
-                       void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, float theta) {
+                       void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, float theta,
+                       const float* freq_factors) {
     FX_REQUIRE(M >= 1 && M <= 64 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K, "qkv_rope: 1..64 rows of a multiple of 8 elements");
     FX_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 32 == 0 && rot >= 0 && rot <= hd && rot % 32 == 0 && bs > 0,
                "qkv_rope: head_dim %d and rotary dimension %d must be multiples of 32", hd, rot);
@@ -1144,6 +1157,7 @@ FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, lon
     g.rope_positions = positions; g.rope_token_seq = token_seq; g.rope_table = table; g.rope_max_blocks = max_blocks;
     g.rope_k_pages = k_pages; g.rope_v_pages = v_pages;
     g.rope_nh = nh; g.rope_nkv = nkv; g.rope_hd = hd; g.rope_bs = bs; g.rope_rot = rot; g.rope_theta = theta;
+    g.rope_freq_factors = freq_factors;
     dim3 grid((nh + 2 * nkv) * (hd / 32), 1);
     if (M <= 16) gemm_bf16_skinny_kernel<1, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);
     else if (M <= 32) gemm_bf16_skinny_kernel<2, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);

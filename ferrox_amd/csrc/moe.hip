@@ -48,6 +48,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         } else {
             sc = 1.0f / (1.0f + expf(-x));
         }
+        if (!(sc >= 0.f)) sc = 0.f;     // a NaN logit makes every score NaN: such scores count as zero, so a choice stays in range
         if (!mine) sc = -1.f;           // below every score, like the loop's start value
         float wsum = 0.f, my_w = 0.f;
         int my_id = 0;
@@ -100,7 +101,8 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         float best = -1.f;
         int bi = 0x7fffffff;
         for (int e = lane; e < E; e += 64) {
-            const float v = score[e];
+            float v = score[e];
+            if (!(v >= 0.f) && v != -2.f) v = 0.f;   // NaN counts as zero (see above): some expert in range is always found
             if (v > best) {  // ascending e within a lane: the first maximum is kept
                 best = v;
                 bi = e;

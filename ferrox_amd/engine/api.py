@@ -32,13 +32,17 @@ class Completion:
 
 class Engine:
     def __init__(self, model_dir: str | None = None, *, config=None, random_weights: int | None = None,
-                 dtype="bfloat16", device="cuda:0", block_size: int = 64, num_pages: int | None = None,
+                 model=None, dtype="bfloat16", device="cuda:0", block_size: int = 64, num_pages: int | None = None,
                  max_seqs: int = 64, max_tokens_per_step: int = 2048, prefill_chunk: int = 2048,
                  ctx_size: int = 0):
+        """One of: `model_dir` (config.json + safetensors), `config` with `random_weights=<seed>`, or `model`,
+        a model that is loaded already (its dtype and device are taken)."""
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         self.dtype = parse_dtype(dtype)
-        if model_dir is not None:
+        if model is not None:
+            self.model, self.dtype = model, model.act_dtype
+        elif model_dir is not None:
             self.model = load_model(model_dir, self.dtype, device)
         elif config is not None and random_weights is not None:
             self.model = random_model(config, int(random_weights), self.dtype, device)
@@ -55,6 +59,7 @@ class Engine:
         self.prefill_chunk = prefill_chunk
         self.eos_token_id = spec.eos_token_id
         self.last_stats: dict = {}
+        self.time_steps = False      # True: every step is bracketed by events and last_stats also says where the time went
 
     @property
     def vocab_size(self) -> int:
@@ -94,6 +99,9 @@ class Engine:
             sched.add(r)
         t0 = time.time()
         n_steps = n_tokens = 0
+        marks = []            # per step: [event at its first device operation, event after its last launch, all decodes?]
+        if self.time_steps:
+            self.runner.before_launch = lambda: marks[-1][0].record()
         try:
             while sched.has_work():
                 batch = sched.schedule()
@@ -103,21 +111,40 @@ class Engine:
                     break
                 entries = [StepEntry(s.request.id, sched.step_tokens(s), [s.n_tokens - 1] if s.samples else [])
                            for s in batch]
+                if self.time_steps:
+                    marks.append([torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True),
+                                  all(s.n_tokens == 1 for s in batch)])
                 logits = self.runner.step(entries)
                 sampled = {}
                 rows = [s.request for s in batch if s.samples]
+                done = marks[-1][1].record if self.time_steps else None
                 if rows:
                     toks = sample_rows(logits, [r.params for r in rows], [r.rng for r in rows],
-                                       [r.generated for r in rows])
+                                       [r.generated for r in rows], launched=done)
                     sampled = {r.id: t for r, t in zip(rows, toks)}
+                elif done is not None:
+                    done()
                 sched.commit(batch, sampled)
                 n_steps += 1
                 n_tokens += sum(s.n_tokens for s in batch)
         finally:
+            self.runner.before_launch = None
             for r in list(sched.running):
                 self.runner.release(r.id)
         self.last_stats = {"steps": n_steps, "tokens": n_tokens, "seconds": time.time() - t0,
                            "preemptions": sched.n_preemptions}
+        if self.time_steps and marks:
+            # from a step's first device operation to the end of its last kernel, as the GPU saw it; between the
+            # end of one step and the first operation of the next the GPU waits for the host (reading the ids
+            # back, scheduling, packing): `host_gap_seconds`.  Waits inside a step (kernels launched one by one
+            # faster than they are submitted) are not seen this way.
+            torch.cuda.synchronize()
+            spans = [a.elapsed_time(b) * 1e-3 for a, b, _ in marks]
+            gaps = [marks[i][1].elapsed_time(marks[i + 1][0]) * 1e-3 for i in range(len(marks) - 1)]
+            dec = [i for i, m in enumerate(marks) if m[2]]
+            self.last_stats.update(gpu_seconds=sum(spans), host_gap_seconds=sum(gaps), decode_steps=len(dec),
+                                   decode_gpu_seconds=sum(spans[i] for i in dec),
+                                   decode_gap_seconds=sum(gaps[i - 1] for i in dec if i > 0))
         return [Completion(r.generated, r.finish_reason or "aborted", len(r.prompt), r.n_preempted) for r in reqs]
 
 

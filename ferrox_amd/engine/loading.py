@@ -6,7 +6,7 @@ import os
 
 import torch
 
-from ..models.registry import config_from_folder, resolve
+from ..models.registry import architecture_of, config_from_folder, resolve
 from ..weights.random_init import RandomSource
 from ..weights.safetensors_io import Checkpoint, LazyTensor, write_safetensors
 from .model import Model
@@ -42,7 +42,7 @@ def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: floa
         arch = resolve(config)
         config = arch.config_class.from_dict(config)
     else:
-        arch = resolve({"architectures": [config.architecture]})
+        arch = architecture_of(config)
     act = parse_dtype(dtype)
     model = Model(arch.build_spec(config, None))
     model.config = config
@@ -56,7 +56,7 @@ def write_random_model(config, folder: str, seed: int, dtype="bfloat16", std: fl
         arch = resolve(config)
         config = arch.config_class.from_dict(config)
     else:
-        arch = resolve({"architectures": [config.architecture]})
+        arch = architecture_of(config)
     store = parse_dtype(dtype)
     os.makedirs(folder, exist_ok=True)
     model = Model(arch.build_spec(config, None))

@@ -4,14 +4,10 @@ from __future__ import annotations
 
 import torch
 
+from .. import debug
 from ..parts.base import (BLOCKS, EMBEDDINGS, HEADS, NORMS, LayerCache, ModelSpec, StepContext, walk_params,
                           walk_parts)
 from ..weights.loader import check_names, upload
-
-
-def group_key(mixer):
-    """Mixers with the same need share pages' ids: all keys, or the last W."""
-    return ("window", int(mixer.window)) if mixer.window else ("full",)
 
 
 class Model:
@@ -37,7 +33,7 @@ class Model:
                     raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache}, which must be an "
                                      f"earlier entry with a cache of its own")
                 a, b = self.blocks[e.layer].mixer, self.blocks[self.schedule[e.cache].layer].mixer
-                if group_key(a) != group_key(b) or a.page_shapes(16) != b.page_shapes(16):
+                if a.cache_group() != b.cache_group() or a.page_shapes(16) != b.page_shapes(16):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache}: "
                                      f"their mixers keep different pages")
         self.act_dtype = None
@@ -89,26 +85,31 @@ class Model:
         for e in self.schedule:
             m = self.blocks[e.layer].mixer
             if m.page_shapes(16):
-                groups[group_key(m)] = m.window
+                key, window = m.cache_group()
+                if groups.setdefault(key, window) != window:
+                    raise ValueError(f"two mixers name the cache group {key!r} with windows {groups[key]} and {window}")
         return groups
 
     # ---- forward ---------------------------------------------------------
     def forward(self, ctx: StepContext, caches: list):
+        debug.region("embed")
         h = self.embedding.forward(ctx.token_ids)
         # blocks that chain their norms: the block before may already have applied this block's first norm
         # to the rows it finished (in the kernel that finished them)
         normed = None
         for i, e in enumerate(self.schedule):
             block = self.blocks[e.layer]
-            if getattr(block, "chains_norms", False):
+            if block.chains_norms:
                 nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
                 then = (nxt.first_norm, nxt.takes_scale_later(ctx.act_dtype)) \
-                    if nxt is not None and getattr(nxt, "chains_norms", False) else None
+                    if nxt is not None and nxt.chains_norms else None
                 normed = block.forward(h, ctx, caches[i], normed=normed, then=then)
             else:
                 block.forward(h, ctx, caches[i])
                 normed = None
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
+        debug.region("final norm")
         x = self.final_norm.forward(h, ctx, rows=ctx.logit_rows)
+        debug.region("head")
         return self.head.forward(x)

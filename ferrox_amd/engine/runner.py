@@ -17,6 +17,7 @@ from dataclasses import dataclass, field
 
 import torch
 
+from .. import debug
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..csrc.build import ensure_built
@@ -53,6 +54,7 @@ class DecodeGraph:
         self.copied.record()
         self.graph = None
         self.logits = None
+        self.trace_calls = None        # where an active routing trace's copies went while this step was recorded
 
     def _context(self) -> StepContext:
         n, mb, m = self.n, self.max_blocks, self.meta
@@ -64,9 +66,7 @@ class DecodeGraph:
                           token_ids=m[0:n], positions=m[n:2 * n], token_seq=m[2 * n:3 * n],
                           q_starts=list(range(n + 1)), kv_lens=[self.kv_bound] * n, slot_ids=m[3 * n:4 * n],
                           slots=None, block_tables=tables, block_size=self.runner.block_size,
-                          logit_rows=m[4 * n:5 * n])
-        ctx._memo["attention_items"] = {"n_decode": n, "n_tiles": 0, "max_kv": self.kv_bound,
-                                        "dec_seq": m[2 * n:3 * n], "dec_tok": m[4 * n:5 * n]}
+                          logit_rows=m[4 * n:5 * n], recorded=True, kv_bound=self.kv_bound)
         return ctx
 
     def run(self, entries) -> torch.Tensor:
@@ -78,6 +78,8 @@ class DecodeGraph:
             self.runner.manager.pack_step([e.req for e in entries], [e.tokens for e in entries],
                                           [e.want for e in entries], self.runner.vocab_size, self._host_ptr,
                                           self._host_words, force_blocks=self.max_blocks)
+        if self.runner.before_launch is not None:
+            self.runner.before_launch()
         self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
         model, caches = self.runner.model, self.runner.storage.caches
@@ -90,6 +92,8 @@ class DecodeGraph:
             collecting = gc.isenabled()
             gc.collect()
             gc.disable()
+            if debug.routing_trace is not None:
+                debug.routing_trace.begin_step()     # the recorded launches write where the eager ones just wrote
             try:
                 with torch.cuda.graph(graph):
                     self.logits = model.forward(self._context(), caches)
@@ -97,7 +101,11 @@ class DecodeGraph:
                 if collecting:
                     gc.enable()
             self.graph = graph
+            if debug.routing_trace is not None:
+                self.trace_calls = debug.routing_trace.calls()
         self.graph.replay()
+        if debug.routing_trace is not None:
+            debug.routing_trace.replayed(self.trace_calls)
         return self.logits
 
 
@@ -116,10 +124,11 @@ class ModelRunner:
         self.storage = CacheStorage(model, self.manager, self.act_dtype, self.device)
         self.vocab_size = model.spec.vocab_size
         # decode steps are replayed from HIP graphs if every mixer can be recorded
-        self.use_graphs = use_graphs and all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
+        self.use_graphs = use_graphs and all(b.mixer.graph_safe for b in model.blocks)
         self.graph_kv_step = graph_kv_step
         self._graphs: dict = {}
         self._host = None                      # pinned staging buffer of the step's int32 data
+        self.before_launch = None              # measurement: called right before a step's first device operation
         self._uploaded = torch.cuda.Event()
 
     # ---- requests ----------------------------------------------------------
@@ -155,11 +164,13 @@ class ModelRunner:
         reqs = [e.req for e in entries]
         token_lists, wants = [e.tokens for e in entries], [e.want for e in entries]
         T, R = sum(len(t) for t in token_lists), sum(len(w) for w in wants)
+        if debug.routing_trace is not None:
+            debug.routing_trace.begin_step()
         if self.use_graphs and n_seqs and all(len(t) == 1 for t in token_lists) and all(len(w) == 1 for w in wants):
             # every sequence brings one token and wants its logits: a recorded decode step
             longest = max(mgr.length(r) for r in reqs)
             bound = -(-longest // self.graph_kv_step) * self.graph_kv_step
-            key = (n_seqs, bound)
+            key = (n_seqs, bound, debug.graph_token())
             if key not in self._graphs:
                 if len(self._graphs) >= 16:
                     self._graphs.pop(next(iter(self._graphs)))
@@ -183,6 +194,8 @@ class ModelRunner:
         host = self._staging(mgr.step_words(T, n_seqs, R, max_blocks))
         packed = mgr.pack_step(reqs, token_lists, wants, self.vocab_size, host.data_ptr(), host.numel())
         dev = torch.empty(packed.total, dtype=torch.int32, device=self.device)
+        if self.before_launch is not None:
+            self.before_launch()
         dev.copy_(host[:packed.total], non_blocking=True)
         self._uploaded.record()
         o = 0

@@ -11,10 +11,19 @@ from ..config.base import ConfigError, read_config_json
 
 @dataclass(frozen=True)
 class Architecture:
+    """One entry of the registry.
+
+    `name` is what config.json gives as `architectures[0]`, `model_type` its `model_type`.
+    `config_class` is the typed configuration: it must offer the class method
+    `from_dict(raw: dict, where: str = ...)`, which reads and validates the keys of config.json (raising
+    `ConfigError`), and `to_dict()`, which gives them back for a config.json to be written; it may offer
+    `defaulted_keys` (names of keys that were absent and got defaults), which the command line reports.
+    Nothing else of it is looked at outside `build_spec`.
+    `build_spec(config, tensor_names or None) -> ModelSpec` turns it into the model's description."""
     name: str
     model_type: str
     config_class: type
-    build_spec: Callable        # (config, tensor_names or None) -> ModelSpec
+    build_spec: Callable
 
 
 _BY_NAME: dict[str, Architecture] = {}
@@ -22,8 +31,19 @@ _BY_TYPE: dict[str, Architecture] = {}
 
 
 def register_architecture(arch: Architecture) -> None:
+    for method in ("from_dict", "to_dict"):
+        if not callable(getattr(arch.config_class, method, None)):
+            raise TypeError(f"architecture '{arch.name}': its configuration class has no {method}()")
     _BY_NAME[arch.name] = arch
     _BY_TYPE[arch.model_type] = arch
+
+
+def architecture_of(config) -> Architecture:
+    """The registered architecture whose configuration class `config` is an instance of."""
+    for arch in _BY_NAME.values():
+        if isinstance(config, arch.config_class):
+            return arch
+    raise ConfigError(f"no registered architecture has a configuration of type {type(config).__name__}")
 
 
 def known_architectures():

@@ -48,7 +48,7 @@ _sigs = {
     ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float],
     ("elementwise", "fx_rope_kv_write"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float],
+                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -59,7 +59,7 @@ _sigs = {
                           c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
     ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
                               c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                              c_int, c_int, c_int, c_int, c_int, c_float],
+                              c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float],
@@ -131,11 +131,21 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     return out
 
 
+def _freq_factors(freq_factors, rotary_dim):
+    if freq_factors is None:
+        return None
+    if freq_factors.dtype != torch.float32 or not freq_factors.is_contiguous() or freq_factors.numel() != rotary_dim // 2:
+        raise KernelError(f"rotary frequency factors must be {rotary_dim // 2} contiguous float32 values")
+    return freq_factors
+
+
 def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads,
-                  head_dim, block_size, rotary_dim, theta, interleaved=False) -> None:
+                  head_dim, block_size, rotary_dim, theta, interleaved=False, freq_factors=None) -> None:
     """Rotate q in place; rotate k and write it and v into the pages (skipped when k_pages is None).
-    q, k, v are 2-D views [T, heads*head_dim] with unit inner stride."""
+    q, k, v are 2-D views [T, heads*head_dim] with unit inner stride.  `freq_factors` (float32
+    [rotary_dim / 2] or None): the angle of pair i is divided by freq_factors[i]."""
     T = q.shape[0]
+    freq_factors = _freq_factors(freq_factors, rotary_dim)
     for t in (q, k, v):
         if t.stride(-1) != 1 or t.dtype != q.dtype:
             raise KernelError("rope_kv_write wants q, k, v of one dtype with unit inner stride")
@@ -150,7 +160,7 @@ def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, 
           _p(v), v.stride(0), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
           _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
           _p(k_pages), _p(v_pages), T, n_heads, n_kv_heads, head_dim, block_size, rotary_dim,
-          1 if interleaved else 0, float(theta))
+          1 if interleaved else 0, float(theta), _p(freq_factors))
 
 
 def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:
@@ -317,7 +327,7 @@ def can_qkv_rope(x, w, n_rows: int, head_dim: int, rotary_dim: int, interleaved:
 
 
 def qkv_rope(x, w, bias, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads, head_dim,
-             block_size, rotary_dim, theta) -> torch.Tensor:
+             block_size, rotary_dim, theta, freq_factors=None) -> torch.Tensor:
     """The q/k/v product of few tokens with the rotation and the cache write in its epilogue: returns
     [T, (n_heads + 2 n_kv_heads) head_dim] whose query columns are rotated (the others are not written); rotated
     keys and the values go into their pages (k_pages None: nowhere).  The bits are those of `gemm` followed by
@@ -342,7 +352,8 @@ def qkv_rope(x, w, bias, positions, token_seq, block_table, k_pages, v_pages, n_
           _p(later.ss) if later else None, later.ss.shape[1] if later else 0, float(later.eps) if later else 0.0,
           _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")), _p(_i32(block_table, "block_table")),
           block_table.shape[1] if block_table is not None else 0, _p(k_pages), _p(v_pages),
-          n_heads, n_kv_heads, head_dim, block_size, rotary_dim, float(theta))
+          n_heads, n_kv_heads, head_dim, block_size, rotary_dim, float(theta),
+          _p(_freq_factors(freq_factors, rotary_dim)))
     return out
 
 

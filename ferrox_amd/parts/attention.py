@@ -12,17 +12,21 @@ import math
 
 import torch
 
-from .. import ops
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec
+from .. import debug, limits, ops
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec, Rotary
 from .linear import Linear, same_dtype
 
 TILE_Q = 64   # queries per work item of the prefill kernels
+NO_ROTATION = Rotary(0, 1.0)
 
 
 def attention_items(ctx):
     """Work items of a step, shared by all attention layers: sequences with one
     new token go to the split decode kernel, the others are cut into blocks of
     TILE_Q consecutive queries."""
+    if ctx.recorded:      # token t is the one token of sequence t; nothing is made from host lists
+        return {"n_decode": ctx.n_seqs, "n_tiles": 0, "max_kv": ctx.kv_bound, "dec_seq": ctx.token_seq,
+                "dec_tok": ctx.token_seq}
     dec_seq, dec_tok, t_seq, t_tok, t_n = [], [], [], [], []
     max_kv = 1
     for s in range(ctx.n_seqs):
@@ -57,8 +61,9 @@ class PagedAttention(Mixer):
                  position: PartSpec, window: int | None = None, scale: float | None = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head_dim {head_dim}: the attention kernels take multiples of 16 from 16 to 256")
+        if head_dim % limits.HEAD_DIM_STEP or not limits.HEAD_DIM_STEP <= head_dim <= limits.HEAD_DIM_MAX:
+            raise ValueError(f"head_dim {head_dim}: the attention kernels take multiples of {limits.HEAD_DIM_STEP} "
+                             f"up to {limits.HEAD_DIM_MAX}")
         self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
         self.bias = bool(bias)
         self.window = int(window) if window else None
@@ -95,10 +100,12 @@ class PagedAttention(Mixer):
     def forward_from_residual(self, norm, ctx, cache, residual) -> bool:
         """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
         more, every block's reading and norming of all rows costs more than the norm kernel)."""
-        if (ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm" or residual.shape[0] > 16
+        rms = norm.rms_params()
+        if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16
                 or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
-        qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=(norm.weight, norm.eps))
+        debug.region("qkv")
+        qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=rms)
         self.forward(None, ctx, cache, residual, qkv=qkv)
         return True
 
@@ -111,12 +118,14 @@ class PagedAttention(Mixer):
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
+        debug.region("qkv")
         if (qkv is None and rot is not None
-                and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot[0], rot[2])):
+                and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved)):
             # few tokens: rotation and cache write happen in the product's epilogue
             qkv = ops.qkv_rope(x, self.qkv.weight, self.qkv.bias, ctx.positions, ctx.token_seq, table,
                                k_pages if cache.writes else None, v_pages if cache.writes else None,
-                               self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1])
+                               self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot.rotary_dim, rot.theta,
+                               rot.freq_factors)
             q = qkv[:, :self.qw]
         else:
             if qkv is None:
@@ -125,12 +134,15 @@ class PagedAttention(Mixer):
                 else:
                     qkv = self.qkv(x)
             q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
+            debug.region("rope + cache write")
             if rot is None:
                 self.position.apply(q, k, ctx)
-                rot = (0, 1.0, False)
+                rot = NO_ROTATION
             ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
                               k_pages if cache.writes else None, v_pages if cache.writes else None,
-                              self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot[0], rot[1], rot[2])
+                              self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot.rotary_dim, rot.theta,
+                              rot.interleaved, rot.freq_factors)
+        debug.region("attention")
         out = torch.empty((ctx.n_tokens, self.qw), dtype=qkv.dtype, device=qkv.device)
         items = ctx.memo("attention_items", lambda: attention_items(ctx))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
@@ -140,4 +152,5 @@ class PagedAttention(Mixer):
         if items["n_decode"]:
             ops.attention_decode(q, out, k_pages, v_pages, table, ctx.positions,
                                  items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"])
+        debug.region("o_proj")
         self.o_proj(out, epilogue=ops.EPI_RESID, out=residual)

@@ -11,11 +11,12 @@ Interfaces (all tensors on the GPU; `h` is the float32 residual stream [T, H],
 `x` an activation [T, H] in `ctx.act_dtype`):
 
   Norm             forward(h, ctx, rows=None) -> x
-  PositionEncoding rotary() -> (rotary_dim, theta, interleaved) when the attention
-                   kernels can apply it themselves, else None and
+  PositionEncoding rotary() -> a `Rotary` (dimension, theta, pairing, optional table of
+                   per-pair frequency factors) when the attention kernels can apply it
+                   themselves, else None and
                    apply(q, k, ctx) -> None rotates q [T, nh*hd], k [T, nkv*hd] in place
   Mixer            window (None or int), page_shapes(block_size) -> {name: shape},
-                   state_shapes() -> {name: (shape, dtype)},
+                   cache_group() -> (key, window), state_shapes() -> {name: (shape, dtype)}, graph_safe,
                    forward(x, ctx, cache, residual) -> None   (adds its output into residual)
   FeedForward      forward(x, ctx, residual) -> None
   Block            forward(h, ctx, cache) -> None
@@ -141,6 +142,13 @@ class StepContext:
     block_tables: dict                 # group key -> int32 [n_seqs, max_blocks]
     block_size: int
     logit_rows: torch.Tensor | None = None   # int32 [R] token indices whose logits are wanted
+    # True while a decode step is recorded for replay (a HIP graph): every sequence brings exactly one
+    # token, token t belongs to sequence t, and what changes from replay to replay is only the content
+    # of the device tensors above.  The host lists then give the shape alone (kv_lens holds `kv_bound`,
+    # which every replay's sequence lengths stay under; `slots` is None): a part must not make device
+    # data from them or choose launches by their values.
+    recorded: bool = False
+    kv_bound: int = 0
     carry: object = None               # what a feed-forward hands on to the next block (its rows, normed), see PreNormBlock
     _memo: dict = field(default_factory=dict)
 
@@ -201,9 +209,28 @@ class Norm(Part):
     def forward(self, h, ctx: StepContext, rows=None):
         raise NotImplementedError
 
+    def rms_params(self):
+        """(weight, eps) if this norm is y = x * rsqrt(mean(x^2) + eps) * weight, which kernels of other parts
+        can apply on their way in or leave to the product that follows; None for any other norm (the parts
+        then call `forward`)."""
+        return None
+
+
+@dataclass(frozen=True)
+class Rotary:
+    """A rotation that the kernels apply themselves while they write the cache: pair i of the first
+    `rotary_dim` dimensions of every q and k head turns by pos * theta^(-2i/rotary_dim), divided by
+    freq_factors[i] if a table is given (float32 [rotary_dim / 2] on the device).  Pairs are
+    (i, i + rotary_dim/2), or (2i, 2i+1) when `interleaved`.  rotary_dim 0 rotates nothing."""
+    rotary_dim: int
+    theta: float
+    interleaved: bool = False
+    freq_factors: torch.Tensor | None = None
+
 
 class PositionEncoding(Part):
-    def rotary(self):
+    def rotary(self) -> "Rotary | None":
+        """A `Rotary` if the encoding is one the kernels apply; None if `apply` has to be called."""
         return None
 
     def apply(self, q, k, ctx: StepContext) -> None:
@@ -212,9 +239,18 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     window: int | None = None
+    graph_safe = False        # True: forward launches the same kernels for every step of one shape (see StepContext.recorded)
 
     def page_shapes(self, block_size: int) -> dict:
         return {}
+
+    def cache_group(self):
+        """(key, window) of the pages this mixer keeps.  Mixers that name the same key share page ids and
+        block tables (each has slabs of its own behind them); `window` says how the group's pages age:
+        None keeps every position, W gives a page back once all its positions are W or more behind every
+        later query.  The key is any hashable value; a mixer whose pages age in a way of its own names a
+        key of its own."""
+        return (("window", int(self.window)), int(self.window)) if self.window else (("full",), None)
 
     def state_shapes(self) -> dict:
         return {}
@@ -222,19 +258,40 @@ class Mixer(Part):
     def forward(self, x, ctx: StepContext, cache: LayerCache, residual) -> None:
         raise NotImplementedError
 
+    # ---- optional: norms fused into the mixer's first kernel (a block asks; the defaults decline) ----
+    def forward_from_residual(self, norm: "Norm", ctx: StepContext, cache: LayerCache, residual) -> bool:
+        """Apply `norm` to the residual stream inside the mixer's first kernel and run the mixer; False
+        (nothing done) if this step or this norm does not allow it, and the block then calls the norm itself."""
+        return False
+
+    def takes_scale_later(self, act_dtype) -> bool:
+        """Whether `forward` accepts an `ops.ScaleLater` (rows times the norm's weight, the scale still to come) as x."""
+        return False
+
 
 class FeedForward(Part):
+    norms_after = False      # True: forward takes then_norm=(norm, scale_later_ok) and may leave norm(residual) in ctx.carry
+
     def forward(self, x, ctx: StepContext, residual) -> None:
         raise NotImplementedError
+
+    def forward_from_residual(self, norm: "Norm", ctx: StepContext, residual, **more) -> bool:
+        """As `Mixer.forward_from_residual`."""
+        return False
 
 
 class Block(Part):
     """A block that sets `chains_norms = True` also has a `first_norm` and takes
     forward(h, ctx, cache, normed=None, then=None): `normed` is first_norm(h) if the block before has made it,
     `then` is (the first norm of the block after, that block's takes_scale_later(dtype)); it returns the
-    rows normed by that norm if one of its kernels has made them, else None."""
+    rows normed by that norm if one of its kernels has made them, else None.  The model passes `normed` and
+    `then` only between neighbours that both chain; every other block is called as forward(h, ctx, cache)."""
     mixer: Mixer
     chains_norms = False
+    first_norm: "Norm | None" = None
+
+    def takes_scale_later(self, act_dtype) -> bool:
+        return False
 
     def forward(self, h, ctx: StepContext, cache: LayerCache) -> None:
         raise NotImplementedError

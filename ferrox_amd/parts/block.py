@@ -1,6 +1,7 @@
 """Arrangements of a mixer, a feed-forward and norms in one layer."""
 from __future__ import annotations
 
+from .. import debug
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block
 
 
@@ -23,8 +24,7 @@ class PreNormBlock(Block):
         return self.norm1
 
     def takes_scale_later(self, act_dtype) -> bool:
-        f = getattr(self.mixer, "takes_scale_later", None)
-        return bool(f and f(act_dtype))
+        return bool(self.mixer.takes_scale_later(act_dtype))
 
     def forward(self, h, ctx, cache, normed=None, then=None):
         """`normed`: norm1(h), if the block before has already made it (a tensor, or an ops.ScaleLater if this
@@ -35,14 +35,13 @@ class PreNormBlock(Block):
         # into its first kernel, and says False when it cannot for this step
         if normed is not None:
             self.mixer.forward(normed, ctx, cache, h)
-        else:
-            fused = getattr(self.mixer, "forward_from_residual", None)
-            if fused is None or not fused(self.norm1, ctx, cache, h):
-                self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
+        elif not self.mixer.forward_from_residual(self.norm1, ctx, cache, h):
+            debug.region("norm")
+            self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
         ctx.carry = None
-        more = {"then_norm": then} if then is not None and getattr(self.ffn, "norms_after", False) else {}
-        fused = getattr(self.ffn, "forward_from_residual", None)
-        if fused is None or not fused(self.norm2, ctx, h, **more):
+        more = {"then_norm": then} if then is not None and self.ffn.norms_after else {}
+        if not self.ffn.forward_from_residual(self.norm2, ctx, h, **more):
+            debug.region("norm")
             self.ffn.forward(self.norm2.forward(h, ctx), ctx, h, **more)
         out, ctx.carry = ctx.carry, None
         return out

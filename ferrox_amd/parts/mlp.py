@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .. import ops
+from .. import debug, ops
 from .base import FEED_FORWARDS, FeedForward, ParamSpec
 from .linear import Linear, same_dtype
 
@@ -31,5 +31,7 @@ class SwiGLU(FeedForward):
         return self.down(self.gate_up(x, epilogue=ops.EPI_SILU_MUL), epilogue=ops.EPI_STORE_F32)
 
     def forward(self, x, ctx, residual, row_scale=None) -> None:
+        debug.region("mlp gate/up")
         act = self.gate_up(x, epilogue=ops.EPI_SILU_MUL)
+        debug.region("mlp down")
         self.down(act, epilogue=ops.EPI_RESID, out=residual, row_scale=row_scale)

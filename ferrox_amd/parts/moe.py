@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from .. import ops
+from .. import debug, limits, ops
 from .base import FEED_FORWARDS, FeedForward, ParamSpec
 from .linear import matmul, same_dtype
 from .mlp import SwiGLU
@@ -32,7 +32,6 @@ def side_stream(device) -> torch.cuda.Stream:
 @FEED_FORWARDS.register("sparse_moe")
 class SparseMoE(FeedForward):
     kernel_libraries = ("elementwise", "gemm", "moe")
-    record = None      # a list here collects every call's expert ids (measurement only)
     norms_after = True   # forward(..., then_norm=norm) may leave norm(residual) in ctx.carry for the next layer
 
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
@@ -40,6 +39,9 @@ class SparseMoE(FeedForward):
                  shared_gate: bool = True):
         if not 1 <= top_k <= n_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{n_experts}")
+        if n_experts > limits.MOE_MAX_EXPERTS or top_k > limits.MOE_MAX_TOP_K:
+            raise ValueError(f"{n_experts} experts / top_k {top_k}: the routing kernels take up to "
+                             f"{limits.MOE_MAX_EXPERTS} experts and {limits.MOE_MAX_TOP_K} per token")
         if gating not in GATINGS:
             raise ValueError(f"gating '{gating}' is not one of {sorted(GATINGS)}")
         self.hidden_size, self.n_experts, self.top_k = int(hidden_size), int(n_experts), int(top_k)
@@ -103,20 +105,22 @@ class SparseMoE(FeedForward):
         block takes an ops.ScaleLater).  For up to 64 rows (what the product for few rows takes) the combine also
         writes them times the norm's weight, with sums of squares, and the product that follows applies the
         scale: the norm costs no launch.  (For many rows a norm kernel of its own is as fast.)"""
-        if then_norm is None or getattr(then_norm[0], "kind", None) != "rmsnorm":
+        if then_norm is None or then_norm[0].rms_params() is None:
             return {}
         norm, later_ok = then_norm
         if n_tokens <= 64 and later_ok and ctx.act_dtype == torch.bfloat16:
-            return dict(scale_later=(norm.weight, norm.eps, ctx.act_dtype))
+            return dict(scale_later=(*norm.rms_params(), ctx.act_dtype))
         return {}
 
     def forward_from_residual(self, norm, ctx, residual, then_norm=None) -> bool:
         """Few tokens: the norm and the router are one launch, and the expert products group the
         (token, slot) pairs themselves instead of reading a sorted layout."""
         T = residual.shape[0]
-        if T > 64 or ctx.act_dtype != torch.bfloat16 or getattr(norm, "kind", None) != "rmsnorm":
+        rms = norm.rms_params()
+        if T > 64 or ctx.act_dtype != torch.bfloat16 or rms is None:
             return False
-        front = ops.moe_front(residual, norm.weight, norm.eps, self.router, self.n_experts, self.top_k,
+        debug.region("router")
+        front = ops.moe_front(residual, rms[0], rms[1], self.router, self.n_experts, self.top_k,
                               self.norm_topk_prob, self.gating, self.has_shared_gate)
         if front is None:
             return False
@@ -135,13 +139,16 @@ class SparseMoE(FeedForward):
         if routed is not None and routed[3] is None and self.shared_pieces and x.dtype == self.w_gate_up_all.dtype:
             # few tokens, unsorted pairs, shared expert as pieces: two launches do all experts
             ids, weights, gate = routed[:3]
-            if SparseMoE.record is not None:
-                SparseMoE.record.append(ids)
+            if debug.routing_trace is not None:
+                debug.routing_trace.put(ids)
             S, n = self.shared_pieces, ids.numel()
+            debug.region("experts gate/up")
             act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k,
                            always=(S, T, True), w_kblocked=self.kblocked)
+            debug.region("experts down")
             y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False),
                          w_kblocked=self.kblocked)
+            debug.region("combine")
             ctx.carry = ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate, **then)
             return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
@@ -154,9 +161,11 @@ class SparseMoE(FeedForward):
             fork.record(main)
             side.wait_event(fork)
             with torch.cuda.stream(side):
+                debug.region("shared expert")
                 shared_out = self.shared.output(x)
                 join.record(side)
         if routed is None:
+            debug.region("router")
             if T > 64 and self.router.shape[0] <= 64 and self.router.dtype == x.dtype:
                 # few experts, many tokens: the router's rows are the short side of the product, so the
                 # kernel for few rows streams the activations once; the logits come out transposed
@@ -166,17 +175,21 @@ class SparseMoE(FeedForward):
             routed = ops.route(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
                                self.has_shared_gate)
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
-        if SparseMoE.record is not None:
-            SparseMoE.record.append(ids)
+        if debug.routing_trace is not None:
+            debug.routing_trace.put(ids)
         kb = dict(w_kblocked=True) if self.kblocked else {}
+        debug.region("experts gate/up")
         if offsets is None:      # few pairs, unsorted: row p of `act` and of `y` is pair p
             act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k, **kb)
+            debug.region("experts down")
             y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids, **kb)
         else:
             act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
                          expert_offsets=offsets, n_rows=T * self.top_k, **kb)
+            debug.region("experts down")
             # each expert's rows go back to the place of their (token, slot) pair
             y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
+        debug.region("combine")
         if overlap:
             main.wait_event(join)
             shared_out.record_stream(main)

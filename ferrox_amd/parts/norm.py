@@ -9,7 +9,6 @@ from .base import NORMS, Norm, ParamSpec
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     kernel_libraries = ("elementwise",)
-    kind = "rmsnorm"       # parts that fuse this norm into their first kernel ask for it by this name
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)
@@ -21,6 +20,9 @@ class RMSNorm(Norm):
 
     def load(self, fetch):
         self.weight = fetch("weight").contiguous()
+
+    def rms_params(self):
+        return self.weight, self.eps
 
     def forward(self, h, ctx, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, ctx.act_dtype, rows=rows)

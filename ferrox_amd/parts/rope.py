@@ -8,7 +8,7 @@ which the reference's registry gives this architecture
 """
 from __future__ import annotations
 
-from .base import POSITION_ENCODINGS, PositionEncoding
+from .base import POSITION_ENCODINGS, PositionEncoding, Rotary
 
 
 class _Rotary(PositionEncoding):
@@ -24,7 +24,7 @@ class _Rotary(PositionEncoding):
             raise ValueError(f"rope theta must be positive, got {self.theta}")
 
     def rotary(self):
-        return self.rotary_dim, self.theta, self.interleaved
+        return Rotary(self.rotary_dim, self.theta, self.interleaved)
 
 
 @POSITION_ENCODINGS.register("rope_neox")
@@ -43,4 +43,4 @@ class NoPositions(PositionEncoding):
         self.head_dim = head_dim
 
     def rotary(self):
-        return 0, 1.0, False
+        return Rotary(0, 1.0)

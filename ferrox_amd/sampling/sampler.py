@@ -59,14 +59,21 @@ class XorShift64:
         return (self.next_u64() >> 40) / float(1 << 24)
 
 
-def sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list) -> list:
+def sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list, launched=None) -> list:
     """One token id per row of `logits` [R, V] (float32, on the GPU).  `params[r]`,
     `rngs[r]`, `histories[r]` (the tokens generated so far) belong to row r.  A generator is
-    advanced only for rows that draw."""
+    advanced only for rows that draw.  `launched()` is called after the kernel is launched and
+    before the host waits for the ids (for measurement)."""
     R = logits.shape[0]
     dev = logits.device
+
+    def ids_of(out):
+        if launched is not None:
+            launched()
+        return out.tolist()
+
     if all(p.greedy and not p.uses_history for p in params):
-        return ops.sample(logits).tolist()
+        return ids_of(ops.sample(logits))
 
     def f32(vals):
         return torch.tensor(vals, dtype=torch.float32, device=dev)
@@ -88,4 +95,4 @@ def sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list)
         kw["rep_penalty"] = f32([p.repetition_penalty for p in params])
         kw["presence"] = f32([p.presence_penalty for p in params])
         kw["frequency"] = f32([p.frequency_penalty for p in params])
-    return ops.sample(logits, **kw).tolist()
+    return ids_of(ops.sample(logits, **kw))

@@ -10,6 +10,14 @@ the layer plan and the window) are marked "convention".
 
 Arithmetic is done in `dtype` (float64 by default, so that the oracle's own
 rounding is far below what the tests look for).
+
+`stored`, where a function takes it, is a rounding applied to exactly those
+tensors that an engine with activations of reduced precision has to store:
+normed rows, q/k/v after the bias, q and k after the rotation, the softmax's
+unnormalised probabilities, the attention output, silu(gate) * up.  With
+`stored=to_bfloat16` the model shows how far rounding at those places alone
+moves the logits, which is what the bfloat16 tests measure the engine against;
+None (the default) rounds nothing.
 """
 from __future__ import annotations
 
@@ -18,6 +26,11 @@ import math
 import os
 
 import torch
+
+
+def to_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """round to bfloat16 (nearest even) and back"""
+    return x.to(torch.bfloat16).to(x.dtype)
 
 
 # --------------------------------------------------------------------------
@@ -61,7 +74,7 @@ def rope_neox_rows(x: torch.Tensor, positions, theta: float) -> torch.Tensor:
 
 
 def causal_attention(q, k, v, n_heads: int, n_kv_heads: int, window: int | None,
-                     scale: float | None = None) -> torch.Tensor:
+                     scale: float | None = None, stored=None) -> torch.Tensor:
     """Causal grouped-query attention over one whole sequence.
 
     q[T, n_heads, hd], k/v[T, n_kv_heads, hd]; row t is the query at position t
@@ -85,8 +98,11 @@ def causal_attention(q, k, v, n_heads: int, n_kv_heads: int, window: int | None,
             vals = v[start:t + 1, kv_h]
             s = (keys @ q[t, h]) * scale
             p = torch.exp(s - s.max())
-            p = p / p.sum()
-            out[t, h] = p @ vals
+            if stored is None:
+                p = p / p.sum()
+                out[t, h] = p @ vals
+            else:                 # the probabilities are rounded for the product, their sum is not
+                out[t, h] = (stored(p) @ vals) / p.sum()
     return out
 
 
@@ -113,10 +129,13 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu_mlp(x, w_gate, w_up, w_down) -> torch.Tensor:
+def swiglu_mlp(x, w_gate, w_up, w_down, stored=None) -> torch.Tensor:
     """down( silu(gate x) * (up x) )   (ferrox-moe/src/lib.rs:655-658,
     ferrox-core/src/matmul.rs:274-280).  Weights are [out, in]."""
-    return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+    act = silu(x @ w_gate.T) * (x @ w_up.T)
+    if stored is not None:
+        act = stored(act)
+    return act @ w_down.T
 
 
 def router_margin(logits: torch.Tensor, k: int) -> float:
@@ -140,7 +159,7 @@ def combine_expert_outputs(routed, shared, hidden_dim: int, dtype=torch.float64)
 
 
 def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w, margins=None, forced_ids=None,
-                  chosen=None):
+                  chosen=None, probs_out=None, stored=None):
     """One token through the sparse block.
 
     Router logits r = router . x with no bias (ferrox-models/src/decoder.rs:2915),
@@ -149,9 +168,12 @@ def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w
     (ferrox-models/src/decoder.rs:2660-2679).
     `experts` is a list of (gate, up, down); `shared` one such triple or None.
     `forced_ids` replaces the router's choice of experts (their weights are still the router's
-    probabilities); `chosen`, a list, receives the ids used.
+    probabilities); `chosen`, a list, receives the ids used; `probs_out`, a list, the router's
+    probabilities of all experts.
     """
     logits = router_w @ x
+    if probs_out is not None:
+        probs_out.append(torch.softmax(logits, 0).tolist())
     ids, w = route_top_k(logits, k, norm_topk_prob)
     if forced_ids is not None and list(forced_ids) != ids:
         ids = [int(e) for e in forced_ids]
@@ -163,10 +185,10 @@ def moe_ffn_token(x, router_w, experts, k, norm_topk_prob, shared, shared_gate_w
         chosen.append(list(ids))
     if margins is not None:
         margins.append(router_margin(logits, k))
-    routed = [(swiglu_mlp(x, *experts[e]), w[j]) for j, e in enumerate(ids)]
+    routed = [(swiglu_mlp(x, *experts[e], stored=stored), w[j]) for j, e in enumerate(ids)]
     shared_out = []
     if shared is not None:
-        y = swiglu_mlp(x, *shared)
+        y = swiglu_mlp(x, *shared, stored=stored)
         if shared_gate_w is not None:
             z = (shared_gate_w.reshape(-1) * x).sum()
             y = y * (1.0 / (1.0 + torch.exp(-z)))
@@ -211,21 +233,26 @@ def load_folder(folder: str, dtype=torch.float64):
 
 
 def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0, margins=None, routing=None,
-            chosen=None) -> torch.Tensor:
+            chosen=None, router_probs=None, stored=None) -> torch.Tensor:
     """Logits[T, V] of one whole sequence (ferrox-models/src/decoder.rs:3014-3678
     followed by the head on every row, decoder.rs:2952-2973).
 
     `start_pos` shifts every position (used by the shift-invariance test only).
     `margins`, a list of T floats if given, receives for every position the smallest
     `router_margin` over the sparse layers.  `routing[t][j]` forces the experts of position t in the
-    j-th sparse layer; `chosen`, a list, receives the experts used in the same shape.
+    j-th sparse layer; `chosen`, a list, receives the experts used in the same shape, and
+    `router_probs`, a list, the router's probabilities of all experts as [position][sparse layer][expert].
+    `stored`: see the head of this file.
     """
+    keep = stored if stored is not None else (lambda t: t)
     T = len(tokens)
     n_sparse = 0
     if chosen is not None:
         chosen[:] = [[] for _ in range(T)]
     if margins is not None:
         margins[:] = [1.0] * T
+    if router_probs is not None:
+        router_probs[:] = [[] for _ in range(T)]
     nh = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads", nh)
     hd = head_dim_of(cfg)
@@ -236,7 +263,7 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
     h = w["model.embed_tokens.weight"][torch.tensor(tokens, dtype=torch.long)].to(dtype)  # no scale: decoder.rs:1279-1284
     for l in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{l}."
-        x = rms_norm(h, w[p + "input_layernorm.weight"], eps)                       # decoder.rs:3225-3228
+        x = keep(rms_norm(h, w[p + "input_layernorm.weight"], eps))                 # decoder.rs:3225-3228
         q = x @ w[p + "self_attn.q_proj.weight"].T
         k = x @ w[p + "self_attn.k_proj.weight"].T
         v = x @ w[p + "self_attn.v_proj.weight"].T
@@ -244,12 +271,13 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
             q = q + w[p + "self_attn.q_proj.bias"]                                   # before rotation:
             k = k + w[p + "self_attn.k_proj.bias"]                                   # decoder.rs:3234-3254
             v = v + w[p + "self_attn.v_proj.bias"]
-        q = rope_neox_rows(q.reshape(T, nh, hd), positions, theta)
-        k = rope_neox_rows(k.reshape(T, nkv, hd), positions, theta)
+        q, k, v = keep(q), keep(k), keep(v)
+        q = keep(rope_neox_rows(q.reshape(T, nh, hd), positions, theta))
+        k = keep(rope_neox_rows(k.reshape(T, nkv, hd), positions, theta))
         v = v.reshape(T, nkv, hd)                                                    # v is not rotated
-        a = causal_attention(q, k, v, nh, nkv, layer_window(cfg, l))
+        a = keep(causal_attention(q, k, v, nh, nkv, layer_window(cfg, l), stored=stored))
         h = h + a.reshape(T, nh * hd) @ w[p + "self_attn.o_proj.weight"].T          # no bias: decoder.rs:3549-3560
-        x2 = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)             # decoder.rs:3563-3566
+        x2 = keep(rms_norm(h, w[p + "post_attention_layernorm.weight"], eps))       # decoder.rs:3563-3566
         if layer_is_sparse(cfg, l):
             E = cfg["num_experts"]
             experts = [(w[p + f"mlp.experts.{e}.gate_proj.weight"],
@@ -264,24 +292,29 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
                 gate_w = w[p + "mlp.shared_expert_gate.weight"]
             layer_margins = [] if margins is not None else None
             layer_chosen = []
+            layer_probs = [] if router_probs is not None else None
             f = torch.stack([
                 moe_ffn_token(x2[t], w[p + "mlp.gate.weight"], experts,
                               cfg["num_experts_per_tok"], cfg.get("norm_topk_prob", False),
                               shared, gate_w, layer_margins,
-                              routing[t][n_sparse] if routing is not None else None, layer_chosen)
+                              routing[t][n_sparse] if routing is not None else None, layer_chosen, layer_probs,
+                              stored)
                 for t in range(T)])
             if chosen is not None:
                 for t in range(T):
                     chosen[t].append(layer_chosen[t])
+            if router_probs is not None:
+                for t in range(T):
+                    router_probs[t].append(layer_probs[t])
             n_sparse += 1
             if margins is not None:
                 for t in range(T):
                     margins[t] = min(margins[t], layer_margins[t])
         else:                                                                        # dense layer: decoder.rs:2902-2913
             f = swiglu_mlp(x2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                           w[p + "mlp.down_proj.weight"])
+                           w[p + "mlp.down_proj.weight"], stored)
         h = h + f
-    x = rms_norm(h, w["model.norm.weight"], eps)                                     # decoder.rs:3674-3677
+    x = keep(rms_norm(h, w["model.norm.weight"], eps))                               # decoder.rs:3674-3677
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) \
         else w["lm_head.weight"]                                                     # loader.rs:1433-1436
     return x @ head.T

@@ -99,46 +99,42 @@ def max_live_tokens(steps: list, round_to: int = 64) -> int:
 # ---- running a trace through the engine ---------------------------------------
 def run_trace(runner, steps: list, routing: dict | None = None) -> dict:
     """(request id, position) -> float32 logits row (CPU).  If `routing` is a dict it receives
-    (request id, position) -> experts chosen in each sparse layer (the step then runs eagerly)."""
+    (request id, position) -> experts chosen in each sparse layer, read from the engine's routing
+    trace (recorded decode steps are replayed as always: the trace's copies are part of them)."""
+    import contextlib
+    from ferrox_amd import debug
     from ferrox_amd.engine.runner import StepEntry
-    from ferrox_amd.parts.moe import SparseMoE
     out, pos = {}, {}
-    graphs = runner.use_graphs
-    if routing is not None:
-        runner.use_graphs = False
-    for st in steps:
-        entries = []
-        for e in st["entries"]:
-            rid = e["id"]
-            if rid not in runner.manager:
-                assert runner.admit(rid), f"no slot for {rid}"
-                pos[rid] = 0
-            assert runner.reserve(rid, len(e["tokens"])), f"out of pages for {rid}"
-            entries.append(StepEntry(rid, e["tokens"], e["want"]))
-        if routing is not None:
-            SparseMoE.record = []
-        logits = runner.step(entries)
-        if routing is not None:
-            per_layer = [t.cpu().tolist() for t in SparseMoE.record]      # [sparse layer][token][slot]
-            SparseMoE.record = None
-            tok = 0
+    with (debug.trace_routing() if routing is not None else contextlib.nullcontext()) as trace:
+        for st in steps:
+            entries = []
             for e in st["entries"]:
-                for i in range(len(e["tokens"])):
-                    routing[(e["id"], pos[e["id"]] + i)] = [layer[tok] for layer in per_layer]
-                    tok += 1
-        runner.manager.check_invariants()
-        row = 0
-        if logits is not None:
-            logits = logits.float().cpu()
-        for e in st["entries"]:
-            for w in e["want"]:
-                out[(e["id"], pos[e["id"]] + w)] = logits[row]
-                row += 1
-            pos[e["id"]] += len(e["tokens"])
-        for rid in st["end"]:
-            runner.release(rid)
-            pos.pop(rid, None)
-    runner.use_graphs = graphs
+                rid = e["id"]
+                if rid not in runner.manager:
+                    assert runner.admit(rid), f"no slot for {rid}"
+                    pos[rid] = 0
+                assert runner.reserve(rid, len(e["tokens"])), f"out of pages for {rid}"
+                entries.append(StepEntry(rid, e["tokens"], e["want"]))
+            logits = runner.step(entries)
+            if routing is not None:
+                per_layer = trace.read()                                  # [sparse layer][token][slot]
+                tok = 0
+                for e in st["entries"]:
+                    for i in range(len(e["tokens"])):
+                        routing[(e["id"], pos[e["id"]] + i)] = [layer[tok] for layer in per_layer]
+                        tok += 1
+            runner.manager.check_invariants()
+            row = 0
+            if logits is not None:
+                logits = logits.float().cpu()
+            for e in st["entries"]:
+                for w in e["want"]:
+                    out[(e["id"], pos[e["id"]] + w)] = logits[row]
+                    row += 1
+                pos[e["id"]] += len(e["tokens"])
+            for rid in st["end"]:
+                runner.release(rid)
+                pos.pop(rid, None)
     return out
 
 
@@ -160,49 +156,132 @@ def plain_logits(folder: str, tokens, with_margins: bool = False):
     return _plain_cache[key] if with_margins else _plain_cache[key][0]
 
 
+_stored_cache: dict = {}
+
+
+def stored_logits(folder: str, tokens, routing):
+    """logits [T, V] of the plain model that rounds to bfloat16 where activations are stored, with the
+    experts of `routing`"""
+    key = (folder, tuple(tokens), repr(routing))
+    if key not in _stored_cache:
+        cfg, w = _plain_model(folder)
+        _stored_cache[key] = plain.forward(cfg, w, list(tokens), routing=routing, stored=plain.to_bfloat16)
+    return _stored_cache[key]
+
+
 def same_choice(a, b) -> bool:
     """the same experts in every sparse layer; their order only decides the order of a sum"""
     return len(a) == len(b) and all(sorted(x) == sorted(y) for x, y in zip(a, b))
 
 
+def near_tie_choice(chosen, probs, margin: float) -> bool:
+    """Whether `chosen` is a top-k of `probs` up to a relative perturbation of `margin`: no expert that
+    was left out has a probability more than `margin` above the smallest one that was taken."""
+    taken = set(chosen)
+    if len(taken) != len(chosen) or not all(0 <= e < len(probs) for e in taken):
+        return False
+    low = min(probs[e] for e in taken)
+    left_out = [p for e, p in enumerate(probs) if e not in taken]
+    return not left_out or low >= (1.0 - margin) * max(left_out)
+
+
+# How the bfloat16 engine is measured.  `plain.forward(..., stored=plain.to_bfloat16)` is the plain model with
+# rounding at exactly the places where an engine with bfloat16 activations stores a tensor (float64 otherwise).
+# Its deviation from the plain model says what those roundings alone do to this model's logits on these tokens:
+# noise on every logit, r = pooled rms((model - plain) / sigma_row) and r_row the same for one row (rows that see
+# few keys are noisier than the pool), and now and then much more on one logit that the model is sensitive at
+# (under a tied head the current token's own logit, ten spreads out, moves by 6 % of a spread where an attention
+# of one narrow head leaves few terms to average over).  An engine that rounds at the same places makes the same
+# roundings wherever its sums agree with the model's to within half a unit in the last place, so most of that
+# deviation it shares with the model, outliers included, and what is left is noise of at most the same scale.
+# The engine is therefore held against the rounding model: every logit within NOISE_SIGMAS * max(r, r_row) *
+# sigma_row of the model's (the largest of a million draws of a Gaussian lies below 5.3 standard deviations; 7
+# leaves a margin of a quarter), and the pooled rms of (engine - model) / sigma_row within RMS_FACTOR * r (two
+# independent sets of roundings would give 1.41 r).  The rounding model itself is pinned to the plain model by
+# construction: it is the same code with `stored` applied at the named tensors.
+# Outlier logits (more than OUTLIER spreads from zero) are coherent sums, to which a relative shift of the
+# sublayers' output against the embedding passes undiminished; there the model's and the engine's roundings need
+# not agree (seen: model +0.34 %, engine +0.07 % of a logit 17 spreads out).  For them the bound grows by
+# OUTLIER_FACTOR * rel * |logit|, rel being the largest relative deviation from the plain model that the rounding
+# model shows on any outlier of the comparison (0.3-0.7 % where there are outliers at all).
+RMS_FACTOR, NOISE_SIGMAS, OUTLIER, OUTLIER_FACTOR = 1.5, 7.0, 5.0, 1.5
+
+
 def compare(got: dict, folder: str, requests: dict, atol: float, rtol: float, what: str,
-            routing: dict | None = None, flip_margin: float = 0.05, stol: float = 0.0) -> float:
+            routing: dict | None = None, flip_margin: float = 0.05, storage: str | None = None) -> float:
     """Every (request, position) of `got` against the plain implementation; returns the largest error.
 
     `routing` (bfloat16 only): the experts the engine chose.  Rounding may flip a choice where two
-    router probabilities nearly tie.  Where the engine's choice differs from the plain model's, the
-    tie must be a near one (relative gap below `flip_margin`), and the plain model is then run with
-    the engine's choice, so that everything else is still compared at every position.
-    The bound on an element is atol + rtol * |plain| + stol * (standard deviation of the plain
-    logits of that position)."""
+    router probabilities nearly tie.  Where the engine's choices differ from the plain model's, the
+    plain model is run again with the engine's choices (so that everything else is still compared at
+    every position, and later layers see what the engine saw), and every choice of that sequence, in
+    every sparse layer, must be a top-k of the plain router's probabilities up to a relative
+    perturbation of `flip_margin`: an expert is only ever exchanged for one whose probability is
+    within that margin.
+    Without `storage` the bound on an element is atol + rtol * |plain|.  With storage="bfloat16" the bounds
+    are what the rounding model above gives for this model and these tokens (atol and rtol are not used)."""
     worst, worst_at, flips, total = 0.0, None, 0, 0
+    rows = []          # (request, position, plain logits, rounding model's logits or None)
     for rid, toks in requests.items():
         ref, margins, chosen = plain_logits(folder, toks, with_margins=True)
+        mine = chosen
         if routing is not None:
             mine = [routing[(rid, p)] for p in range(len(toks))]
             differ = [p for p in range(len(toks)) if not same_choice(mine[p], chosen[p])]
-            for p in differ:
-                assert margins[p] < flip_margin, (f"{what}: request {rid} position {p}: the engine chose experts "
-                                                  f"{mine[p]}, the plain model {chosen[p]} with a margin of {margins[p]:.3f}")
             if differ:
                 flips += len(differ)
                 cfg, w = _plain_model(folder)
-                ref = plain.forward(cfg, w, list(toks), routing=mine)
+                probs = []
+                ref = plain.forward(cfg, w, list(toks), routing=mine, router_probs=probs)
+                for p in range(len(toks)):
+                    for j, ids in enumerate(mine[p]):
+                        assert near_tie_choice(ids, probs[p][j], flip_margin), (
+                            f"{what}: request {rid} position {p} sparse layer {j}: the engine chose experts {ids}, "
+                            f"the plain router's probabilities are {[round(x, 5) for x in probs[p][j]]}")
+            else:
+                mine = chosen
+        model = None
+        if storage is not None:
+            assert storage == "bfloat16"
+            model = stored_logits(folder, toks, mine)
         for p in range(len(toks)):
             assert (rid, p) in got, f"{what}: no logits for request {rid} position {p}"
-            g = got[(rid, p)].double()
-            assert torch.isfinite(g).all(), f"{what}: non-finite logits for {rid} position {p}"
-            total += 1
-            err = (g - ref[p]).abs()
-            bound = atol + rtol * ref[p].abs() + stol * float(ref[p].std())
-            if (err > bound).any():
-                i = int((err - bound).argmax())
-                raise AssertionError(f"{what}: request {rid} position {p} vocab {i}: engine {float(g[i]):.7f}, "
-                                     f"plain {float(ref[p][i]):.7f}, |diff| {float(err[i]):.3e} > {float(bound[i]):.3e}")
-            if float(err.max()) > worst:
-                worst, worst_at = float(err.max()), (rid, p)
-    # a flip is only accepted above where the plain model's own margin is below `flip_margin`; their
-    # share must stay small (one position is the least a short trace can show)
-    assert flips <= max(1, 0.1 * total), f"{what}: {flips} of {total} positions were routed differently"
-    print(f"[{what}] largest |engine - plain| = {worst:.3e} at {worst_at}; {flips}/{total} positions routed on a near-tie")
+            rows.append((rid, p, ref[p], model[p] if model is not None else None))
+    r, rel, noise_rows = 0.0, 0.0, []
+    if storage is not None:
+        noise_rows = [float(((m - ref) / ref.std()).pow(2).mean()) for _, _, ref, m in rows]
+        r = (sum(noise_rows) / len(noise_rows)) ** 0.5
+        for _, _, ref, m in rows:
+            far = ref.abs() > OUTLIER * ref.std()
+            if far.any():
+                rel = max(rel, float(((m - ref).abs() / ref.abs())[far].max()))
+    mine_sq, n_elems = 0.0, 0
+    for k, (rid, p, ref, model_row) in enumerate(rows):
+        g = got[(rid, p)].double()
+        assert torch.isfinite(g).all(), f"{what}: non-finite logits for {rid} position {p}"
+        total += 1
+        if storage is None:
+            err = (g - ref).abs()
+            bound = atol + rtol * ref.abs()
+        else:
+            err = (g - model_row).abs()
+            bound = torch.full_like(err, NOISE_SIGMAS * max(r, noise_rows[k] ** 0.5) * float(ref.std()))
+            bound = bound + OUTLIER_FACTOR * rel * ref.abs() * (ref.abs() > OUTLIER * ref.std())
+            mine_sq += float((err / ref.std()).pow(2).sum())
+            n_elems += err.numel()
+        if (err > bound).any():
+            i = int((err - bound).argmax())
+            other = f"rounding model {float(model_row[i]):.7f}, " if storage is not None else ""
+            raise AssertionError(f"{what}: request {rid} position {p} vocab {i}: engine {float(g[i]):.7f}, {other}"
+                                 f"plain {float(ref[i]):.7f}, |diff| {float(err[i]):.3e} > {float(bound[i]):.3e}")
+        if float(err.max()) > worst:
+            worst, worst_at = float(err.max()), (rid, p)
+    note = ""
+    if storage is not None:
+        mine_rms = (mine_sq / max(1, n_elems)) ** 0.5
+        note = (f"; rms/spread: engine - rounding model {mine_rms:.4f}, rounding model - plain {r:.4f}; outliers move "
+                f"by up to {rel:.4f} of themselves in the rounding model")
+        assert mine_rms <= RMS_FACTOR * r, (f"{what}: the engine deviates from the rounding model by {mine_rms:.4f} spreads "
+                                            f"(rms); rounding at the stored tensors alone moves the logits by {r:.4f}")
+    print(f"[{what}] largest |engine - {'rounding model' if storage else 'plain'}| = {worst:.3e} at {worst_at}; {flips}/{total} positions routed on a near-tie{note}")
     return worst

@@ -51,6 +51,10 @@ def test_defaults_are_reported():
     ({"quantization_config": {"bits": 4}}, "quantized"),
     ({"mlp_only_layers": [7]}, "mlp_only_layers"),
     ({"head_dim": 15}, "head_dim"),
+    ({"head_dim": 24}, "head_dim"),                       # even, but no multiple of 16: refused when read, not at the first step
+    ({"head_dim": 272}, "head_dim"),
+    ({"num_experts": 1025}, "num_experts"),
+    ({"num_experts": 64, "num_experts_per_tok": 33}, "num_experts_per_tok"),
     ({"use_sliding_window": True, "sliding_window": 0, "max_window_layers": 0}, "sliding_window"),
     ({"rms_norm_eps": -1.0}, "rms_norm_eps"),
 ])

@@ -101,22 +101,17 @@ def test_combine_of_many_rows_equals_that_of_few(T, H, k, S, sorted_rows):
 @pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
 def test_gemm_every_wide_tile(tile, M, N, K):
     """The many-row kernel picks its tile by the sizes; here each tile shape is made to run the same products."""
-    from ferrox_amd import ops
-    from ferrox_amd.csrc.build import load_library
-    lib = load_library("gemm")
+    from ferrox_amd import debug, ops
     dtype = torch.bfloat16
     a, w, bias = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1), rnd(N, dtype=dtype, seed=2)
     ref = a.double() @ w.double().T
     h = rnd(M, N, seed=3)
     h0 = h.clone()
-    lib.fx_gemm_set_wide(tile)
-    try:
+    with debug.kernel_switch("gemm", "wide", tile):
         got = ops.gemm(a, w, bias=bias)
         ops.gemm(a, w, epilogue=ops.EPI_RESID, out=h)
         w2 = rnd(2 * N, K, dtype=dtype, seed=4, scale=0.5)
         act = ops.gemm(a, w2, epilogue=ops.EPI_SILU_MUL)
-    finally:
-        lib.fx_gemm_set_wide(1)
     close(got, ref + bias.double(), dtype, "store+bias")
     close(h, h0.double() + ref, dtype, "residual")
     close(act, plain.silu(a.double() @ w2[:N].double().T) * (a.double() @ w2[N:].double().T), dtype, "silu(gate)*up")
@@ -125,9 +120,7 @@ def test_gemm_every_wide_tile(tile, M, N, K):
 @pytest.mark.parametrize("tile", [12, 256])
 def test_grouped_gemm_tiles_agree(tile):
     """An expert's rows in tiles of 192 (weights three steps deep) and of 256 give the same sums."""
-    from ferrox_amd import ops
-    from ferrox_amd.csrc.build import load_library
-    lib = load_library("gemm")
+    from ferrox_amd import debug, ops
     T, E, k, I, H = 900, 6, 2, 64, 256
     x = rnd(T, H, dtype=torch.bfloat16)
     w_gu = rnd(E, 2 * I, H, dtype=torch.bfloat16, seed=1, scale=0.3)
@@ -136,11 +129,8 @@ def test_grouped_gemm_tiles_agree(tile):
     first = torch.where(torch.rand(T, generator=g) < 0.66, 0, 1)
     ids = torch.stack([first, 2 + torch.randint(0, E - 2, (T,), generator=g)], dim=1).to(torch.int32).to(DEV)
     offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
-    lib.fx_gemm_set_wide(tile)
-    try:
+    with debug.kernel_switch("gemm", "wide", tile):
         act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
-    finally:
-        lib.fx_gemm_set_wide(1)
     xs = x.double()[sorted_token.long()]
     off = offsets.cpu().tolist()
     assert off[1] - off[0] > 256
@@ -439,9 +429,68 @@ def test_qkv_product_that_rotates_and_writes_the_cache(later, T, H, nh, nkv, hd,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,bs,rot,interleaved", [(3, 1, 32, 8, 32, False), (2, 2, 64, 16, 32, False),
+                                                          (2, 1, 48, 8, 24, True), (4, 2, 128, 64, 128, False)])
+def test_rope_with_frequency_factors(dtype, nh, nkv, hd, bs, rot, interleaved):
+    """A table of per-pair factors divides the angles (ferrox-core/src/attention.rs:319-333): the rotating
+    kernel, and for bfloat16 split halves also the q/k/v product that rotates in its epilogue, against the
+    formula; a table of ones gives the bits of no table."""
+    from ferrox_amd import ops
+    theta, T = 1e4, 20
+    g = torch.Generator().manual_seed(rot)
+    factors = (1.0 + 7.0 * torch.rand(rot // 2, generator=g)).to(DEV)
+    q, k, v = rnd(T, nh * hd, dtype=dtype), rnd(T, nkv * hd, dtype=dtype, seed=1), rnd(T, nkv * hd, dtype=dtype, seed=2)
+    pos = torch.arange(3, 3 + T, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    n_blocks = -(-(3 + T) // bs)
+    table = torch.arange(n_blocks, dtype=torch.int32, device=DEV).flip(0)[None].contiguous()
+    pages = lambda: (torch.zeros(n_blocks, nkv, bs, hd, dtype=dtype, device=DEV), torch.zeros(n_blocks, nkv, hd, bs, dtype=dtype, device=DEV))
+
+    def want(x, heads):
+        x = x.double().cpu().reshape(T, heads, hd)
+        i = torch.arange(rot // 2, dtype=torch.float64)
+        ang = pos.double().cpu()[:, None] * (1.0 / theta ** (2 * i / rot))[None, :] / factors.double().cpu()[None, :]
+        c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        out = x.clone()
+        ia, ib = (2 * i.long(), 2 * i.long() + 1) if interleaved else (i.long(), i.long() + rot // 2)
+        out[..., ia], out[..., ib] = x[..., ia] * c - x[..., ib] * s_, x[..., ia] * s_ + x[..., ib] * c
+        return out
+
+    kp, vp = pages()
+    q1 = q.clone()
+    ops.rope_kv_write(q1, k, v, pos, seq, table, kp, vp, nh, nkv, hd, bs, rot, theta, interleaved, freq_factors=factors)
+    close(q1.reshape(T, nh, hd), want(q, nh), dtype, "rotated queries")
+    page_of, slot = table[0].cpu()[(pos.cpu() // bs).long()].long(), (pos.cpu() % bs).long()
+    close(kp.cpu()[page_of, :, slot, :], want(k, nkv), dtype, "key pages")
+    # a table of ones is no table
+    ones = torch.ones(rot // 2, device=DEV)
+    kp1, vp1 = pages()
+    kp0, vp0 = pages()
+    qa, qb = q.clone(), q.clone()
+    ops.rope_kv_write(qa, k, v, pos, seq, table, kp1, vp1, nh, nkv, hd, bs, rot, theta, interleaved, freq_factors=ones)
+    ops.rope_kv_write(qb, k, v, pos, seq, table, kp0, vp0, nh, nkv, hd, bs, rot, theta, interleaved)
+    assert torch.equal(qa, qb) and torch.equal(kp1, kp0)
+    with pytest.raises(ops.KernelError):
+        ops.rope_kv_write(qa, k, v, pos, seq, table, kp1, vp1, nh, nkv, hd, bs, rot, theta, interleaved, freq_factors=ones[:-1])
+    if dtype == torch.bfloat16 and not interleaved and rot % 32 == 0 and hd % 32 == 0:
+        H = 96
+        w = rnd((nh + 2 * nkv) * hd, H, dtype=dtype, seed=5, scale=0.1)
+        x = rnd(T, H, dtype=dtype, seed=6)
+        assert ops.can_qkv_rope(x, w, T, hd, rot, False)
+        k1, v1 = pages()
+        got = ops.qkv_rope(x, w, None, pos, seq, table, k1, v1, nh, nkv, hd, bs, rot, theta, freq_factors=factors)
+        ref = ops.gemm(x, w)
+        qw, kvw = nh * hd, nkv * hd
+        k2, v2 = pages()
+        ops.rope_kv_write(ref[:, :qw], ref[:, qw:qw + kvw], ref[:, qw + kvw:], pos, seq, table, k2, v2, nh, nkv, hd, bs, rot,
+                          theta, freq_factors=factors)
+        assert torch.equal(got[:, :qw], ref[:, :qw]) and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,hd,bs,window", [(4, 4, 16, 16, 0), (3, 1, 32, 8, 16), (6, 3, 48, 4, 40), (2, 2, 128, 64, 0),
                                                  (8, 2, 80, 16, 7), (4, 1, 256, 32, 100), (4, 2, 64, 64, 50), (3, 1, 128, 128, 90),
-                                                 (2, 1, 64, 64, 0)])
+                                                 (2, 1, 64, 64, 0), (2, 2, 128, 64, 70)])
 def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
     """Whole sequences through the tiled kernel, and their last tokens again through the decode
     kernel, against the plain attention on the same rotated, rounded q/k/v."""

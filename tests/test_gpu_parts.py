@@ -13,7 +13,7 @@ from ferrox_amd import ops
 from ferrox_amd.engine.model import Model
 from ferrox_amd.engine.runner import ModelRunner, StepEntry
 from ferrox_amd.parts import (FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, FeedForward, LayerSpec, Mixer, ModelSpec,
-                              ParamSpec, PartSpec, PositionEncoding, ScheduleEntry)
+                              ParamSpec, PartSpec, PositionEncoding, Rotary, ScheduleEntry)
 from ferrox_amd.weights import RandomSource
 
 pytestmark = pytest.mark.gpu
@@ -66,6 +66,61 @@ class RunningMean(Mixer):
             mean = run / (ctx.positions[b:e].float()[:, None] + 1.0)
             y = mean.to(self.weight.dtype) @ self.weight.T
             ops.residual_add(residual[b:e], y.contiguous())
+
+
+@MIXERS.register("test_window_mean")
+class WindowMean(Mixer):
+    """y_t = W * mean(x_s for t - span < s <= t): a mixer that keeps its inputs in pages of a cache group of its
+    own, which ages by a window; written with torch operations on device tensors only, so that a decode step can
+    be recorded (`graph_safe`): nothing is read from the context's host lists, every index comes from
+    `positions`, `token_seq` and the block table."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, span: int):
+        self.hidden_size, self.span, self.window = hidden_size, span, span
+        self.weight = None
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec((self.hidden_size, self.hidden_size))}
+
+    def load(self, fetch):
+        self.weight = fetch("mix.weight")
+
+    def cache_group(self):
+        return ("test_window_mean", self.span), self.span
+
+    def page_shapes(self, block_size):
+        return {"x": (block_size, self.hidden_size)}
+
+    def forward(self, x, ctx, cache, residual):
+        pages, table, bs = cache.pages["x"], ctx.block_tables[cache.group], cache.block_size
+        pos, seq = ctx.positions.long(), ctx.token_seq.long()
+        pages[table[seq, pos // bs].long(), pos % bs] = x                                  # write, then read
+        back = pos[:, None] - torch.arange(self.span, device=x.device)[None, :]           # [T, span] positions read
+        seen = back >= 0
+        back = back.clamp_min(0)
+        rows = pages[table[seq[:, None], back // bs].long(), back % bs].float()            # [T, span, H]
+        mean = (rows * seen[:, :, None]).sum(1) / seen.sum(1, keepdim=True)
+        ops.residual_add(residual, (mean.to(self.weight.dtype) @ self.weight.T).contiguous())
+
+
+@POSITION_ENCODINGS.register("test_banded_rope")
+class BandedRope(PositionEncoding):
+    """Split-half rotary whose pair i turns slower by a factor of its own, 1 + 8 |b_i| with b a tensor of the
+    checkpoint: the kernels rotate, the part only hands them the table."""
+
+    def __init__(self, head_dim: int, theta: float):
+        self.head_dim, self.theta = head_dim, theta
+        self.factors = None
+
+    def param_specs(self):
+        return {"bands": ParamSpec((self.head_dim // 2,))}
+
+    def load(self, fetch):
+        self.factors = (1.0 + 8.0 * fetch("bands").float().abs()).contiguous()
+
+    def rotary(self):
+        return Rotary(self.head_dim, self.theta, False, self.factors)
 
 
 @POSITION_ENCODINGS.register("test_decay_positions")
@@ -351,3 +406,82 @@ def test_another_position_encoding_and_a_feed_forward_with_routing(dtype, tol):
     # (the two toy parts call library matrix products, whose rounding depends on the number of rows:
     # whole and cut agree within the tolerance, not bit for bit)
     assert float((whole - want)[keep].abs().max()) < tol * scale and float((cut - want)[keep].abs().max()) < tol * scale
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_a_recordable_mixer_with_a_cache_group_of_its_own(dtype, tol):
+    """registered above from outside the package: it names its own cache group (pages that a window of its own
+    ages), and its decode steps are recorded and replayed like the built-in attention's, with no change to the
+    step function"""
+    H, V, span, bs = 32, 50, 5, 4
+    layers = [layer(0, H, PartSpec("test_window_mean", {"hidden_size": H, "span": span}, prefix="wm."), PartSpec("test_no_ffn")),
+              layer(1, H, attention_spec(H, 2, 2, 16), PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 48}, prefix="mlp."))]
+    model, w = build(spec_of(H, V, layers), dtype)
+    assert model.cache_groups() == {("test_window_mean", span): span, ("full",): None}
+    # the mixer's own group gets few pages (a whole prompt of 45 tokens takes 12 of them for the length of its
+    # step): they are given back as its window passes them, and taken again
+    runner = ModelRunner(model, block_size=bs, num_pages={("full",): 40, ("test_window_mean", span): 13}, max_seqs=3)
+    assert runner.use_graphs and runner.storage.caches[0].pages["x"].shape == (13, bs, H)
+    reqs = {"a": TOKS, "b": TOKS[5:30], "c": TOKS[::-1]}
+    whole = ru.run_trace(runner, ru.trace_whole(reqs))
+    steps = [{"entries": [{"id": r, "tokens": t[:6], "want": list(range(6))} for r, t in reqs.items()], "end": []}]
+    for i in range(6, len(TOKS)):                                     # then all three decode in lockstep, recorded
+        live = [r for r, t in reqs.items() if i < len(t)]
+        steps.append({"entries": [{"id": r, "tokens": [reqs[r][i]], "want": [0]} for r in live],
+                      "end": [r for r in live if i == len(reqs[r]) - 1]})
+    decoded = ru.run_trace(runner, steps)
+    assert {key[0] for key in runner._graphs} == {2, 3}, "the decode steps were not recorded"
+    for key in whole:
+        assert float((whole[key] - decoded[key]).abs().max()) <= tol * float(whole[key].abs().max()), key
+    toks = reqs["a"]
+    T = len(toks)
+    h = w["emb.weight"][torch.tensor(toks)]
+    x = plain.rms_norm(h, w["l0.n1.weight"], 1e-5)
+    mean = torch.stack([x[max(0, t - span + 1):t + 1].mean(0) for t in range(T)])
+    h = h + mean @ w["l0.wm.mix.weight"].T
+    x = plain.rms_norm(h, w["l1.n1.weight"], 1e-5)
+    proj = lambda n: x @ w[f"l1.attn.{n}_proj.weight"].T + w[f"l1.attn.{n}_proj.bias"]
+    q, k, v = (plain.rope_neox_rows(proj("q").reshape(T, 2, 16), range(T), 1e4),
+               plain.rope_neox_rows(proj("k").reshape(T, 2, 16), range(T), 1e4), proj("v").reshape(T, 2, 16))
+    h = h + plain.causal_attention(q, k, v, 2, 2, None).reshape(T, 32) @ w["l1.attn.o_proj.weight"].T
+    x = plain.rms_norm(h, w["l1.n2.weight"], 1e-5)
+    h = h + plain.swiglu_mlp(x, w["l1.mlp.gate_proj.weight"], w["l1.mlp.up_proj.weight"], w["l1.mlp.down_proj.weight"])
+    want = head_of(w, h)
+    got = torch.stack([decoded[("a", p)] for p in range(T)]).double()
+    assert float((got - want).abs().max()) < tol * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_a_rotary_with_a_table_of_frequency_factors(dtype, tol):
+    """registered above from outside the package; the table reaches the rotating kernels (the one that rotates
+    and writes the cache, and for few bfloat16 tokens the q/k/v product that does so in its epilogue)"""
+    H, V, nh, nkv, hd, theta, T = 64, 50, 2, 1, 32, 300.0, len(TOKS)
+    mixer = PartSpec("paged_attention", {"hidden_size": H, "n_heads": nh, "n_kv_heads": nkv, "head_dim": hd, "bias": True,
+                                         "window": None, "position": PartSpec("test_banded_rope", {"head_dim": hd, "theta": theta},
+                                                                              prefix="pos.")}, prefix="attn.")
+    model, w = build(spec_of(H, V, [layer(0, H, mixer, PartSpec("test_no_ffn"))]), dtype, std=0.3)
+    assert "l0.attn.pos.bands" in model.named_params()
+    whole, cut = run_whole_and_cut(model, TOKS, block_size=16)
+    h = w["emb.weight"][torch.tensor(TOKS)]
+    x = plain.rms_norm(h, w["l0.n1.weight"], 1e-5)
+    proj = lambda n: x @ w[f"l0.attn.{n}_proj.weight"].T + w[f"l0.attn.{n}_proj.bias"]
+    factors = 1.0 + 8.0 * w["l0.attn.pos.bands"].abs()
+    assert float(factors.max()) > 2.0
+
+    def rotate(t):
+        out = t.clone()
+        for p in range(T):
+            for i in range(hd // 2):
+                ang = p / (theta ** (2 * i / hd)) / float(factors[i])
+                a, b = t[p, :, i], t[p, :, i + hd // 2]
+                out[p, :, i], out[p, :, i + hd // 2] = a * math.cos(ang) - b * math.sin(ang), a * math.sin(ang) + b * math.cos(ang)
+        return out
+
+    q, k, v = rotate(proj("q").reshape(T, nh, hd)), rotate(proj("k").reshape(T, nkv, hd)), proj("v").reshape(T, nkv, hd)
+    want = head_of(w, h + plain.causal_attention(q, k, v, nh, nkv, None).reshape(T, nh * hd) @ w["l0.attn.o_proj.weight"].T)
+    unbanded = head_of(w, h + plain.causal_attention(plain.rope_neox_rows(proj("q").reshape(T, nh, hd), range(T), theta),
+                                                      plain.rope_neox_rows(proj("k").reshape(T, nkv, hd), range(T), theta),
+                                                      v, nh, nkv, None).reshape(T, nh * hd) @ w["l0.attn.o_proj.weight"].T)
+    scale = float(want.abs().max())
+    assert float((unbanded - want).abs().max()) > 10 * tol * scale, "the factors make no difference in this test"
+    assert float((whole - want).abs().max()) < tol * scale and float((cut - want).abs().max()) < tol * scale

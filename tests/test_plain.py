@@ -191,6 +191,124 @@ def test_prefix_property_and_bias_is_live(tiny):
     assert torch.equal(plain.forward(untied, w1, toks), full)
 
 
+# ---- the block's wiring --------------------------------------------------------
+WIRING = {"num_hidden_layers": 2, "hidden_size": 24, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 8,
+          "num_experts": 3, "num_experts_per_tok": 2, "norm_topk_prob": False, "moe_intermediate_size": 10,
+          "shared_expert_intermediate_size": 12, "intermediate_size": 14, "decoder_sparse_step": 1,
+          "mlp_only_layers": [1], "vocab_size": 40, "rope_theta": 100.0, "rms_norm_eps": 1e-30,
+          "use_sliding_window": False, "tie_word_embeddings": False}
+
+
+def wiring_weights(cfg, scale=0.4):
+    """random tensors under the checkpoint's names (layer 0 sparse with a shared expert, layer 1 dense)"""
+    g = torch.Generator().manual_seed(11)
+    r = lambda *shape: torch.randn(*shape, dtype=D, generator=g) * scale
+    H, hd = cfg["hidden_size"], cfg["head_dim"]
+    qw, kvw = cfg["num_attention_heads"] * hd, cfg["num_key_value_heads"] * hd
+    w = {"model.embed_tokens.weight": r(cfg["vocab_size"], H), "lm_head.weight": r(cfg["vocab_size"], H),
+         "model.norm.weight": 1 + r(H)}
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        w[p + "input_layernorm.weight"], w[p + "post_attention_layernorm.weight"] = 1 + r(H), 1 + r(H)
+        for n, rows in (("q", qw), ("k", kvw), ("v", kvw)):
+            w[p + f"self_attn.{n}_proj.weight"], w[p + f"self_attn.{n}_proj.bias"] = r(rows, H), r(rows)
+        w[p + "self_attn.o_proj.weight"] = r(H, qw)
+        if plain.layer_is_sparse(cfg, l):
+            I, S = cfg["moe_intermediate_size"], cfg["shared_expert_intermediate_size"]
+            w[p + "mlp.gate.weight"] = r(cfg["num_experts"], H)
+            for e in range(cfg["num_experts"]):
+                for n, shape in (("gate", (I, H)), ("up", (I, H)), ("down", (H, I))):
+                    w[p + f"mlp.experts.{e}.{n}_proj.weight"] = r(*shape)
+            for n, shape in (("gate", (S, H)), ("up", (S, H)), ("down", (H, S))):
+                w[p + f"mlp.shared_expert.{n}_proj.weight"] = r(*shape)
+            w[p + "mlp.shared_expert_gate.weight"] = r(1, H)
+        else:
+            I = cfg["intermediate_size"]
+            for n, shape in (("gate", (I, H)), ("up", (I, H)), ("down", (H, I))):
+                w[p + f"mlp.{n}_proj.weight"] = r(*shape)
+    return w
+
+
+WIRING_TOKENS = [3, 17, 5, 5, 39, 0, 21, 8, 30, 11, 2]
+
+
+def test_norms_stand_before_the_sublayers():
+    """Pre-norm (ferrox-models/src/decoder.rs:1-5, 2155-2173): every sublayer reads norm(h) and adds into h, so
+    scaling what enters the residual stream (the embedding and each sublayer's last matrix) by c scales h by c
+    everywhere and leaves the logits alone (eps -> 0).  A norm after a sublayer, a sublayer that reads h itself,
+    or a residual taken from the normed rows would each break this."""
+    w = wiring_weights(WIRING)
+    base = plain.forward(WIRING, w, WIRING_TOKENS)
+    into_stream = [n for n in w if n == "model.embed_tokens.weight" or n.endswith("o_proj.weight")
+                   or n.endswith("down_proj.weight")]
+    assert len(into_stream) == 1 + 2 + 3 + 1 + 1
+    scaled = {n: (t * 7.5 if n in into_stream else t) for n, t in w.items()}
+    assert torch.allclose(plain.forward(WIRING, scaled, WIRING_TOKENS), base, atol=1e-9)
+    # and each of them matters: scaling one alone changes the logits
+    for n in into_stream:
+        one = dict(w, **{n: w[n] * 7.5})
+        assert not torch.allclose(plain.forward(WIRING, one, WIRING_TOKENS), base, atol=1e-6), n
+    # the final norm is applied (scaling the last layer's output alone would otherwise scale the logits)
+    assert float(base.abs().max()) < 1e3
+
+
+def test_values_are_not_rotated_and_queries_are_rotated_whole():
+    """With zero q and k every score is zero, attention is the running mean of the values, and those are
+    W_v x + b_v as they are: no rotation (ferrox-models/src/decoder.rs:2106-2111 rotates q and k only), head h
+    of the output reading kv head h // group (ferrox-core/src/attention.rs:432-438).  And with q and k back, the
+    rotation covers the whole head: changing the last pair's partner dimension changes the scores."""
+    cfg = dict(WIRING, num_hidden_layers=1, mlp_only_layers=[0])
+    w = wiring_weights(cfg)
+    p = "model.layers.0."
+    for n in ("q", "k"):
+        w[p + f"self_attn.{n}_proj.weight"] = torch.zeros_like(w[p + f"self_attn.{n}_proj.weight"])
+        w[p + f"self_attn.{n}_proj.bias"] = torch.zeros_like(w[p + f"self_attn.{n}_proj.bias"])
+    T, H, nh, nkv, hd = len(WIRING_TOKENS), 24, 4, 2, 8
+    h = w["model.embed_tokens.weight"][torch.tensor(WIRING_TOKENS)]
+    x = plain.rms_norm(h, w[p + "input_layernorm.weight"], 1e-30)
+    v = (x @ w[p + "self_attn.v_proj.weight"].T + w[p + "self_attn.v_proj.bias"]).reshape(T, nkv, hd)
+    mean = torch.cumsum(v, 0) / torch.arange(1, T + 1, dtype=D)[:, None, None]
+    a = torch.stack([mean[:, hh // (nh // nkv)] for hh in range(nh)], dim=1)            # [T, nh, hd], head-major
+    h = h + a.reshape(T, nh * hd) @ w[p + "self_attn.o_proj.weight"].T
+    x2 = plain.rms_norm(h, w[p + "post_attention_layernorm.weight"], 1e-30)
+    h = h + plain.swiglu_mlp(x2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    want = plain.rms_norm(h, w["model.norm.weight"], 1e-30) @ w["lm_head.weight"].T
+    assert torch.allclose(plain.forward(cfg, w, WIRING_TOKENS), want, atol=1e-10)
+    # rotation over the whole head: q = k = one-hot in the last dimension of the first half of head 0 and
+    # its partner (dimension hd-1); a rotation of fewer dimensions would leave these scores position-free
+    w = wiring_weights(cfg)
+    q, k = torch.zeros(T, nh, hd, dtype=D), torch.zeros(T, nkv, hd, dtype=D)
+    q[:, :, hd // 2 - 1] = 1.0
+    k[:, :, hd // 2 - 1] = 1.0
+    rq, rk = plain.rope_neox_rows(q, range(T), 100.0), plain.rope_neox_rows(k, range(T), 100.0)
+    assert float(rq[5, 0, hd - 1].abs()) > 1e-3                                         # the pair (hd/2-1, hd-1) turns
+    s = torch.einsum("td,sd->ts", rq[:, 0], rk[:, 0])
+    assert abs(float(s[9, 2] - s[8, 1])) < 1e-12 and abs(float(s[9, 2] - s[9, 3])) > 1e-6
+
+
+def test_heads_are_concatenated_head_major():
+    """Permuting whole heads of q, k and v together with the matching column blocks of o_proj changes nothing
+    (ferrox-models/src/decoder.rs:2150-2157: the heads' outputs lie one after the other); a concat that
+    interleaves the heads' dimensions would not survive it.  Permuting the column blocks alone does change it."""
+    cfg, w = WIRING, wiring_weights(WIRING)
+    base = plain.forward(cfg, w, WIRING_TOKENS)
+    nh, nkv, hd = 4, 2, 8
+    group = nh // nkv
+    kv_perm = [1, 0]
+    q_perm = [kv_perm[hh // group] * group + hh % group for hh in range(nh)]             # q heads follow their kv head
+    rows = lambda perm: torch.cat([torch.arange(hh * hd, (hh + 1) * hd) for hh in perm])
+    moved, only_o = dict(w), dict(w)
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}.self_attn."
+        for n, perm in (("q", q_perm), ("k", kv_perm), ("v", kv_perm)):
+            moved[p + f"{n}_proj.weight"] = w[p + f"{n}_proj.weight"][rows(perm)]
+            moved[p + f"{n}_proj.bias"] = w[p + f"{n}_proj.bias"][rows(perm)]
+        moved[p + "o_proj.weight"] = w[p + "o_proj.weight"][:, rows(q_perm)]
+        only_o[p + "o_proj.weight"] = w[p + "o_proj.weight"][:, rows(q_perm)]
+    assert torch.allclose(plain.forward(cfg, moved, WIRING_TOKENS), base, atol=1e-10)
+    assert not torch.allclose(plain.forward(cfg, only_o, WIRING_TOKENS), base, atol=1e-6)
+
+
 # ---- sampler ----------------------------------------------------------------
 def test_xorshift_stream():
     r = plain.XorShift64(1)
