@@ -9,6 +9,7 @@
 // attention.rs:146-175 over tiles of 64 keys that start at multiples of 64, so a
 // query's result does not depend on what else is computed with it.
 #include "common.h"
+#include "attention.h"
 
 FX_DEFINE_LAST_ERROR()
 
@@ -1084,5 +1085,63 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
+                              chunk, waves);
+}
+
+// ---------------------------------------------------------------------------
+// fx_attn_decode_static: fx_attn_decode for callers that cannot allocate (see attention.h).  The chunks' partial
+// results, which fx_attn_decode's caller brings in part_o and part_ml, live in this array instead.  Each GPU that
+// the library runs on holds its own copy until the process ends.  Every call on a GPU uses that GPU's copy from its
+// start: two calls that overlap on one GPU (two streams, two threads) race; calls that follow each other on one
+// stream do not.  Nothing in it has to start at zero: every chunk writes its (m, l) and its outputs before the merge
+// reads them, and the merge reads no chunk of another call's larger shape.
+// ---------------------------------------------------------------------------
+#define FX_ATTN_STATIC_FLOATS (4u << 20)       // 16 MiB: e.g. 64 queries x 16 heads x 31 chunks x (128 + 2) floats
+static __device__ __align__(256) float fx_attn_scratch[FX_ATTN_STATIC_FLOATS];
+
+#define FX_MAX_DEVICES 64
+static float* g_attn_scratch_ptr[FX_MAX_DEVICES];    // per device: the address of that device's copy (null: not asked yet)
+
+// The array's name is only a host-side stand-in; its memory on the current device is found with
+// hipGetSymbolAddress, once per device, with that device current.
+static int attn_scratch_of_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    FX_REQUIRE(e == hipSuccess, "attn_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+    FX_REQUIRE(dev >= 0 && dev < FX_MAX_DEVICES, "attn_decode_static: device %d is beyond the %d this library keeps", dev, FX_MAX_DEVICES);
+    float* p = __atomic_load_n(&g_attn_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(fx_attn_scratch));
+        FX_REQUIRE(e == hipSuccess && sym, "attn_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        p = (float*)sym;
+        __atomic_store_n(&g_attn_scratch_ptr[dev], p, __ATOMIC_RELEASE);     // (two threads would store the same address)
+    }
+    *out = p;
+    return 0;
+}
+
+FX_API int fx_attn_static_init(void) {
+    float* p;
+    return attn_scratch_of_current_device(&p);
+}
+
+FX_API long fx_attn_static_capacity(void) { return (long)FX_ATTN_STATIC_FLOATS; }
+
+FX_API int fx_attn_decode_static(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
+                                 const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
+                                 const int* positions, const int* item_seq, const int* item_tok, int n_items,
+                                 int nh, int nkv, int hd, int bs, int window, float scale, int splits, int chunk, int waves) {
+    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, splits, chunk)) return 1;
+    if (n_items <= 0) return 0;
+    const size_t n_o = (size_t)n_items * nh * splits * hd, n_ml = (size_t)n_items * nh * splits * 2;
+    FX_REQUIRE(n_o + n_ml <= FX_ATTN_STATIC_FLOATS,
+               "attn_decode_static: %d queries x %d heads x %d chunks x (%d + 2) floats = %zu are more than the %u this entry "
+               "point holds; use fewer chunks or fx_attn_decode with buffers of your own",
+               n_items, nh, splits, hd, n_o + n_ml, FX_ATTN_STATIC_FLOATS);
+    float* scratch = nullptr;
+    if (attn_scratch_of_current_device(&scratch)) return 1;
+    return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
+                              item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, scratch, scratch + n_o, splits,
                               chunk, waves);
 }

@@ -54,7 +54,11 @@ def _host_compiler() -> str | None:
 
 
 def _sources(name: str) -> tuple:
-    return (name + ".cpp",) if name in HOST_LIBRARIES else (name + ".hip",) + HEADERS
+    """The file that is compiled first, then what it includes (all of it goes into the hash)."""
+    if name in HOST_LIBRARIES:
+        return (name + ".cpp",)
+    own = (name + ".h",) if os.path.isfile(os.path.join(HERE, name + ".h")) else ()
+    return (name + ".hip",) + HEADERS + own
 
 
 def _source_hash(name: str) -> str:
