@@ -201,7 +201,9 @@ class Bench:
                      max_tokens_per_step=2048, prefill_chunk=2048, ctx_size=ctx + new_tokens + 8)
         eng.time_steps = True
         prompts = self.prompts(batch, ctx)
-        eng.generate(prompts[:1], max_new_tokens=4, ignore_eos=True)               # loads and records what it needs
+        # once untimed: decode steps are recorded (a HIP graph per number of sequences and length bound) the first
+        # time their shape occurs, which costs a few hundred ms that a serving process pays once
+        eng.generate(prompts, max_new_tokens=new_tokens, ignore_eos=True)
         self.torch.cuda.synchronize()
         t0 = time.perf_counter()
         out = eng.generate(prompts, max_new_tokens=new_tokens, ignore_eos=True)
@@ -291,11 +293,12 @@ def run_workload(name: str, args) -> int:
     bs = args.block_size
     results = []
 
-    def serve(prompts, new_tokens, chunk, budget, max_seqs, pages, label):
+    def serve(prompts, new_tokens, chunk, budget, max_seqs, pages, label, warm=True):
         eng = Engine(model=model, block_size=bs, num_pages=pages, max_seqs=max_seqs, max_tokens_per_step=budget,
                      prefill_chunk=chunk, ctx_size=cfg["max_position_embeddings"])
         eng.time_steps = True
-        eng.generate([prompts[0][:64]], max_new_tokens=2, ignore_eos=True)
+        if warm:                                   # record the decode graphs of this batch shape ahead of the timed run
+            eng.generate([p[:max(2, min(len(p), 64))] for p in prompts], max_new_tokens=min(new_tokens, 4), ignore_eos=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         out = eng.generate(prompts, max_new_tokens=new_tokens, ignore_eos=True)

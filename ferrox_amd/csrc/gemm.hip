@@ -1074,12 +1074,16 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 // Switches for tests and measurement (ferrox_amd/debug.py is their one caller): they pick, whatever the sizes,
 // a kernel variant that the sizes would otherwise choose.  The product path never sets them.
 static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per wave of the product for few rows (0: by the sizes)
+static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
+static int g_skinny_waves = 0; // "skinny_waves": 4 or 8 waves that split K in a block of that product (0: by the sizes)
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
 static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "skinny_sets")) { g_skinny_nw = value; return 0; }
+    if (!strcmp(key, "skinny_row_tiles")) { g_skinny_mt = value; return 0; }
+    if (!strcmp(key, "skinny_waves")) { g_skinny_waves = value; return 0; }
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
-    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, wide)", key);
+    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, wide)", key);
     return 1;
 }
 
@@ -1117,9 +1121,20 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
     }
 }
 
-// mt: row tiles per block (1, 2, 4); nw: 16-row weight sets per wave.  Four waves split K (eight stream no faster).
-static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int m_tiles, hipStream_t s) {
+// mt: row tiles per block (1, 2, 4); nw: 16-row weight sets per wave; waves: 4 or 8 split K.
+static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int waves, int m_tiles, hipStream_t s) {
 #define FX_SK(MT_, W_, NW_) launch_skinny_cfg<MT_, W_, NW_>(g, epi, m_tiles, s)
+    if (waves == 8 && mt * nw <= 4) {
+        if (nw == 2) {
+            if (mt == 1) FX_SK(1, 8, 2);
+            else FX_SK(2, 8, 2);
+        } else {
+            if (mt == 1) FX_SK(1, 8, 1);
+            else if (mt == 2) FX_SK(2, 8, 1);
+            else FX_SK(4, 8, 1);
+        }
+        return;
+    }
     if (nw == 2) {
         if (mt == 1) FX_SK(1, 4, 2);
         else if (mt == 2) FX_SK(2, 4, 2);
@@ -1234,7 +1249,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > 32 && K % 64 == 0 &&
                               !g_no_wide && ceil_div(N, 128) >= 512;
     if (g.vec_ok && (per_group <= 64 || pair_ids) && !many_columns) {
-        const int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
+        int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
+        if (g_skinny_mt && !pair_ids) mt = g_skinny_mt;
         const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16 + n_always
                                      : M / (16 * mt) + (expert_offsets ? nonempty : (M % (16 * mt) != 0));
         const bool dual = epi == EPI_SILU_MUL;
@@ -1244,7 +1260,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 160) ? 2 : 1;
         if (!dual && (norm_w || (M <= 2 && (long)ceil_div(N, 16) * m_tiles >= 4096))) nw = 1;
         if ((g_skinny_nw == 1 && !dual) || (g_skinny_nw == 2 && !norm_w)) nw = g_skinny_nw;
-        launch_skinny(g, epi, mt, nw, m_tiles, s);
+        launch_skinny(g, epi, mt, nw, g_skinny_waves == 8 ? 8 : 4, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }

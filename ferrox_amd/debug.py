@@ -21,7 +21,8 @@ import ctypes
 
 import torch
 
-KERNEL_SWITCH_DEFAULTS = {("gemm", "skinny_sets"): 0, ("gemm", "wide"): 1, ("attention", "direct_stages"): 2}
+KERNEL_SWITCH_DEFAULTS = {("gemm", "skinny_sets"): 0, ("gemm", "skinny_row_tiles"): 0, ("gemm", "skinny_waves"): 0,
+                          ("gemm", "wide"): 1, ("attention", "direct_stages"): 2}
 
 
 class RoutingTrace:
