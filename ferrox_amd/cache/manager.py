@@ -59,6 +59,9 @@ def _native():
         lib.fxc_pack_step.restype = ctypes.c_long
         lib.fxc_pack_step.argtypes = [ctypes.c_void_p, ctypes.c_int, _I64P, _I32P, _I32P, _I32P, _I32P, ctypes.c_int,
                                       ctypes.c_int, ctypes.c_void_p, ctypes.c_long, _I32P, _I32P, _I32P]
+        lib.fxc_pack_decode.restype = ctypes.c_long
+        lib.fxc_pack_decode.argtypes = [ctypes.c_void_p, ctypes.c_int, _I64P, _I32P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                        _I32P, ctypes.c_int, ctypes.c_void_p, ctypes.c_long, _I32P]
         _lib = lib
     return _lib
 
@@ -311,9 +314,12 @@ class CacheManager:
             raise ValueError(msg)
         return PackedStep(int(total), int(sizes[0]), int(sizes[1]), int(sizes[2]), starts[:n].tolist(), lens[:n].tolist())
 
-    def pack_decode(self, reqs: list, tokens: list, vocab: int, out_ptr: int, capacity: int, force_blocks: int) -> None:
-        """pack_step for the common step in which every request brings one token and wants its logits;
-        the arrays that do not change from step to step are kept from the last call."""
+    def pack_decode(self, reqs: list, tokens: list, vocab: int, out_ptr: int, capacity: int, force_blocks: int,
+                    pad_to: int | None = None, pad_pages: list | None = None, pad_slot: int = 0) -> None:
+        """The common step in which every request brings one token and wants its logits, laid out for
+        `pad_to` >= len(reqs) sequences: the rows past the requests are stand-ins that write to the page
+        `pad_pages[group]` and the state slot `pad_slot`, which no request owns.  The arrays that do not
+        change from step to step are kept from the last call."""
         n = len(reqs)
         key = tuple(reqs)
         kept = self._decode_arrays
@@ -324,19 +330,21 @@ class CacheManager:
                 if h is None:
                     raise ValueError(f"request {r!r} was not admitted")
                 handles[i] = h
-            kept = self._decode_arrays = (key, handles, np.ones(n, dtype=np.int32), np.arange(n + 1, dtype=np.int32),
-                                          np.zeros(n, dtype=np.int32), np.zeros(3, dtype=np.int32),
-                                          np.zeros(n, dtype=np.int32), np.zeros(n, dtype=np.int32))
-        _, handles, ones, want_start, want, sizes, starts, lens = kept
+            kept = self._decode_arrays = (key, handles, np.zeros(n, dtype=np.int32))
+        _, handles, lens = kept
         try:
             toks = np.asarray(tokens, dtype=np.int32).reshape(-1)
         except (OverflowError, TypeError, ValueError) as e:
             raise ValueError(f"token ids must be integers: {e}") from None
         if toks.size != n:
             raise ValueError("one token per request")
+        pads = np.asarray(pad_pages if pad_pages is not None else [0] * len(self.groups), dtype=np.int32)
+        if pads.size != len(self.groups):
+            raise ValueError("one stand-in page per group")
         ip = lambda a: a.ctypes.data_as(_I32P)
-        total = self._lib.fxc_pack_step(self._h, n, handles.ctypes.data_as(_I64P), ip(ones), ip(toks), ip(want_start),
-                                        ip(want), vocab, force_blocks, out_ptr, capacity, ip(sizes), ip(starts), ip(lens))
+        total = self._lib.fxc_pack_decode(self._h, n, handles.ctypes.data_as(_I64P), ip(toks), vocab, force_blocks,
+                                          n if pad_to is None else int(pad_to), ip(pads), int(pad_slot), out_ptr, capacity,
+                                          ip(lens))
         if total < 0:
             self._decode_arrays = None
             raise ValueError(self._core.error())

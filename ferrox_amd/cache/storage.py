@@ -1,9 +1,11 @@
 """Device memory behind the cache manager's page ids and slot ids.
 
 Each schedule entry with a cache of its own gets, for every page tensor its
-mixer names, a slab [num_pages, *page_shape], and for every state tensor a slab
-[n_slots, *state_shape].  An entry that reads another entry's cache sees that
-entry's page slabs, read-only.
+mixer names, a slab [num_pages + 1, *page_shape], and for every state tensor a slab
+[n_slots + 1, *state_shape].  An entry that reads another entry's cache sees that
+entry's page slabs, read-only.  The one page and the one slot past the manager's
+own belong to no request: the stand-in rows that fill a recorded decode step up
+to its fixed number of sequences write there (`pad_page`, `pad_slot`).
 """
 from __future__ import annotations
 
@@ -16,6 +18,8 @@ class CacheStorage:
     def __init__(self, model, manager, dtype: torch.dtype, device):
         self.caches: list[LayerCache] = []
         self.bytes = 0
+        self.pad_pages = [g.pool.num_pages for g in manager.groups.values()]     # per group, in the manager's order
+        self.pad_slot = manager.slots.n_slots
         bs = manager.block_size
         for i, e in enumerate(model.schedule):
             mixer = model.blocks[e.layer].mixer
@@ -23,7 +27,7 @@ class CacheStorage:
             key = mixer.cache_group()[0] if shapes else None
             state = {}
             for name, (shape, sdtype) in mixer.state_shapes().items():
-                state[name] = torch.zeros((manager.slots.n_slots, *shape), dtype=sdtype or dtype, device=device)
+                state[name] = torch.zeros((manager.slots.n_slots + 1, *shape), dtype=sdtype or dtype, device=device)
                 self.bytes += state[name].numel() * state[name].element_size()
             if e.cache is not None:
                 owner = self.caches[e.cache]
@@ -33,7 +37,7 @@ class CacheStorage:
             if shapes:
                 n = manager.groups[key].pool.num_pages
                 for name, shape in shapes.items():
-                    pages[name] = torch.zeros((n, *shape), dtype=dtype, device=device)
+                    pages[name] = torch.zeros((n + 1, *shape), dtype=dtype, device=device)
                     self.bytes += pages[name].numel() * pages[name].element_size()
             self.caches.append(LayerCache(pages, state, key, bs, writes=True))
 

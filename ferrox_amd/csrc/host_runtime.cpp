@@ -332,3 +332,61 @@ FX_API long fxc_pack_step(void* h, int n, const int64_t* reqs, const int* n_tok,
     sizes[2] = max_blocks;
     return total;
 }
+
+// A step in which each of n requests brings one token and wants its logits, laid out for pad_to >= n sequences
+// (a recorded step has a fixed number of them):
+//   tokens[N] | positions[N] | token_seq[N] | slots[N] | rows[N] | tables[groups][N][max_blocks],  N = pad_to.
+// Rows n .. N-1 are stand-ins that no request owns: token 0 at position 0 of a sequence of its own, whose one
+// block in group g is pad_pages[g] (a page beyond the pool, which the device slabs hold for this purpose) and
+// whose state slot is pad_slot; what they compute is never looked at.  `lens` receives the n lengths after the
+// step.  Returns the number of int32 written, or -2 with a message.
+FX_API long fxc_pack_decode(void* h, int n, const int64_t* reqs, const int* tokens, int vocab, int force_blocks,
+                            int pad_to, const int* pad_pages, int pad_slot, int* out, long cap, int* lens) {
+    Manager* m = (Manager*)h;
+    if (pad_to < n) return fail(m, "a step of %ld sequences cannot be laid out for %ld", n, pad_to);
+    int max_blocks = 1;
+    for (int e = 0; e < n; ++e) {
+        Seq* s = m->find(reqs[e]);
+        if (!s) return fail(m, "request %ld was not admitted", (long)reqs[e]);
+        if (s->length < 1) return fail(m, "request %ld: more tokens than reserved positions (%ld)", (long)reqs[e], s->length);
+        for (int f = 0; f < e; ++f)
+            if (reqs[f] == reqs[e]) return fail(m, "request %ld appears twice in one step", (long)reqs[e]);
+        const int id = tokens[e];
+        if (vocab >= 0 && (id < 0 || id >= vocab)) return fail(m, "token id %ld is outside the vocabulary of %ld", id, vocab);
+        lens[e] = s->length;
+        max_blocks = std::max(max_blocks, m->blocks_for(s->length));
+    }
+    if (force_blocks > 0) {
+        if (force_blocks < max_blocks) return fail(m, "tables of %ld blocks cannot hold %ld", force_blocks, max_blocks);
+        max_blocks = force_blocks;
+    }
+    const long N = pad_to, G = (long)m->pools.size();
+    const long total = 5 * N + G * N * max_blocks;
+    if (total > cap) return fail(m, "step buffer of %ld words is too small for %ld", cap, total);
+    int* o_tok = out;
+    int* o_pos = out + N;
+    int* o_seq = out + 2 * N;
+    int* o_slot = out + 3 * N;
+    int* o_rows = out + 4 * N;
+    int* o_tab = out + 5 * N;
+    for (long e = 0; e < N; ++e) {
+        Seq* s = e < n ? m->find(reqs[e]) : nullptr;
+        o_tok[e] = s ? tokens[e] : 0;
+        o_pos[e] = s ? s->length - 1 : 0;
+        o_seq[e] = (int)e;
+        o_slot[e] = s ? s->slot : pad_slot;
+        o_rows[e] = (int)e;
+        for (long g = 0; g < G; ++g) {
+            int* row = o_tab + (g * N + e) * max_blocks;
+            for (int b = 0; b < max_blocks; ++b) {
+                if (s) {
+                    const std::vector<int>& tab = s->tables[g];
+                    row[b] = (b < (int)tab.size() && tab[b] >= 0) ? tab[b] : 0;
+                } else {
+                    row[b] = pad_pages[g];
+                }
+            }
+        }
+    }
+    return total;
+}

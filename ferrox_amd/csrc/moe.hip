@@ -271,12 +271,21 @@ static int align_groups_per_row(long n, int E, size_t bytes, size_t* shm) {
     return (int)per_row;
 }
 
+// After the experts, `n_always` further ones that each of the n / k tokens takes (a shared expert cut into pieces):
+// piece s owns the sorted rows n + s T .. n + (s + 1) T, row n + s T + t being token t, and its output row has the
+// same number.
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int n, int k, int E, int per_row,
                                                          int* __restrict__ expert_offsets,
                                                         int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
-                                                        int* __restrict__ inv) {
+                                                        int* __restrict__ inv, int n_always) {
     extern __shared__ int lds[];
     align_block(ids, n, k, E, per_row, lds, lds + E + 1, expert_offsets, sorted_token, sorted_pair, inv);
+    const int T = n / k;
+    for (int i = threadIdx.x; i < n_always * T; i += blockDim.x) {
+        sorted_token[n + i] = i % T;
+        if (sorted_pair) sorted_pair[n + i] = n + i;
+    }
+    for (int s = threadIdx.x; s < n_always; s += blockDim.x) expert_offsets[E + 1 + s] = n + (s + 1) * T;
 }
 
 // Many pairs: the same sort by many blocks, in two launches.  First every wave counts the experts of its
@@ -566,11 +575,12 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
 
 // gcnt: room for ceil(n / 64) * E ints (or null: one block does it all, whatever n)
 FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* expert_offsets,
-                        int* sorted_token, int* sorted_pair, int* inv, int* gcnt) {
+                        int* sorted_token, int* sorted_pair, int* inv, int* gcnt, int n_always) {
     FX_REQUIRE(n >= 0 && k > 0 && n % k == 0, "moe_align: n=%d must be a multiple of k=%d", n, k);
+    FX_REQUIRE(n_always >= 0 && (n_always == 0 || n <= 2048), "moe_align: experts that every token takes are for up to 2048 pairs");
     FX_REQUIRE(E >= 1, "moe_align: E=%d", E);
     FX_REQUIRE(E <= 4096, "moe_align: %d experts are more than this kernel's 4096", E);
-    if (gcnt && n > 2048 && (size_t)(E + 1 + E + 2 * SORT_WAVES * E) * 4 <= 60 * 1024) {
+    if (gcnt && n > 2048 && !n_always && (size_t)(E + 1 + E + 2 * SORT_WAVES * E) * 4 <= 60 * 1024) {
         const int G = (n + 63) / 64, blocks = (G + SORT_WAVES - 1) / SORT_WAVES;
         moe_count_kernel<<<blocks, SORT_WAVES * 64, (size_t)SORT_WAVES * E * 4, (hipStream_t)stream>>>(ids, n, E, gcnt);
         FX_CHECK_LAUNCH("moe_count");
@@ -583,7 +593,7 @@ FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* 
     const int per_row = align_groups_per_row(n, E, 60 * 1024, &shm);
     const int nt = n > 4096 ? 1024 : (n > 256 ? 512 : 256);
     moe_align_kernel<<<1, nt, shm, (hipStream_t)stream>>>(ids, n, k, E, per_row, expert_offsets, sorted_token, sorted_pair,
-                                                          inv);
+                                                          inv, n_always);
     FX_CHECK_LAUNCH("moe_align");
     return 0;
 }

@@ -70,14 +70,16 @@ class DecodeGraph:
         return ctx
 
     def run(self, entries) -> torch.Tensor:
+        """The logits of the entries' tokens (one each).  Fewer entries than the step was recorded for are
+        filled up with stand-in rows, which write to a page and a slot that no request owns."""
         self.copied.synchronize()                  # the last upload has left the staging buffer
-        if all(e.want[0] == 0 for e in entries):
-            self.runner.manager.pack_decode([e.req for e in entries], [e.tokens[0] for e in entries],
-                                            self.runner.vocab_size, self._host_ptr, self._host_words, self.max_blocks)
-        else:
-            self.runner.manager.pack_step([e.req for e in entries], [e.tokens for e in entries],
-                                          [e.want for e in entries], self.runner.vocab_size, self._host_ptr,
-                                          self._host_words, force_blocks=self.max_blocks)
+        for e in entries:
+            if e.want[0] != 0:
+                raise ValueError(f"request {e.req!r}: wanted place {e.want[0]} is outside its one token")
+        storage = self.runner.storage
+        self.runner.manager.pack_decode([e.req for e in entries], [e.tokens[0] for e in entries], self.runner.vocab_size,
+                                        self._host_ptr, self._host_words, self.max_blocks, pad_to=self.n,
+                                        pad_pages=storage.pad_pages, pad_slot=storage.pad_slot)
         if self.runner.before_launch is not None:
             self.runner.before_launch()
         self.meta.copy_(self.host, non_blocking=True)
@@ -106,7 +108,7 @@ class DecodeGraph:
         self.graph.replay()
         if debug.routing_trace is not None:
             debug.routing_trace.replayed(self.trace_calls)
-        return self.logits
+        return self.logits[:len(entries)]
 
 
 class ModelRunner:
@@ -170,11 +172,14 @@ class ModelRunner:
             # every sequence brings one token and wants its logits: a recorded decode step
             longest = max(mgr.length(r) for r in reqs)
             bound = -(-longest // self.graph_kv_step) * self.graph_kv_step
-            key = (n_seqs, bound, debug.graph_token())
+            # more than eight sequences are recorded in steps of eight and filled up with stand-in rows: a batch
+            # that shrinks by one request at a time then records a step once in eight times, not every time
+            n_rec = n_seqs if n_seqs <= 8 else -(-n_seqs // 8) * 8
+            key = (n_rec, bound, debug.graph_token())
             if key not in self._graphs:
-                if len(self._graphs) >= 16:
+                if len(self._graphs) >= 32:
                     self._graphs.pop(next(iter(self._graphs)))
-                self._graphs[key] = DecodeGraph(self, n_seqs, bound)
+                self._graphs[key] = DecodeGraph(self, n_rec, bound)
             try:
                 logits = self._graphs[key].run(entries)
             except RuntimeError as err:

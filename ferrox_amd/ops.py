@@ -73,7 +73,7 @@ _sigs = {
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
                               c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 5,
-    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
 }
@@ -492,18 +492,21 @@ def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE
     return x, ids, weights, gate
 
 
-def moe_align(ids: torch.Tensor, n_experts: int):
+def moe_align(ids: torch.Tensor, n_experts: int, always: int = 0):
     """For ids [T, k]: (expert_offsets [E+1], sorted_token [n], sorted_pair [n], inv [n]): sorted row i
-    belongs to pair sorted_pair[i] = t*k + j of token sorted_token[i]; inv is the inverse map."""
+    belongs to pair sorted_pair[i] = t*k + j of token sorted_token[i]; inv is the inverse map.
+    `always` = S: S further experts follow that every token takes (a shared expert cut into pieces): the
+    offsets have E+1+S entries and the sorted arrays n + S*T, piece s owning rows n + s*T + t (token t), whose
+    output rows have the same numbers (up to 2048 pairs)."""
     T, k = ids.shape
     n = T * k
     dev = ids.device
-    offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
-    buf = torch.empty((3, n), dtype=torch.int32, device=dev)
+    offsets = torch.empty((n_experts + 1 + always,), dtype=torch.int32, device=dev)
+    buf = torch.empty((3, n + always * T), dtype=torch.int32, device=dev)
     # many pairs are sorted by many blocks, which hand each other the counts of every group of 64 pairs
     gcnt = torch.empty((-(-n // 64), n_experts), dtype=torch.int32, device=dev) if n > 2048 else None
     _call("moe", "fx_moe_align", _stream(), _p(_i32(ids, "ids")), n, k, n_experts, _p(offsets), _p(buf[0]), _p(buf[1]),
-          _p(buf[2]), _p(gcnt))
+          _p(buf[2]), _p(gcnt), int(always))
     return offsets, buf[0], buf[1], buf[2]
 
 

@@ -129,13 +129,32 @@ class SparseMoE(FeedForward):
         if T <= 16 and ids.numel() <= 64 and aligned:       # the expert products take the pairs unsorted
             self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None), then_norm=then_norm)
         else:
-            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts),
-                         then_norm=then_norm)
+            # the shared expert's pieces ride along as experts that every token takes, behind the sorted pairs
+            S = self.shared_pieces if x.dtype == self.w_gate_up_all.dtype and ids.numel() <= 2048 else 0
+            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts, always=S),
+                         then_norm=then_norm, sorted_pieces=S)
         return True
 
-    def forward(self, x, ctx, residual, routed=None, then_norm=None) -> None:
+    def forward(self, x, ctx, residual, routed=None, then_norm=None, sorted_pieces: int = 0) -> None:
         T = x.shape[0]
         then = self._then(then_norm, ctx, T)
+        if sorted_pieces:
+            # up to 64 tokens, sorted pairs: the shared expert as `sorted_pieces` pieces behind the experts in the same
+            # two launches (its own two products would stream its weights to 64 rows far below the memory's speed)
+            ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
+            if debug.routing_trace is not None:
+                debug.routing_trace.put(ids)
+            S, n = sorted_pieces, ids.numel()
+            kb = dict(w_kblocked=True) if self.kblocked else {}
+            debug.region("experts gate/up")
+            act = matmul(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets,
+                         n_rows=n + S * T, **kb)
+            debug.region("experts down")
+            y = matmul(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
+            debug.region("combine")
+            ctx.carry = ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate,
+                                        **then)
+            return
         if routed is not None and routed[3] is None and self.shared_pieces and x.dtype == self.w_gate_up_all.dtype:
             # few tokens, unsorted pairs, shared expert as pieces: two launches do all experts
             ids, weights, gate = routed[:3]

@@ -194,3 +194,30 @@ def test_pack_decode_writes_what_pack_step_writes():
         m.pack_decode(["c", "b"], [5, 100], 100, got.ctypes.data, 4096, 6)
     with pytest.raises(ValueError, match="not admitted"):
         m.pack_decode(["zz"], [5], 100, got.ctypes.data, 4096, 6)
+
+
+def test_pack_decode_fills_up_with_stand_in_rows():
+    """a recorded step has a fixed number of sequences: the rows past the requests are a token 0 at position 0 of a
+    sequence whose only block is the group's stand-in page and whose state slot is the stand-in slot"""
+    import numpy as np
+    m = CacheManager({FULL: None, WIN: 16}, 16, block_size=8, n_slots=4)
+    for r, n in (("a", 21), ("b", 40)):
+        m.admit(r)
+        m.extend(r, n)
+    N, mb = 5, 6
+    got = np.full(4096, -7, dtype=np.int32)
+    m.pack_decode(["b", "a"], [7, 3], 100, got.ctypes.data, 4096, mb, pad_to=N, pad_pages=[16, 17], pad_slot=4)
+    assert got[:N].tolist() == [7, 3, 0, 0, 0]
+    assert got[N:2 * N].tolist() == [39, 20, 0, 0, 0]
+    assert got[2 * N:3 * N].tolist() == [0, 1, 2, 3, 4] and got[4 * N:5 * N].tolist() == [0, 1, 2, 3, 4]
+    assert got[3 * N:4 * N].tolist() == [m.slot("b"), m.slot("a"), 4, 4, 4]
+    o = 5 * N
+    assert got[o:o + mb].tolist() == m.table("b", FULL) + [0] and got[o + mb:o + 2 * mb].tolist() == m.table("a", FULL) + [0] * 3
+    assert got[o + 2 * mb:o + 5 * mb].tolist() == [16] * (3 * mb)                   # stand-ins, group FULL
+    o += N * mb
+    assert got[o:o + mb].tolist() == [max(x, 0) for x in m.table("b", WIN)] + [0]
+    assert got[o + 2 * mb:o + 5 * mb].tolist() == [17] * (3 * mb)                   # stand-ins, group WIN
+    assert got[5 * N + 2 * N * mb] == -7
+    with pytest.raises(ValueError, match="cannot be laid out"):
+        m.pack_decode(["b", "a"], [7, 3], 100, got.ctypes.data, 4096, mb, pad_to=1, pad_pages=[16, 17], pad_slot=4)
+    m.check_invariants()

@@ -395,19 +395,23 @@ def test_recorded_decode_steps_equal_launched_ones(model_folders):
         assert float((replayed[key] - launched[key]).abs().max()) <= 1e-2 * float(launched[key].abs().max()), key
 
 
-def trace_lockstep_decode(requests: dict, tail: int, prefill_together: int = 8) -> list:
-    """All requests live at once: their heads go in a few steps of several whole prompts each,
-    then every step carries one token of every request (what a serving batch of decodes looks like)."""
+def trace_lockstep_decode(requests: dict, tail: int, prefill_together: int = 8, stagger: int = 1) -> list:
+    """All requests live at once: their heads go in a few steps of several whole prompts each, then every
+    step carries one token of every request that has tokens left (what a serving batch of decodes looks
+    like).  Request i decodes its last tail - i % stagger tokens, so with stagger > 1 the batch shrinks
+    step by step towards the end."""
     steps, ids = [], list(requests)
+    tails = {rid: tail - i % stagger for i, rid in enumerate(ids)}
     for o in range(0, len(ids), prefill_together):
         entries = []
         for rid in ids[o:o + prefill_together]:
-            head = len(requests[rid]) - tail
+            head = len(requests[rid]) - tails[rid]
             entries.append({"id": rid, "tokens": requests[rid][:head], "want": list(range(head))})
         steps.append({"entries": entries, "end": []})
     for i in range(tail):
-        steps.append({"entries": [{"id": rid, "tokens": [requests[rid][len(requests[rid]) - tail + i]], "want": [0]}
-                                  for rid in ids], "end": ids if i == tail - 1 else []})
+        live = [rid for rid in ids if i < tails[rid]]
+        steps.append({"entries": [{"id": rid, "tokens": [requests[rid][len(requests[rid]) - tails[rid] + i]], "want": [0]}
+                                  for rid in live], "end": [rid for rid in live if i == tails[rid] - 1]})
     return steps
 
 
@@ -427,8 +431,11 @@ def test_recorded_decode_steps_of_many_requests(model_folders, name, n_live, dty
     folder, runner = runner_for(model_folders, name, dtype, block_size=bs, num_pages=pages, max_seqs=n_live)
     assert runner.use_graphs
     routing = {} if dtype == "bfloat16" else None
-    got = ru.run_trace(runner, trace_lockstep_decode(reqs, tail), routing)
-    assert any(key[0] == n_live for key in runner._graphs), "the decode steps were not recorded"
+    # (from 9 sequences on a step is recorded for the next multiple of eight and filled up with stand-in rows; the
+    # requests finish a few at a time, so the batch shrinks through several recorded sizes)
+    got = ru.run_trace(runner, trace_lockstep_decode(reqs, tail, stagger=5), routing)
+    sizes = {key[0] for key in runner._graphs}
+    assert -(-n_live // 8) * 8 in sizes and len(sizes) >= 2, f"recorded sizes {sorted(sizes)}"
     assert runner.manager.n_free_pages() == pages
     check(got, folder, reqs, dtype, f"{name} {dtype} {n_live} requests decoded from graphs", routing)
 
@@ -444,7 +451,8 @@ def test_recorded_decode_steps_at_production_width(model_folders):
         folder, runner = runner_for(model_folders, "D", "bfloat16", block_size=64, num_pages=n_live + 2, max_seqs=n_live)
         routing = {}
         got = ru.run_trace(runner, trace_lockstep_decode(reqs, tail, prefill_together=5), routing)
-        assert any(key[0] == n_live for key in runner._graphs), "the decode steps were not recorded"
+        recorded = n_live if n_live <= 8 else -(-n_live // 8) * 8          # from nine on: the next multiple of eight
+        assert any(key[0] == recorded for key in runner._graphs), "the decode steps were not recorded"
         check(got, folder, reqs, "bfloat16", f"D bfloat16 {n_live} requests decoded from graphs", routing, cfg["hidden_size"])
 
 

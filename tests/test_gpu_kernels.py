@@ -703,6 +703,36 @@ def test_sort_by_expert_at_large_sizes(T, E, k):
     assert inv.cpu()[order].tolist() == list(range(T * k))
 
 
+@pytest.mark.parametrize("T,E,k,S", [(24, 60, 4, 4), (64, 8, 2, 3), (17, 5, 1, 1), (40, 6, 3, 2)])
+def test_sort_by_expert_with_experts_that_every_token_takes(T, E, k, S):
+    """S further experts behind the sorted pairs, each with all T tokens as its rows (a shared expert cut into
+    pieces), and the grouped products over that layout against one product per expert"""
+    from ferrox_amd import ops
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    plain_sort = ops.moe_align(ids, E)
+    offsets, sorted_token, sorted_pair, _ = ops.moe_align(ids, E, always=S)
+    n = T * k
+    assert offsets.cpu().tolist() == plain_sort[0].cpu().tolist() + [n + (s + 1) * T for s in range(S)]
+    assert sorted_token.cpu().tolist() == plain_sort[1].cpu().tolist() + list(range(T)) * S
+    assert sorted_pair.cpu().tolist() == plain_sort[2].cpu().tolist() + list(range(n, n + S * T))
+    H, I = 64, 32
+    x = rnd(T, H, dtype=torch.bfloat16)
+    w_gu, w_dn = rnd(E + S, 2 * I, H, dtype=torch.bfloat16, seed=1, scale=0.3), rnd(E + S, H, I, dtype=torch.bfloat16, seed=2, scale=0.3)
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=n + S * T)
+    y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+    assert y.shape == (n + S * T, H)
+    xd = x.double().cpu()
+    for s_ in range(S):                      # piece s: every token through expert E + s
+        e = E + s_
+        a = (plain.silu(xd @ w_gu[e, :I].double().cpu().T) * (xd @ w_gu[e, I:].double().cpu().T)).to(torch.bfloat16).double()
+        close(y[n + s_ * T:n + (s_ + 1) * T], a @ w_dn[e].double().cpu().T, torch.bfloat16, f"piece {s_}")
+    t, j = 3 % T, k - 1                      # and a routed pair
+    e = int(ids[t, j])
+    a = (plain.silu(xd[t] @ w_gu[e, :I].double().cpu().T) * (xd[t] @ w_gu[e, I:].double().cpu().T)).to(torch.bfloat16).double()
+    close(y[t * k + j], a @ w_dn[e].double().cpu().T, torch.bfloat16, "a routed pair")
+
+
 @pytest.mark.parametrize("T,E,k", [(1, 8, 2), (8, 60, 4), (64, 60, 4), (33, 130, 8), (65, 6, 3), (300, 60, 4)])
 def test_route_in_one_launch_equals_two(T, E, k):
     """selection and sort fused for small batches give what the two kernels give"""

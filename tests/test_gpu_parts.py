@@ -311,7 +311,7 @@ def test_a_mixer_with_state_of_its_own(dtype, tol):
     model, w = build(spec_of(H, V, layers), dtype)
     assert model.cache_groups() == {("full",): None}
     runner = ModelRunner(model, block_size=8, num_pages=32, max_seqs=3)
-    assert runner.storage.caches[0].state["sum"].shape == (3, H) and not runner.storage.caches[0].pages
+    assert runner.storage.caches[0].state["sum"].shape == (3 + 1, H) and not runner.storage.caches[0].pages    # + the stand-in slot
     reqs = {"a": TOKS, "b": TOKS[5:30], "c": TOKS[::-1]}
     whole = ru.run_trace(runner, ru.trace_whole(reqs))
     mixed = ru.run_trace(runner, ru.trace_mixed(reqs, seed=4, max_live=3))       # slots are taken again, state starts at zero
@@ -421,7 +421,7 @@ def test_a_recordable_mixer_with_a_cache_group_of_its_own(dtype, tol):
     # the mixer's own group gets few pages (a whole prompt of 45 tokens takes 12 of them for the length of its
     # step): they are given back as its window passes them, and taken again
     runner = ModelRunner(model, block_size=bs, num_pages={("full",): 40, ("test_window_mean", span): 13}, max_seqs=3)
-    assert runner.use_graphs and runner.storage.caches[0].pages["x"].shape == (13, bs, H)
+    assert runner.use_graphs and runner.storage.caches[0].pages["x"].shape == (13 + 1, bs, H)      # + the stand-in page
     reqs = {"a": TOKS, "b": TOKS[5:30], "c": TOKS[::-1]}
     whole = ru.run_trace(runner, ru.trace_whole(reqs))
     steps = [{"entries": [{"id": r, "tokens": t[:6], "want": list(range(6))} for r, t in reqs.items()], "end": []}]
