@@ -512,3 +512,21 @@ def test_command_line_generates_and_refuses(model_folders, tmp_path):
     refused(run_cli("-m", str(wrong), "--tokens", ids, "--dtype", "fp32"), "shape")
     refused(run_cli("-m", folder, "--tokens", "1,2,999999", "--dtype", "fp32"), "vocabulary")
     refused(run_cli("-m", folder, "--tokens", ",".join(["1"] * 300), "--dtype", "fp32"), "context")
+
+
+def test_generation_of_a_batch_that_shrinks(model_folders):
+    """twelve requests that ask for different numbers of tokens, through the entry point: the decode batch shrinks one
+    request at a time through the recorded sizes (16 with stand-in rows, then 8 and below as they are), and every
+    request still generates what the plain model generates for it alone"""
+    import plain_qwen2moe as plain
+    from ferrox_amd.engine.api import Engine
+    folder = model_folders("A", "float32")
+    cfg, w = plain.load_folder(folder)
+    prompts = list(ru.make_requests(cfg["vocab_size"], [3 + (5 * i) % 11 for i in range(12)], 21).values())
+    lengths = [4 + i for i in range(12)]
+    engine = Engine(folder, dtype="float32", block_size=16, num_pages=40, max_seqs=12, max_tokens_per_step=64, prefill_chunk=16)
+    got = engine.generate_detailed(prompts, lengths)
+    sizes = {key[0] for key in engine.runner._graphs}
+    assert 16 in sizes and any(n <= 8 for n in sizes), f"recorded sizes {sorted(sizes)}"
+    for p, n, g in zip(prompts, lengths, got):
+        assert g.token_ids == plain.greedy_generate(cfg, w, p, n) and g.finish_reason == "length"
