@@ -697,57 +697,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         // a dead row reads the first row of A instead: its products land in rows that are never stored
         xrow[mt] = NORM ? (live ? (const bf16*)((const float*)g.A + off) : nullptr) : (const bf16*)g.A + off;
     }
-    // rope epilogue: what thread (lane, wave) needs for its pairs of outputs, rows 16 mt + lane % 16, column
-    // 4 (lane / 16) + wave of the two sets, is fetched and worked out here, while the weights are on their way
-    float rope_sn[MT], rope_cs[MT], rope_rstd[MT], rope_b0 = 0.f, rope_b1 = 0.f;
-    size_t rope_page[MT];
-    int rope_slot[MT];
-    if constexpr (ROPE) {
-        const int cc = grp * 4 + wave;
-        const bool to_pages = rope_head >= g.rope_nh && g.rope_k_pages;
-        // first every load that depends on nothing, then the page ids, which need position and sequence
-        int row_of[MT], pos[MT], seq[MT];
-        float total[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            row_of[mt] = min(r0 + 16 * mt + li, r_end - 1);
-            pos[mt] = g.rope_positions[row_of[mt]];
-            seq[mt] = to_pages ? g.rope_token_seq[row_of[mt]] : 0;
-        }
-        // (without a bias the same loads read the positions instead: a branch around them would wait for them)
-        const void* bias_or = g.bias ? g.bias : (const void*)g.rope_positions;
-        const int bias_dt = g.bias ? g.bias_dtype : FX_F32;
-        const RawElement e0 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c0 + cc : 0);
-        const RawElement e1 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c1 + cc : 0);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            total[mt] = g.row_ss ? sum_in_order(g.row_ss + (size_t)row_of[mt] * g.row_ss_n, g.row_ss_n) : 0.f;
-        rope_b0 = element_as_float(e0);
-        rope_b1 = element_as_float(e1);
-        const int p = 16 * rope_j + cc;
-        const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
-        const float freq_div = rope_rotated && g.rope_freq_factors ? g.rope_freq_factors[p] : 1.f;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            rope_page[mt] = 0;
-            rope_slot[mt] = 0;
-            if (to_pages) {
-                rope_page[mt] = (size_t)g.rope_table[(size_t)seq[mt] * g.rope_max_blocks + pos[mt] / g.rope_bs];
-                rope_slot[mt] = pos[mt] % g.rope_bs;
-            }
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            rope_rstd[mt] = g.row_ss ? row_rstd(total[mt], g.K, g.norm_eps) : 1.f;
-            rope_sn[mt] = 0.f;
-            rope_cs[mt] = 1.f;
-            if (rope_rotated) {
-                float angle = (float)pos[mt] * freq;
-                if (g.rope_freq_factors) angle = angle / freq_div;
-                sincosf(angle, &rope_sn[mt], &rope_cs[mt]);
-            }
-        }
-    }
     f32x4_t acc[MT][NW];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -810,14 +759,89 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     constexpr std::false_type masked{};
     const int s_whole = min(s_end, g.K / 128);       // pieces before this one lie inside K
     int sp = wave * per;
+    // Few accumulators leave registers for two pieces (see the loop below).  The first piece's loads leave here,
+    // and so do the old values that a block adds its product to: nothing of the epilogue waits for memory then.
+    constexpr bool TWO = MT * NW <= 4 && !NORM;
+    uint4 w0[TWO ? NW : 1][4], x0[TWO ? MT : 1][4];
+    if constexpr (TWO && !ROPE) {
+        if (sp < s_whole) load_piece(whole, sp, w0, x0);
+    }
+    constexpr int SETS = DUAL ? NW / 2 : NW;      // column groups of a block
+    constexpr int OUTS = MT * SETS;               // accumulator tiles (dual: pairs of them) that become output tiles
+    float old_first[4] = {0.f, 0.f, 0.f, 0.f}, row_scale_first = 1.f;     // of this thread's first output tile
+    if constexpr (EPI == EPI_RESID) {
+        if (tid < OUTS * 64) {
+            const int mt = (tid >> 6) / SETS, a = (tid >> 6) % SETS;
+            const int ml = pairs ? pair_c : r0 + mt * 16 + li;
+            if (pairs ? ml >= 0 : ml < r_end) {
+                const int m = (g.c_rows && !pairs) ? g.c_rows[ml] : ml;
+                if (g.row_scale) row_scale_first = g.row_scale[ml];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    old_first[r] = ((const float*)g.C)[(size_t)m * g.ldc + min(n0 + a * 16 + grp * 4 + r, g.N - 1)];
+            }
+        }
+    }
+    // rope epilogue: what thread (lane, wave) needs for its pairs of outputs, rows 16 mt + lane % 16, column
+    // 4 (lane / 16) + wave of the two sets, is fetched and worked out here, while the weights are on their way
+    float rope_sn[MT], rope_cs[MT], rope_rstd[MT], rope_b0 = 0.f, rope_b1 = 0.f;
+    size_t rope_page[MT];
+    int rope_slot[MT];
+    if constexpr (ROPE) {
+        const int cc = grp * 4 + wave;
+        const bool to_pages = rope_head >= g.rope_nh && g.rope_k_pages;
+        // first every load that depends on nothing, then the page ids, which need position and sequence
+        int row_of[MT], pos[MT], seq[MT];
+        float total[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            row_of[mt] = min(r0 + 16 * mt + li, r_end - 1);
+            pos[mt] = g.rope_positions[row_of[mt]];
+            seq[mt] = to_pages ? g.rope_token_seq[row_of[mt]] : 0;
+        }
+        // (without a bias the same loads read the positions instead: a branch around them would wait for them)
+        const void* bias_or = g.bias ? g.bias : (const void*)g.rope_positions;
+        const int bias_dt = g.bias ? g.bias_dtype : FX_F32;
+        const RawElement e0 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c0 + cc : 0);
+        const RawElement e1 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c1 + cc : 0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            total[mt] = g.row_ss ? sum_in_order(g.row_ss + (size_t)row_of[mt] * g.row_ss_n, g.row_ss_n) : 0.f;
+        rope_b0 = element_as_float(e0);
+        rope_b1 = element_as_float(e1);
+        const int p = 16 * rope_j + cc;
+        const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
+        const float freq_div = rope_rotated && g.rope_freq_factors ? g.rope_freq_factors[p] : 1.f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            rope_page[mt] = 0;
+            rope_slot[mt] = 0;
+            if (to_pages) {
+                rope_page[mt] = (size_t)g.rope_table[(size_t)seq[mt] * g.rope_max_blocks + pos[mt] / g.rope_bs];
+                rope_slot[mt] = pos[mt] % g.rope_bs;
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            rope_rstd[mt] = g.row_ss ? row_rstd(total[mt], g.K, g.norm_eps) : 1.f;
+            rope_sn[mt] = 0.f;
+            rope_cs[mt] = 1.f;
+            if (rope_rotated) {
+                float angle = (float)pos[mt] * freq;
+                if (g.rope_freq_factors) angle = angle / freq_div;
+                sincosf(angle, &rope_sn[mt], &rope_cs[mt]);
+            }
+        }
+    }
     // Few accumulators leave registers for two pieces: the loads of the next piece are then issued before the
     // products of this one, so a wave always has a piece on its way from memory.  Each product follows the
     // loads issued after its own in straight-line code.
-    constexpr bool TWO = MT * NW <= 4 && !NORM;
     if constexpr (TWO) {
         if (sp < s_whole) {
-            uint4 w0[NW][4], x0[MT][4], w1[NW][4], x1[MT][4];
-            load_piece(whole, sp, w0, x0);
+            uint4 w1[NW][4], x1[MT][4];
+            // (the rotating product fetches what its epilogue needs first: behind the weights those short loads
+            // would wait for them, and measured it is slower)
+            if constexpr (ROPE) load_piece(whole, sp, w0, x0);
             for (; sp + 2 < s_whole; sp += 2) {
                 load_piece(whole, sp + 1, w1, x1);
                 multiply_piece(w0, x0);
@@ -899,8 +923,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         }
         return;
     }
-    constexpr int SETS = DUAL ? NW / 2 : NW;      // column groups of a block
-    constexpr int OUTS = MT * SETS;               // accumulator tiles (dual: pairs of them) that become output tiles
     for (int idx = tid; idx < OUTS * 64; idx += WAVES * 64) {
         const int t = idx >> 6, L = idx & 63;
         const int mt = t / SETS, a = t % SETS;
@@ -925,13 +947,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
                 for (int q = 0; q < 4; ++q) total += red_ss[w][mt][(L & 15) + 16 * q];
             rstd = row_rstd(total, g.K, g.norm_eps);
         }
-        // what a row block adds to, and its scale: fetched together, ahead of the stores
+        // what a row block adds to, and its scale: the first tile's came in at the start, a further one's are
+        // fetched together, ahead of the stores
         float old[4] = {0.f, 0.f, 0.f, 0.f}, row_scale = 1.f;
         if (EPI == EPI_RESID) {
-            if (g.row_scale) row_scale = g.row_scale[ml];
+            if (idx == tid) {
+                row_scale = row_scale_first;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                old[r] = ((const float*)g.C)[(size_t)m * g.ldc + min(n0 + a * 16 + (L >> 4) * 4 + r, g.N - 1)];
+                for (int r = 0; r < 4; ++r) old[r] = old_first[r];
+            } else {
+                if (g.row_scale) row_scale = g.row_scale[ml];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    old[r] = ((const float*)g.C)[(size_t)m * g.ldc + min(n0 + a * 16 + (L >> 4) * 4 + r, g.N - 1)];
+            }
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
