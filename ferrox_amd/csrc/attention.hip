@@ -269,6 +269,12 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
     const int hd = a.hd, S = a.splits;
     const float* po = a.part_o + ((size_t)item * a.nh + h) * S * hd;
     const float* pml = a.part_ml + ((size_t)item * a.nh + h) * S * 2;
+    // the first chunks' outputs for this thread's first dimension leave before anything else: they need no weight
+    // to be fetched, only to be used (an empty chunk wrote nothing, and what is read there is dropped below)
+    constexpr int EARLY = 16;
+    float early[EARLY];
+#pragma unroll
+    for (int s = 0; s < EARLY; ++s) early[s] = po[(size_t)min(s, S - 1) * hd + min(tid, hd - 1)];
     float m = NEG_INF;
     for (int s = tid; s < S; s += 128) m = fmaxf(m, pml[2 * s]);
     m = wave_max(m);
@@ -284,8 +290,17 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
     for (int s = 0; s < S; ++s) l += wsm[s] * ((wsm[s] > 0.f) ? pml[2 * s + 1] : 0.f);   // ascending, the same in every thread
     for (int d = tid; d < hd; d += 128) {
         float acc = 0.f;
+        int s0 = 0;
+        if (d == tid) {
+#pragma unroll
+            for (int s = 0; s < EARLY; ++s) {
+                const float w = s < S ? wsm[s] : 0.f;
+                acc = (s < S) ? fmaf(w, (w > 0.f) ? early[s] : 0.f, acc) : acc;
+            }
+            s0 = min(S, EARLY);
+        }
 #pragma unroll 8
-        for (int s = 0; s < S; ++s) {
+        for (int s = s0; s < S; ++s) {
             const float w = wsm[s];
             const float v = (w > 0.f) ? po[(size_t)s * hd + d] : 0.f;   // an empty chunk wrote nothing
             acc = fmaf(w, v, acc);

@@ -1317,9 +1317,13 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         }
         // an expert's share of up to 192 rows: the product streams the weights once and multiplies little, so it
         // is bound by how many of them are on their way; a ring of three weight tiles beside two of the rows
-        const bool few_rows = expert_offsets && (g_wide_force ? g_wide_force == 12 : per_group <= 176);
+        // plain rows: tiles of 192 x 256 where they divide the work more evenly (2,048 rows against 11,264 weight
+        // rows: 484 tiles for two rounds of the 256 CUs instead of 352 tiles of 256 x 256)
+        const double s12 = expert_offsets ? 0.0 : score(192, 256, 0.92);
+        const bool few_rows = g_wide_force ? g_wide_force == 12
+                                           : (expert_offsets ? per_group <= 176 : (s12 > s256 && s12 > s192 && s12 > s128 && s12 > s64));
         if (few_rows)
-            launch_wide<12, 256, 3, 2>(g, epi, M / 192 + nonempty, s);
+            launch_wide<12, 256, 3, 2>(g, epi, M / 192 + (expert_offsets ? nonempty : (M % 192 != 0)), s);
         else if (s192 > s256 && s192 >= s128 && s192 >= s64)
             launch_wide<16, 192, 2>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);
         else if (s256 >= s128 && s256 >= s64)

@@ -97,7 +97,7 @@ def test_combine_of_many_rows_equals_that_of_few(T, H, k, S, sorted_rows):
     close(h_all, want, torch.float32, "combined rows")
 
 
-@pytest.mark.parametrize("tile", [256, 192, 128, 64])
+@pytest.mark.parametrize("tile", [256, 192, 128, 64, 12])      # 12: tiles of 192 rows x 256 weight rows
 @pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
 def test_gemm_every_wide_tile(tile, M, N, K):
     """The many-row kernel picks its tile by the sizes; here each tile shape is made to run the same products."""
