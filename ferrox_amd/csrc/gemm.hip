@@ -647,7 +647,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     for (int mt = 0; mt < MT; ++mt) ss[mt] = 0.f;
     constexpr int NACC = MT * NW;
     constexpr int COLS = DUAL ? 8 * NW : 16 * NW;   // output columns of a block
-    __shared__ f32x4_t red[WAVES][NACC][64];
+    // K is cut into PARTS parts whose sums are added in their order: one part per wave, or, with fewer than four
+    // waves, VW consecutive parts per wave with accumulators of their own, so that one, two and four waves give
+    // the same bits
+    constexpr int VW = WAVES < 4 ? 4 / WAVES : 1, PARTS = WAVES * VW;
+    __shared__ f32x4_t red[PARTS][NACC][64];
     int r0 = 0, r_end = 0, expert = 0, pair_a = -1, pair_c = -1;
     const bool pairs = MT == 1 && g.pair_ids != nullptr;
     if (pairs) {
@@ -697,15 +701,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         // a dead row reads the first row of A instead: its products land in rows that are never stored
         xrow[mt] = NORM ? (live ? (const bf16*)((const float*)g.A + off) : nullptr) : (const bf16*)g.A + off;
     }
-    f32x4_t acc[MT][NW];
+    f32x4_t acc[VW][MT][NW];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int p = 0; p < VW; ++p)
 #pragma unroll
-        for (int a = 0; a < NW; ++a) acc[mt][a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int a = 0; a < NW; ++a) acc[p][mt][a] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     const int n_super = (g.K + 127) / 128;
-    const int per = (n_super + WAVES - 1) / WAVES;
-    const int s_end = min(n_super, (wave + 1) * per);
+    const int per = (n_super + PARTS - 1) / PARTS;      // pieces per part
+    const int s_end = min(n_super, (wave + 1) * VW * per);
     // One piece: its loads (four per set of weight rows and per row tile), then its products.  FULL: the piece
     // lies inside K, so every load is unconditional and the compiler can count the loads in flight.
     auto load_piece = [&](auto full, int sp, uint4 (&w)[NW][4], uint4 (&x)[MT][4]) {
@@ -744,7 +750,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             }
         }
     };
-    auto multiply_piece = [&](const uint4 (&w)[NW][4], const uint4 (&x)[MT][4]) {
+    auto multiply_into = [&](f32x4_t (&to)[MT][NW], const uint4 (&w)[NW][4], const uint4 (&x)[MT][4]) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -752,13 +758,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
                 const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[mt][u]);
 #pragma unroll
                 for (int a = 0; a < NW; ++a)
-                    acc[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[a][u]), xb, acc[mt][a], 0, 0, 0);
+                    to[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[a][u]), xb, to[mt][a], 0, 0, 0);
             }
+    };
+    // piece sp belongs to part sp / per, the (sp / per - wave * VW)-th of this wave (the same for all its lanes)
+    auto multiply_piece = [&](int sp, const uint4 (&w)[NW][4], const uint4 (&x)[MT][4]) {
+        if constexpr (VW == 1) {
+            multiply_into(acc[0], w, x);
+        } else {
+            const int p = sp / per - wave * VW;
+            if (p == 0) multiply_into(acc[0], w, x);
+            else if (p == 1) multiply_into(acc[1], w, x);
+            else if constexpr (VW == 4) {
+                if (p == 2) multiply_into(acc[2], w, x);
+                else multiply_into(acc[3], w, x);
+            }
+        }
     };
     constexpr std::true_type whole{};
     constexpr std::false_type masked{};
     const int s_whole = min(s_end, g.K / 128);       // pieces before this one lie inside K
-    int sp = wave * per;
+    int sp = wave * VW * per;
     // Few accumulators leave registers for two pieces (see the loop below).  The first piece's loads leave here,
     // and so do the old values that a block adds its product to: nothing of the epilogue waits for memory then.
     constexpr bool TWO = MT * NW <= 4 && !NORM;
@@ -844,17 +864,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             if constexpr (ROPE) load_piece(whole, sp, w0, x0);
             for (; sp + 2 < s_whole; sp += 2) {
                 load_piece(whole, sp + 1, w1, x1);
-                multiply_piece(w0, x0);
+                multiply_piece(sp, w0, x0);
                 load_piece(whole, sp + 2, w0, x0);
-                multiply_piece(w1, x1);
+                multiply_piece(sp + 1, w1, x1);
             }
             if (sp + 1 < s_whole) {
                 load_piece(whole, sp + 1, w1, x1);
-                multiply_piece(w0, x0);
-                multiply_piece(w1, x1);
+                multiply_piece(sp, w0, x0);
+                multiply_piece(sp + 1, w1, x1);
                 sp += 2;
             } else {
-                multiply_piece(w0, x0);
+                multiply_piece(sp, w0, x0);
                 sp += 1;
             }
         }
@@ -862,18 +882,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         for (; sp < s_whole; ++sp) {
             uint4 w[NW][4], x[MT][4];
             load_piece(whole, sp, w, x);
-            multiply_piece(w, x);
+            multiply_piece(sp, w, x);
         }
     }
     for (; sp < s_end; ++sp) {          // the piece that K ends in
         uint4 w[NW][4], x[MT][4];
         load_piece(masked, sp, w, x);
-        multiply_piece(w, x);
+        multiply_piece(sp, w, x);
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int p = 0; p < VW; ++p)
 #pragma unroll
-        for (int a = 0; a < NW; ++a) red[wave][mt * NW + a][lane] = acc[mt][a];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int a = 0; a < NW; ++a) red[wave * VW + p][mt * NW + a][lane] = acc[p][mt][a];
     if constexpr (NORM) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) red_ss[wave][mt][lane] = ss[mt];
@@ -890,7 +912,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             if (ml >= r_end) continue;
             f32x4_t v0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v1 = v0;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
+            for (int w = 0; w < PARTS; ++w) {
                 v0 += red[w][mt * NW][L];
                 v1 += red[w][mt * NW + 1][L];
             }
@@ -928,7 +950,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         const int mt = t / SETS, a = t % SETS;
         f32x4_t v = (f32x4_t){0.f, 0.f, 0.f, 0.f}, v2 = v;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
+        for (int w = 0; w < PARTS; ++w) {
             v += red[w][mt * NW + (DUAL ? 2 * a : a)][L];
             if (DUAL) v2 += red[w][mt * NW + 2 * a + 1][L];
         }
@@ -1104,7 +1126,7 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 // a kernel variant that the sizes would otherwise choose.  The product path never sets them.
 static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per wave of the product for few rows (0: by the sizes)
 static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
-static int g_skinny_waves = 0; // "skinny_waves": 4 or 8 waves that split K in a block of that product (0: by the sizes)
+static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
 static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
@@ -1150,7 +1172,7 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
     }
 }
 
-// mt: row tiles per block (1, 2, 4); nw: 16-row weight sets per wave; waves: 4 or 8 split K.
+// mt: row tiles per block (1, 2, 4); nw: 16-row weight sets per wave; waves: 4 or 8 split K (1 or 2 with one row tile).
 static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int waves, int m_tiles, hipStream_t s) {
 #define FX_SK(MT_, W_, NW_) launch_skinny_cfg<MT_, W_, NW_>(g, epi, m_tiles, s)
     if (waves == 8 && mt * nw <= 4) {
@@ -1161,6 +1183,16 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int waves,
             if (mt == 1) FX_SK(1, 8, 1);
             else if (mt == 2) FX_SK(2, 8, 1);
             else FX_SK(4, 8, 1);
+        }
+        return;
+    }
+    if (waves <= 2 && mt == 1) {
+        if (waves == 1) {
+            if (nw == 2) FX_SK(1, 1, 2);
+            else FX_SK(1, 1, 1);
+        } else {
+            if (nw == 2) FX_SK(1, 2, 2);
+            else FX_SK(1, 2, 1);
         }
         return;
     }
@@ -1289,7 +1321,16 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         int nw = (dual || (long)ceil_div(N, 32) * m_tiles >= 160) ? 2 : 1;
         if (!dual && (norm_w || (M <= 2 && (long)ceil_div(N, 16) * m_tiles >= 4096))) nw = 1;
         if ((g_skinny_nw == 1 && !dual) || (g_skinny_nw == 2 && !norm_w)) nw = g_skinny_nw;
-        launch_skinny(g, epi, mt, nw, g_skinny_waves == 8 ? 8 : 4, m_tiles, s);
+        // Waves per block: four, a part of K each.  Unsorted pairs: one wave that runs through all four parts when
+        // the blocks number no more than the 3,072 waves that the GPU holds at a time, else two (a wave then spends
+        // less of its time finding its rows and more of it streaming; measured at the sizes of the engine, one
+        // token's gate/up product 20.5 against 23.3 us, its down product 11.2 against 12.0, sixteen tokens' 96 and
+        // 53 against 104 and 62 us, eight tokens' within 3 %).  The sums are the same bits either way.
+        int waves = 4;
+        if (pair_ids) waves = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles <= 3072 ? 1 : 2;
+        else if (expert_offsets && mt == 1) waves = 2;      // sorted, up to 16 rows per expert: 152 against 159 us at 64 tokens
+        if (g_skinny_waves == 8 || g_skinny_waves == 4 || g_skinny_waves == 2 || g_skinny_waves == 1) waves = g_skinny_waves;
+        launch_skinny(g, epi, mt, nw, waves, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }
