@@ -5,10 +5,13 @@
 extern "C" {
 #endif
 
-// Queries in blocks: item i covers item_n[i] <= 64 consecutive tokens of one sequence.
+// Queries in blocks: item i covers item_n[i] <= tile_q consecutive tokens of one sequence.  tile_q is 64, or 128
+// where fx_attn_tile_queries says so (bfloat16, head_dim 64 or 128, pages of a multiple of 64 keys).
+int fx_attn_tile_queries(int dtype, int hd, int bs);
 int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void* out, long ldo, const void* k_pages,
                   const void* v_pages, const int* block_table, int max_blocks, const int* positions, const int* item_seq,
-                  const int* item_tok, const int* item_n, int n_items, int nh, int nkv, int hd, int bs, int window, float scale);
+                  const int* item_tok, const int* item_n, int n_items, int nh, int nkv, int hd, int bs, int window, float scale,
+                  int tile_q);
 
 // Single queries.  The keys are cut into `splits` chunks of `chunk` positions; the chunks' partial results go through
 // part_o [n_items, nh, splits, hd] and part_ml [n_items, nh, splits, 2] (float32, brought by the caller).

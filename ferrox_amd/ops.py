@@ -62,7 +62,8 @@ _sigs = {
                               c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float],
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
+    ("attention", "fx_attn_tile_queries"): [c_int, c_int, c_int],
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
@@ -374,13 +375,22 @@ def can_fuse_norm(h: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:
             and h.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
+    """The most consecutive queries of a sequence that one item of attention_tiles may cover at these sizes: 64,
+    or 128 where the kernel gives a wave two blocks of 16 queries (every operand it reads then serves two products)."""
+    f, _ = _fn("attention", "fx_attn_tile_queries")
+    return int(f(dtype_code(dtype), int(head_dim), int(block_size)))
+
+
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
-                    n_heads, n_kv_heads, head_dim, block_size, window, scale) -> None:
+                    n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64) -> None:
+    """Blocks of queries: item i is item_n[i] <= tile_q consecutive tokens of sequence item_seq[i] from token
+    item_tok[i] on; tile_q is 64 or attention_tile_queries(...)."""
     _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
           _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
-          int(window or 0), float(scale))
+          int(window or 0), float(scale), int(tile_q))
 
 
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,

@@ -16,14 +16,13 @@ from .. import debug, limits, ops
 from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec, Rotary
 from .linear import Linear, same_dtype
 
-TILE_Q = 64   # queries per work item of the prefill kernels
 NO_ROTATION = Rotary(0, 1.0)
 
 
-def attention_items(ctx):
-    """Work items of a step, shared by all attention layers: sequences with one
+def attention_items(ctx, tile_q: int = 64):
+    """Work items of a step, shared by the attention layers of one item size: sequences with one
     new token go to the split decode kernel, the others are cut into blocks of
-    TILE_Q consecutive queries."""
+    tile_q consecutive queries."""
     if ctx.recorded:      # token t is the one token of sequence t; nothing is made from host lists
         return {"n_decode": ctx.n_seqs, "n_tiles": 0, "max_kv": ctx.kv_bound, "dec_seq": ctx.token_seq,
                 "dec_tok": ctx.token_seq}
@@ -36,10 +35,10 @@ def attention_items(ctx):
             dec_tok.append(b)
             max_kv = max(max_kv, ctx.kv_lens[s])
         else:
-            for t0 in range(b, e, TILE_Q):
+            for t0 in range(b, e, tile_q):
                 t_seq.append(s)
                 t_tok.append(t0)
-                t_n.append(min(TILE_Q, e - t0))
+                t_n.append(min(tile_q, e - t0))
     flat = dec_seq + dec_tok + t_seq + t_tok + t_n
     dev = torch.tensor(flat, dtype=torch.int32, device=ctx.device) if flat else None
     nd, nt = len(dec_seq), len(t_seq)
@@ -114,6 +113,24 @@ class PagedAttention(Mixer):
         w = self.qkv.weight
         return act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0
 
+    def tile_queries(self, ctx, dtype, block_size: int) -> int:
+        """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many and the
+        blocks still fill the GPU's 512 places for them.  Blocks of a portion that starts a prompt differ in work up
+        to the portion's length in keys, so they count by their mean share of the longest (measured at 16 and 28
+        heads of 128: items of 128 gain 8-25 % from 448 such blocks on and lose 10-35 % at 256 and below)."""
+        if ctx.recorded:
+            return 64
+        widest = ops.attention_tile_queries(dtype, self.head_dim, block_size)
+        if widest == 64:
+            return 64
+        even_blocks = 0.0
+        for s in range(ctx.n_seqs):
+            n = ctx.q_starts[s + 1] - ctx.q_starts[s]
+            if n > 1:
+                before = ctx.kv_lens[s] - n
+                even_blocks += -(-n // widest) * self.n_heads * (before + n / 2) / (before + n)
+        return widest if even_blocks >= 400 else 64
+
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
@@ -144,11 +161,13 @@ class PagedAttention(Mixer):
                               rot.interleaved, rot.freq_factors)
         debug.region("attention")
         out = torch.empty((ctx.n_tokens, self.qw), dtype=qkv.dtype, device=qkv.device)
-        items = ctx.memo("attention_items", lambda: attention_items(ctx))
+        tile_q = ctx.memo(f"attention tile {self.n_heads} {self.head_dim} {cache.block_size} {q.dtype}",
+                          lambda: self.tile_queries(ctx, q.dtype, cache.block_size))
+        items = ctx.memo(f"attention_items {tile_q}", lambda: attention_items(ctx, tile_q))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
         if items["n_tiles"]:
             ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
-                                items["tile_seq"], items["tile_tok"], items["tile_n"], *common)
+                                items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q)
         if items["n_decode"]:
             ops.attention_decode(q, out, k_pages, v_pages, table, ctx.positions,
                                  items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"])

@@ -256,24 +256,26 @@ def test_far_key_and_window_edge_stand_out(model_folders):
                     assert float((out[2] - hidden).abs().max()) < tol
 
 
-@pytest.mark.parametrize("hd,bs", [(64, 64), (128, 64), (32, 16)])
-def test_window_edge_inside_a_tile_of_64_queries(hd, bs):
-    """A full tile of 64 queries (the prefill kernels' fast path without per-element masks, and the per-row
-    window edge inside a tile): for several rows the key at distance W-1 stands out and must be found, the key
+@pytest.mark.parametrize("hd,bs,nq", [(64, 64, 64), (128, 64, 64), (32, 16, 64), (64, 64, 128), (128, 64, 128)])
+def test_window_edge_inside_a_tile_of_64_queries(hd, bs, nq):
+    """A full tile of 64 queries, or one item of 128 where the kernel takes them (the prefill kernels' fast path
+    without per-element masks, and the per-row window edge inside a tile): for several rows the key at distance W-1 stands out and must be found, the key
     at distance W stands out and must stay hidden.  For row 16 the edge falls between two tiles of 64 keys,
     which is also a page's edge."""
     import math
     import plain_qwen2moe as plain
     from ferrox_amd import ops
     dev, W, P0, nh, nkv = "cuda:0", 100, 275, 2, 2
-    L = P0 + 64
-    rows = [0, 5, 16, 31, 47, 63]
+    L = P0 + nq
+    rows = [0, 5, 16, 31, 47, 63] + ([64, 70, 80, 111, 127] if nq == 128 else [])
     assert (P0 + 16 - (W - 1)) % 64 == 0 and (P0 + 16 - (W - 1)) % bs == 0
     for dtype in (torch.float32, torch.bfloat16):
+        if nq > 64 and ops.attention_tile_queries(dtype, hd, bs) < nq:
+            continue
         g = torch.Generator().manual_seed(hd + bs)
         k = torch.randn(L, nkv, hd, generator=g) * 0.1
         v = torch.randn(L, nkv, hd, generator=g)
-        q = torch.randn(64, nh, hd, generator=g) * 0.1
+        q = torch.randn(nq, nh, hd, generator=g) * 0.1
         for i, r in enumerate(rows):
             p, d = P0 + r, 3 + 2 * i
             q[r, :, :] = 0.0
@@ -291,13 +293,13 @@ def test_window_edge_inside_a_tile_of_64_queries(hd, bs):
             k_pages[pg, :, p % bs, :] = k[p]
             v_pages[pg, :, :, p % bs] = v[p]
         k_pages, v_pages = k_pages.to(dtype).to(dev), v_pages.to(dtype).to(dev)
-        qd = q.reshape(64, nh * hd).to(dtype).to(dev)
-        pos = torch.arange(P0, P0 + 64, dtype=torch.int32, device=dev)
+        qd = q.reshape(nq, nh * hd).to(dtype).to(dev)
+        pos = torch.arange(P0, P0 + nq, dtype=torch.int32, device=dev)
         item = lambda x: torch.tensor([x], dtype=torch.int32, device=dev)
-        out = torch.zeros(64, nh * hd, dtype=dtype, device=dev)
-        ops.attention_tiles(qd, out, k_pages, v_pages, table, pos, item(0), item(0), item(64), nh, nkv, hd, bs, W,
-                            1.0 / math.sqrt(hd))
-        out = out.double().cpu().reshape(64, nh, hd)
+        out = torch.zeros(nq, nh * hd, dtype=dtype, device=dev)
+        ops.attention_tiles(qd, out, k_pages, v_pages, table, pos, item(0), item(0), item(nq), nh, nkv, hd, bs, W,
+                            1.0 / math.sqrt(hd), tile_q=nq)
+        out = out.double().cpu().reshape(nq, nh, hd)
         # the plain attention over the whole sequence, from the values the pages hold
         qs = torch.zeros(L, nh, hd, dtype=torch.float64)
         qs[P0:] = q.to(dtype).double()
@@ -374,6 +376,32 @@ def test_production_layer_sizes(model_folders, name, dtype):
     routing = {} if dtype == "bfloat16" else None
     got = ru.run_trace(runner, ru.trace_mixed(reqs, seed=5, decode_tail=20), routing)
     check(got, folder, reqs, dtype, f"{name} {dtype} mixed", routing, width)
+
+
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_prompt_portions_in_items_of_128_queries(model_folders, name, monkeypatch):
+    """The attention part takes items of 128 queries only where their blocks fill the GPU; here it is made to take
+    them for every portion that the kernel allows (whole prompts, and portions of changing size beside single
+    tokens), with a window on one layer of E."""
+    from ferrox_amd import ops
+    from ferrox_amd.parts.attention import PagedAttention
+    chosen = []
+
+    def widest(self, ctx, dtype, block_size):
+        chosen.append(64 if ctx.recorded else ops.attention_tile_queries(dtype, self.head_dim, block_size))
+        return chosen[-1]
+
+    monkeypatch.setattr(PagedAttention, "tile_queries", widest)
+    reqs = requests_for(name)
+    folder, runner = runner_for(model_folders, name, "bfloat16", block_size=64, num_pages=24)
+    width = TINY[name][0]["hidden_size"]
+    routing = {}
+    got = ru.run_trace(runner, ru.trace_whole(reqs), routing)
+    check(got, folder, reqs, "bfloat16", f"{name} items of 128, whole", routing, width)
+    routing = {}
+    got = ru.run_trace(runner, ru.trace_mixed(reqs, seed=5, decode_tail=20), routing)
+    check(got, folder, reqs, "bfloat16", f"{name} items of 128, mixed", routing, width)
+    assert 128 in chosen
 
 
 def test_recorded_decode_steps_equal_launched_ones(model_folders):

@@ -521,6 +521,21 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
     out = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
     ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale)
     close(out, ref, dtype, "tiled attention")
+    tq = ops.attention_tile_queries(dtype, hd, bs)
+    assert tq == (128 if dtype == torch.bfloat16 and bs % 64 == 0 and hd in (64, 128) else 64)
+    if tq > 64:       # larger items where the kernel takes them: a wave then holds two blocks of 16 queries
+        t_seq, t_tok, t_n = [], [], []
+        for s, L in enumerate(seq_lens):
+            for t0 in range(0, L, tq):
+                t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(tq, L - t0))
+        wide = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
+        ops.attention_tiles(q_rot, wide, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale,
+                            tile_q=tq)
+        close(wide, ref, dtype, f"tiled attention, items of {tq}")
+    else:
+        with pytest.raises(ops.KernelError):
+            ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window,
+                                scale, tile_q=128)
     # the last token of every sequence as a single query
     out2 = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
     last = [starts[s + 1] - 1 for s in range(len(seq_lens))]
