@@ -92,16 +92,25 @@ class DecodeGraph:
             # no garbage collection while the stream is recording: a tensor of an earlier step that is freed
             # then makes the allocator query events, which a recording stream does not allow
             collecting = gc.isenabled()
-            gc.collect()
             gc.disable()
             if debug.routing_trace is not None:
                 debug.routing_trace.begin_step()     # the recorded launches write where the eager ones just wrote
+            # (capture_begin / capture_end on a stream of its own rather than `with torch.cuda.graph(...)`: that
+            # context manager also gives the allocator's cached memory back to the driver first, which with tens of
+            # GB in the cache costs a recording several hundred milliseconds)
+            main, side = torch.cuda.current_stream(), self.runner.capture_stream
+            side.wait_stream(main)
             try:
-                with torch.cuda.graph(graph):
-                    self.logits = model.forward(self._context(), caches)
+                with torch.cuda.stream(side):
+                    graph.capture_begin()
+                    try:
+                        self.logits = model.forward(self._context(), caches)
+                    finally:
+                        graph.capture_end()
             finally:
                 if collecting:
                     gc.enable()
+            main.wait_stream(side)
             self.graph = graph
             if debug.routing_trace is not None:
                 self.trace_calls = debug.routing_trace.calls()
@@ -128,6 +137,7 @@ class ModelRunner:
         # decode steps are replayed from HIP graphs if every mixer can be recorded
         self.use_graphs = use_graphs and all(b.mixer.graph_safe for b in model.blocks)
         self.graph_kv_step = graph_kv_step
+        self.capture_stream = torch.cuda.Stream(device=self.device) if use_graphs else None     # default priority
         self._graphs: dict = {}
         self._host = None                      # pinned staging buffer of the step's int32 data
         self.before_launch = None              # measurement: called right before a step's first device operation
