@@ -330,6 +330,24 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
 
+// Maximum and sum over the four lanes li, li + 16, li + 32, li + 48 that share a row, in every one of them, with the
+// two lane-swapping moves of gfx950 (rows of 16 lanes pairwise, then the halves of the wave): the same values in the
+// same order as two exchanges through the LDS crossbar (__shfl_xor by 16 and by 32) would give, without the LDS.
+__device__ __forceinline__ float quad_max(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned v = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned v = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // One step of the one-pass softmax on a lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r
 // (key0 = tile start + 16g), in base 2: t = score * c with c = scale * log2(e), m and l are the
 // running maximum (of t) and sum of this lane's row, shared by the row's four lanes.  MASKED: only
@@ -338,21 +356,20 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 template <bool MASKED>
 __device__ __forceinline__ float softmax_step(f32x4_t (&sc)[4], int key0, int lo, int hi, float c, float& m, float& l,
                                               uint4& p_lo, uint4& p_hi) {
+    // the maximum is taken over the raw scores and scaled once (c > 0, and rounding keeps the order); a score's
+    // exponent is then one fused multiply-add, score * c - maximum
     float mt = NEG_INF;
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float v = sc[kb][r] * c;
             if (MASKED) {
                 const int key = key0 + 4 * kb + r;
-                v = (key >= lo && key <= hi) ? v : NEG_INF;
+                sc[kb][r] = (key >= lo && key <= hi) ? sc[kb][r] : NEG_INF;
             }
-            sc[kb][r] = v;
-            mt = fmaxf(mt, v);
+            mt = fmaxf(mt, sc[kb][r]);
         }
-    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    mt = quad_max(mt) * c;
     const float m_new = fmaxf(m, mt);
     const float m_use = (m_new == NEG_INF) ? 0.f : m_new;      // a row that has seen nothing yet
     const float alpha = __builtin_amdgcn_exp2f(m - m_use);      // exp2(-inf) = 0
@@ -362,13 +379,12 @@ __device__ __forceinline__ float softmax_step(f32x4_t (&sc)[4], int key0, int lo
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            p[4 * kb + r] = __builtin_amdgcn_exp2f(sc[kb][r] - m_use);
+            p[4 * kb + r] = __builtin_amdgcn_exp2f(fmaf(sc[kb][r], c, -m_use));
             ps += p[4 * kb + r];
         }
     p_lo = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
     p_hi = make_uint4(pack_bf16(p[8], p[9]), pack_bf16(p[10], p[11]), pack_bf16(p[12], p[13]), pack_bf16(p[14], p[15]));
-    ps += __shfl_xor(ps, 16, 64);
-    ps += __shfl_xor(ps, 32, 64);
+    ps = quad_sum(ps);
     l = l * ((m_new == NEG_INF) ? 1.f : alpha) + ps;
     m = m_new;
     return (m_new == NEG_INF) ? 1.f : alpha;
