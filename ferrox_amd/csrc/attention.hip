@@ -849,14 +849,15 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
 typedef __attribute__((address_space(1))) const void* fx_global_ptr;
 typedef __attribute__((address_space(3))) void* fx_lds_ptr;
 
-// R: blocks of 16 queries per wave (an item is up to 64 R queries).  With two, every operand of keys and of values
-// that a wave reads from LDS serves two products.
-template <int HD, int NS, int R>
-__global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
+// W waves per block, 16 queries each: an item is up to 16 W queries.  Eight waves share every tile that the block
+// brings into LDS between twice as many queries, and four of them per SIMD (two blocks on a CU) hide each other's
+// waits; four waves (items of 64) are for prompt portions too short to fill the GPU with larger items.
+template <int HD, int NS, int W = 4>
+__global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArgs a) {
     constexpr int KS = HD / 32, CB = HD / 16;
     constexpr int NCH = HD / 8;                 // 16-byte chunks of a key row
     constexpr int KROWS = 1024 / (2 * HD);      // key rows of a wave-load
-    constexpr int NLOAD = HD / 32;              // wave-loads per wave for the keys of a tile, and as many for the values
+    constexpr int NLOAD = HD / (8 * W);         // wave-loads per wave for the keys of a tile, and as many for the values
     constexpr int TILE = 2 * 64 * HD;           // elements of a stage: keys, then values
     static_assert(NS == 2 || NS == 3, "two or three stages");
     __shared__ __attribute__((aligned(1024))) bf16 tiles[NS * TILE];
@@ -877,42 +878,34 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
     const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
     const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
     const int kv_end = pmax + 1;
-    // this wave's queries: 16 R consecutive ones, block r of them at tok0 + 16 r
-    const int tok0 = tok_first + 16 * R * wave, n = max(0, min(16 * R, n_all - 16 * R * wave));
-    int lo[R], hi[R];
+    const int tok0 = tok_first + 16 * wave, n = min(16, n_all - 16 * wave);
+    int lo = 1, hi = 0;
+    const bf16* qrow = nullptr;
+    if (li < n) {
+        hi = a.positions[tok0 + li];
+        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * HD;
+    }
     int w_lo = 0x7fffffff, w_hi = -1;
     int w_lo_max = 0x7fffffff, w_hi_min = -1;
     if (n > 0) {
         w_hi = a.positions[tok0 + n - 1];
         w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
-        if (n == 16 * R) {
+        if (n == 16) {
             w_hi_min = a.positions[tok0];
             w_lo_max = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
         }
     }
     const float c2 = a.scale * LOG2E;
-    float m[R], l[R];
-    f32x4_t o[R][CB];
-    bf16x8_t qf[R][KS];
+    float m = NEG_INF, l = 0.f;
+    f32x4_t o[CB];
+    bf16x8_t qf[KS];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        lo[r] = 1;
-        hi[r] = 0;
-        m[r] = NEG_INF;
-        l[r] = 0.f;
-        const bf16* qrow = nullptr;
-        if (16 * r + li < n) {
-            hi[r] = a.positions[tok0 + 16 * r + li];
-            lo[r] = a.window > 0 ? max(0, hi[r] - a.window + 1) : 0;
-            qrow = (const bf16*)a.q + (size_t)(tok0 + 16 * r + li) * a.ldq + (size_t)h * HD;
-        }
+    for (int cb = 0; cb < CB; ++cb) o[cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) o[r][cb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int u = 0; u < KS; ++u) {
-            const uint4 v = qrow ? *(const uint4*)(qrow + 32 * u + 8 * g) : make_uint4(0, 0, 0, 0);
-            qf[r][u] = __builtin_bit_cast(bf16x8_t, v);
-        }
+    for (int u = 0; u < KS; ++u) {
+        const uint4 v = qrow ? *(const uint4*)(qrow + 32 * u + 8 * g) : make_uint4(0, 0, 0, 0);
+        qf[u] = __builtin_bit_cast(bf16x8_t, v);
     }
     int first_blk, last_blk, unused;
     page_slot(a, kv_begin, first_blk, unused);
@@ -923,7 +916,7 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
     int k_src[NLOAD], v_src[NLOAD];
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
-        const int j = wave + 4 * i;                          // wave-load j of HD / 8
+        const int j = wave + W * i;                          // wave-load j of HD / 8
         const int row = KROWS * j + lane / NCH;              // LDS key row 16 kb + 4 a + b
         const int key = 16 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
         k_src[i] = key * HD + (((lane % NCH) ^ (NCH == 16 ? (row & 15) : ((row >> 1) & 7))) * 8);
@@ -939,11 +932,11 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
         bf16* st = tiles + stage * TILE;
 #pragma unroll
         for (int i = 0; i < NLOAD; ++i)
-            __builtin_amdgcn_global_load_lds((fx_global_ptr)(kbase + k_src[i]), (fx_lds_ptr)(st + (wave + 4 * i) * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(kbase + k_src[i]), (fx_lds_ptr)(st + (wave + W * i) * 512), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < NLOAD; ++i)
             __builtin_amdgcn_global_load_lds((fx_global_ptr)(vbase + v_src[i]),
-                                             (fx_lds_ptr)(st + 64 * HD + (wave + 4 * i) * 512), 16, 0, 0);
+                                             (fx_lds_ptr)(st + 64 * HD + (wave + W * i) * 512), 16, 0, 0);
     };
     // operands: key row 16 kb + li, chunk 4 u + g; value row 16 cb + li, chunks 2 g and 2 g + 1
     const int k_at = li * HD, v_at = 64 * HD + li * 64;
@@ -961,7 +954,7 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
         if (kt0 + 64 * (NS - 1) < kv_end) issue(kt0 + 64 * (NS - 1), (stage + NS - 1) % NS);
         bf16* st = tiles + stage * TILE;
         if (kt0 < kv_begin || kt0 + 64 > kv_end) {              // a tile at the edge: values of keys outside become zeros
-            for (int idx = tid; idx < HD * 64; idx += 256) {
+            for (int idx = tid; idx < HD * 64; idx += W * 64) {
                 const int d = idx >> 6, key = idx & 63;
                 if (kt0 + key < kv_begin || kt0 + key >= kv_end)
                     st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
@@ -969,54 +962,43 @@ __global__ __launch_bounds__(256, 2) void attn_mfma_direct_kernel(AttnArgs a) {
             lds_barrier();      // the zeros are in LDS (a bare s_barrier does not wait for this wave's stores) before any wave reads values
         }
         if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;           // nothing in this tile for this wave's rows
-        f32x4_t sc[R][4];
+        f32x4_t sc[4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) sc[r][kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
                 const bf16x8_t kf = *(const bf16x8_t*)(st + k_at + kb * 16 * HD + (((4 * u + g) ^ ksw) * 8));
-#pragma unroll
-                for (int r = 0; r < R; ++r) sc[r][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[r][u], sc[r][kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u], sc[kb], 0, 0, 0);
             }
         }
         const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
-        uint4 p_lo[R], p_hi[R];
-        bool rescale[R];
-        float al[R][4];
+        uint4 p_lo, p_hi;
+        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi);
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+        float al[4] = {1.f, 1.f, 1.f, 1.f};
+        if (rescale) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const float alpha = whole ? softmax_step<false>(sc[r], kt0 + 16 * g, lo[r], hi[r], c2, m[r], l[r], p_lo[r], p_hi[r])
-                                      : softmax_step<true>(sc[r], kt0 + 16 * g, lo[r], hi[r], c2, m[r], l[r], p_lo[r], p_hi[r]);
-            rescale[r] = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) al[r][j] = 1.f;
-            if (rescale[r]) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) al[r][j] = __shfl(alpha, 4 * g + j, 64);
-            }
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             const bf16* vr = st + v_at + cb * 16 * 64;
-            const uint4 v0 = *(const uint4*)(vr + (((2 * g) ^ vsw) * 8)), v1 = *(const uint4*)(vr + (((2 * g + 1) ^ vsw) * 8));
-#pragma unroll
-            for (int r = 0; r < R; ++r) o[r][cb] = pv_step(o[r][cb], rescale[r], al[r], p_lo[r], p_hi[r], v0, v1);
+            o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, *(const uint4*)(vr + (((2 * g) ^ vsw) * 8)),
+                            *(const uint4*)(vr + (((2 * g + 1) ^ vsw) * 8)));
         }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        const float lr = __shfl(l, row, 64);
+        if (row < n) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = 16 * r + 4 * g + j;
-            const float lr = __shfl(l[r], 4 * g + j, 64);
-            if (row < n) {
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb)
-                    from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * HD + 16 * cb + li, o[r][cb][j] / lr);
-            }
+            for (int cb = 0; cb < CB; ++cb)
+                from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * HD + 16 * cb + li, o[cb][r] / lr);
         }
+    }
 }
 
 // Switch for tests and measurement (ferrox_amd/debug.py is its one caller); the product path never sets it.
@@ -1070,11 +1052,11 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
-        if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 2><<<grid_blocks, 256, 0, s>>>(a);
-        else if (tile_q == 128) attn_mfma_direct_kernel<64, 2, 2><<<grid_blocks, 256, 0, s>>>(a);
-        else if (bs % 64 == 0 && hd == 128 && g_direct == 3) attn_mfma_direct_kernel<128, 3, 1><<<grid_blocks, 256, 0, s>>>(a);
-        else if (bs % 64 == 0 && hd == 128 && g_direct) attn_mfma_direct_kernel<128, 2, 1><<<grid_blocks, 256, 0, s>>>(a);
-        else if (bs % 64 == 0 && hd == 64 && g_direct) attn_mfma_direct_kernel<64, 2, 1><<<grid_blocks, 256, 0, s>>>(a);
+        if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
+        else if (tile_q == 128) attn_mfma_direct_kernel<64, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 128 && g_direct == 3) attn_mfma_direct_kernel<128, 3><<<grid_blocks, 256, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 128 && g_direct) attn_mfma_direct_kernel<128, 2><<<grid_blocks, 256, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 64 && g_direct) attn_mfma_direct_kernel<64, 2><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 64) attn_mfma_block_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 128) attn_mfma_block_kernel<128><<<grid_blocks, 256, 0, s>>>(a);

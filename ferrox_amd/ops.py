@@ -377,7 +377,7 @@ def can_fuse_norm(h: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:
 
 def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
     """The most consecutive queries of a sequence that one item of attention_tiles may cover at these sizes: 64,
-    or 128 where the kernel gives a wave two blocks of 16 queries (every operand it reads then serves two products)."""
+    or 128 where the kernel has a block of eight waves for them."""
     f, _ = _fn("attention", "fx_attn_tile_queries")
     return int(f(dtype_code(dtype), int(head_dim), int(block_size)))
 

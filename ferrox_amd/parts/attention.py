@@ -114,10 +114,11 @@ class PagedAttention(Mixer):
         return act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0
 
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
-        """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many and the
-        blocks still fill the GPU's 512 places for them.  Blocks of a portion that starts a prompt differ in work up
-        to the portion's length in keys, so they count by their mean share of the longest (measured at 16 and 28
-        heads of 128: items of 128 gain 8-25 % from 448 such blocks on and lose 10-35 % at 256 and below)."""
+        """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many (a block
+        of eight waves then shares every tile of keys it brings in between twice as many queries) and the blocks
+        still number about one per CU.  Blocks of a portion that starts a prompt differ in work up to the portion's
+        length in keys, so they count by their mean share of the longest (measured at 16 and 28 heads of 128:
+        items of 128 gain up to 26 % from 448 such blocks on, are even at 256 and lose 8-13 % at 128)."""
         if ctx.recorded:
             return 64
         widest = ops.attention_tile_queries(dtype, self.head_dim, block_size)
@@ -129,7 +130,7 @@ class PagedAttention(Mixer):
             if n > 1:
                 before = ctx.kv_lens[s] - n
                 even_blocks += -(-n // widest) * self.n_heads * (before + n / 2) / (before + n)
-        return widest if even_blocks >= 400 else 64
+        return widest if even_blocks >= 250 else 64
 
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         table = ctx.block_tables[cache.group]

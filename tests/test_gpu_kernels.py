@@ -523,7 +523,7 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
     close(out, ref, dtype, "tiled attention")
     tq = ops.attention_tile_queries(dtype, hd, bs)
     assert tq == (128 if dtype == torch.bfloat16 and bs % 64 == 0 and hd in (64, 128) else 64)
-    if tq > 64:       # larger items where the kernel takes them: a wave then holds two blocks of 16 queries
+    if tq > 64:       # larger items where the kernel takes them: blocks of eight waves
         t_seq, t_tok, t_n = [], [], []
         for s, L in enumerate(seq_lens):
             for t0 in range(0, L, tq):
