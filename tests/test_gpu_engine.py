@@ -404,6 +404,26 @@ def test_prompt_portions_in_items_of_128_queries(model_folders, name, monkeypatc
     assert 128 in chosen
 
 
+def test_how_many_queries_an_item_of_a_prompt_portion_takes(model_folders):
+    """The attention part's choice between items of 64 and of 128 queries: by the number of evenly loaded blocks that
+    the step's portions give (a portion that starts a prompt counts half), never for recorded steps, and 64 where
+    the kernel has no larger items (float32, small heads)."""
+    from types import SimpleNamespace as NS
+    folder, runner = runner_for(model_folders, "D", "bfloat16", block_size=64, num_pages=24)
+    att = runner.model.blocks[0].mixer                       # 16 heads of 128
+    ask = lambda portions, recorded=False, dtype=torch.bfloat16, bs=64: att.tile_queries(
+        NS(recorded=recorded, n_seqs=len(portions), q_starts=[sum(n for n, _ in portions[:i]) for i in range(len(portions) + 1)],
+           kv_lens=[before + n for n, before in portions]), dtype, bs)
+    assert ask([(2048, 0)]) == 64                            # 16 x 16 blocks, half-loaded on average: 128
+    assert ask([(4096, 0)]) == 128                           # 32 x 16 x 0.5 = 256
+    assert ask([(2048, 22528)]) == 64                        # 16 x 16 x 0.96 = 245
+    assert ask([(2048, 22528), (512, 4096)]) == 128          # + 4 x 16 x 0.94
+    assert ask([(1, 500)] * 8) == 64                         # single tokens are no portions
+    assert ask([(4096, 0)], recorded=True) == 64
+    assert ask([(4096, 0)], dtype=torch.float32) == 64
+    assert ask([(4096, 0)], bs=16) == 64
+
+
 def test_recorded_decode_steps_equal_launched_ones(model_folders):
     """bfloat16 decode steps replayed from a HIP graph, several times with other work between the
     replays, against the same steps launched kernel by kernel (the bound on the sequence length
