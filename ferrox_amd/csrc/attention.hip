@@ -852,15 +852,20 @@ typedef __attribute__((address_space(3))) void* fx_lds_ptr;
 // W waves per block, 16 queries each: an item is up to 16 W queries.  Eight waves share every tile that the block
 // brings into LDS between twice as many queries, and four of them per SIMD (two blocks on a CU) hide each other's
 // waits; four waves (items of 64) are for prompt portions too short to fill the GPU with larger items.
-template <int HD, int NS, int W = 4>
-__global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArgs a) {
+// G = 2: two such groups of W waves share the item's queries and take its tiles of keys in turn (group 0 the even
+// ones, group 1 the odd ones), each with stages, running maxima, sums and outputs of its own; group 1 hands its
+// results over through LDS at the end and group 0 merges them.  An item's chain of tiles is then half as long,
+// which is what bounds a prompt portion of few items over many keys.
+template <int HD, int NS, int W = 4, int G = 1>
+__global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(AttnArgs a) {      // two blocks on a CU, or one of two groups
+    static_assert(G == 1 || (G == 2 && NS == 2), "one group, or two with two stages each");
     constexpr int KS = HD / 32, CB = HD / 16;
     constexpr int NCH = HD / 8;                 // 16-byte chunks of a key row
     constexpr int KROWS = 1024 / (2 * HD);      // key rows of a wave-load
     constexpr int NLOAD = HD / (8 * W);         // wave-loads per wave for the keys of a tile, and as many for the values
     constexpr int TILE = 2 * 64 * HD;           // elements of a stage: keys, then values
     static_assert(NS == 2 || NS == 3, "two or three stages");
-    __shared__ __attribute__((aligned(1024))) bf16 tiles[NS * TILE];
+    __shared__ __attribute__((aligned(1024))) bf16 tiles[G * NS * TILE];
     __shared__ int page_copy[PAGE_COPY];
     const int per_xcd = (a.n_items * a.nh + 7) / 8;
     const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
@@ -869,7 +874,8 @@ __global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArg
     // the blocks that come to share a CU (two fit, handed out in turn) have about the same work together
     const int h = logical / a.n_items;
     const int item = (h & 1) ? logical % a.n_items : a.n_items - 1 - logical % a.n_items;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = G == 1 ? (int)threadIdx.x : (int)threadIdx.x % (W * 64), lane = tid & 63, wave = tid >> 6;      // within the group
+    const int grp = G == 1 ? 0 : (int)threadIdx.x / (W * 64);
     const int li = lane & 15, g = lane >> 4;
     const int kvh = h / (a.nh / a.nkv);
     const int tok_first = a.item_tok[item], n_all = a.item_n[item];
@@ -929,7 +935,7 @@ __global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArg
         const size_t page = (size_t)__builtin_amdgcn_readfirstlane(pl.page(blk));
         const bf16* kbase = (const bf16*)a.k_pages + ((page * a.nkv + kvh) * bs + slot) * HD;
         const bf16* vbase = (const bf16*)a.v_pages + (page * a.nkv + kvh) * HD * bs + slot;
-        bf16* st = tiles + stage * TILE;
+        bf16* st = tiles + (grp * NS + stage) * TILE;
 #pragma unroll
         for (int i = 0; i < NLOAD; ++i)
             __builtin_amdgcn_global_load_lds((fx_global_ptr)(kbase + k_src[i]), (fx_lds_ptr)(st + (wave + W * i) * 512), 16, 0, 0);
@@ -942,26 +948,39 @@ __global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArg
     const int k_at = li * HD, v_at = 64 * HD + li * 64;
     const int ksw = NCH == 16 ? li : (li >> 1) & 7, vsw = (li >> 1) & 7;
 
+    // Every wave of the block goes through the same barriers: the loop runs over rounds of G tiles, of which group
+    // grp takes tile grp (a round's last tiles may not exist: that group then only keeps step).
     const int kt_first = (kv_begin / 64) * 64;
-    issue(kt_first, 0);
+    if (kt_first + 64 * grp < kv_end) issue(kt_first + 64 * grp, 0);
     if (NS == 3 && kt_first + 64 < kv_end) issue(kt_first + 64, 1);
     int stage = 0;
-    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, stage = (stage + 1 == NS ? 0 : stage + 1)) {
+    for (int round0 = kt_first; round0 < kv_end; round0 += 64 * G, stage = (stage + 1 == NS ? 0 : stage + 1)) {
+        const int kt0 = round0 + 64 * grp;
         // this wave's part of the tile has landed (with three stages the next tile's loads may still fly)
         if (NS == 3 && kt0 + 64 < kv_end) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLOAD) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();                           // ... everyone's has, and the stage read last is free
-        if (kt0 + 64 * (NS - 1) < kv_end) issue(kt0 + 64 * (NS - 1), (stage + NS - 1) % NS);
-        bf16* st = tiles + stage * TILE;
-        if (kt0 < kv_begin || kt0 + 64 > kv_end) {              // a tile at the edge: values of keys outside become zeros
-            for (int idx = tid; idx < HD * 64; idx += W * 64) {
-                const int d = idx >> 6, key = idx & 63;
-                if (kt0 + key < kv_begin || kt0 + key >= kv_end)
-                    st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
+        if (kt0 + 64 * G * (NS - 1) < kv_end) issue(kt0 + 64 * G * (NS - 1), (stage + NS - 1) % NS);
+        bf16* st = tiles + (grp * NS + stage) * TILE;
+        // a tile at the edge: values of keys outside become zeros.  Whether any tile of the round is one is the
+        // same for all waves, so all of them meet at the barrier behind the zeros.
+        bool any_edge = false;
+#pragma unroll
+        for (int q = 0; q < G; ++q) {
+            const int kq = round0 + 64 * q;
+            any_edge = any_edge || (kq < kv_end && (kq < kv_begin || kq + 64 > kv_end));
+        }
+        if (any_edge) {
+            if (kt0 < kv_end && (kt0 < kv_begin || kt0 + 64 > kv_end)) {
+                for (int idx = tid; idx < HD * 64; idx += W * 64) {
+                    const int d = idx >> 6, key = idx & 63;
+                    if (kt0 + key < kv_begin || kt0 + key >= kv_end)
+                        st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
+                }
             }
             lds_barrier();      // the zeros are in LDS (a bare s_barrier does not wait for this wave's stores) before any wave reads values
         }
-        if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;           // nothing in this tile for this wave's rows
+        if (kt0 >= kv_end || kt0 > w_hi || kt0 + 64 <= w_lo) continue;      // no such tile, or nothing in it for this wave's rows
         f32x4_t sc[4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
@@ -989,6 +1008,31 @@ __global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArg
                             *(const uint4*)(vr + (((2 * g + 1) ^ vsw) * 8)));
         }
     }
+    if constexpr (G == 2) {
+        // group 1 hands over maximum, sum and outputs, lane for lane, through the LDS that the tiles no longer need
+        __syncthreads();
+        float* hand = (float*)tiles + (size_t)wave * ((2 + 4 * CB) * 64);
+        if (grp == 1) {
+            hand[lane] = m;
+            hand[64 + lane] = l;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) hand[(2 + 4 * cb + r) * 64 + lane] = o[cb][r];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = hand[lane], l1 = hand[64 + lane];
+        const float mn = fmaxf(m, m1), mu = (mn == NEG_INF) ? 0.f : mn;
+        const float f0 = __builtin_amdgcn_exp2f(m - mu), f1 = __builtin_amdgcn_exp2f(m1 - mu);
+        l = l * f0 + l1 * f1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float a0 = __shfl(f0, 4 * g + r, 64), a1 = __shfl(f1, 4 * g + r, 64);      // of the accumulator's row 4 g + r
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) o[cb][r] = o[cb][r] * a0 + hand[(2 + 4 * cb + r) * 64 + lane] * a1;
+        }
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
@@ -1003,9 +1047,11 @@ __global__ __launch_bounds__(W * 64, W / 2) void attn_mfma_direct_kernel(AttnArg
 
 // Switch for tests and measurement (ferrox_amd/debug.py is its one caller); the product path never sets it.
 static int g_direct = 2;     // "direct_stages": 0 keeps prefill on the kernel that stages tiles through registers; 2 (default), 3: stages
+static int g_groups = 0;     // "direct_groups": 1 or 2 groups of waves per block of 64 queries in that kernel (0: by the number of blocks)
 FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "direct_stages")) { g_direct = value; return 0; }
-    FX_REQUIRE(false, "attention: no debug switch '%s' (direct_stages)", key);
+    if (!strcmp(key, "direct_groups")) { g_groups = value; return 0; }
+    FX_REQUIRE(false, "attention: no debug switch '%s' (direct_stages, direct_groups)", key);
     return 1;
 }
 
@@ -1049,11 +1095,17 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.n_items = n_items;
     dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
     hipStream_t s = (hipStream_t)stream;
+    // no more blocks than CUs: a block's chain of tiles is what takes the time, and two groups of waves halve it
+    // (measured: 512-token portions at depth 8k-24k 130 and 360 us against 214 and 616 us; from 448 blocks on, one
+    // group and two blocks to a CU are as fast or faster)
+    const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= 256;
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
         if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
         else if (tile_q == 128) attn_mfma_direct_kernel<64, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 128 && g_direct == 2 && two_groups) attn_mfma_direct_kernel<128, 2, 4, 2><<<grid_blocks, 512, 0, s>>>(a);
+        else if (bs % 64 == 0 && hd == 64 && g_direct == 2 && two_groups) attn_mfma_direct_kernel<64, 2, 4, 2><<<grid_blocks, 512, 0, s>>>(a);
         else if (bs % 64 == 0 && hd == 128 && g_direct == 3) attn_mfma_direct_kernel<128, 3><<<grid_blocks, 256, 0, s>>>(a);
         else if (bs % 64 == 0 && hd == 128 && g_direct) attn_mfma_direct_kernel<128, 2><<<grid_blocks, 256, 0, s>>>(a);
         else if (bs % 64 == 0 && hd == 64 && g_direct) attn_mfma_direct_kernel<64, 2><<<grid_blocks, 256, 0, s>>>(a);

@@ -256,15 +256,16 @@ def test_far_key_and_window_edge_stand_out(model_folders):
                     assert float((out[2] - hidden).abs().max()) < tol
 
 
-@pytest.mark.parametrize("hd,bs,nq", [(64, 64, 64), (128, 64, 64), (32, 16, 64), (64, 64, 128), (128, 64, 128)])
-def test_window_edge_inside_a_tile_of_64_queries(hd, bs, nq):
+@pytest.mark.parametrize("hd,bs,nq,groups", [(64, 64, 64, 1), (128, 64, 64, 1), (64, 64, 64, 2), (128, 64, 64, 2), (32, 16, 64, 0),
+                                             (64, 64, 128, 0), (128, 64, 128, 0)])
+def test_window_edge_inside_a_tile_of_64_queries(hd, bs, nq, groups):
     """A full tile of 64 queries, or one item of 128 where the kernel takes them (the prefill kernels' fast path
     without per-element masks, and the per-row window edge inside a tile): for several rows the key at distance W-1 stands out and must be found, the key
     at distance W stands out and must stay hidden.  For row 16 the edge falls between two tiles of 64 keys,
-    which is also a page's edge."""
+    which is also a page's edge.  `groups`: one or two groups of waves per block, where the kernel has them."""
     import math
     import plain_qwen2moe as plain
-    from ferrox_amd import ops
+    from ferrox_amd import debug, ops
     dev, W, P0, nh, nkv = "cuda:0", 100, 275, 2, 2
     L = P0 + nq
     rows = [0, 5, 16, 31, 47, 63] + ([64, 70, 80, 111, 127] if nq == 128 else [])
@@ -297,8 +298,9 @@ def test_window_edge_inside_a_tile_of_64_queries(hd, bs, nq):
         pos = torch.arange(P0, P0 + nq, dtype=torch.int32, device=dev)
         item = lambda x: torch.tensor([x], dtype=torch.int32, device=dev)
         out = torch.zeros(nq, nh * hd, dtype=dtype, device=dev)
-        ops.attention_tiles(qd, out, k_pages, v_pages, table, pos, item(0), item(0), item(nq), nh, nkv, hd, bs, W,
-                            1.0 / math.sqrt(hd), tile_q=nq)
+        with debug.kernel_switch("attention", "direct_groups", groups):
+            ops.attention_tiles(qd, out, k_pages, v_pages, table, pos, item(0), item(0), item(nq), nh, nkv, hd, bs, W,
+                                1.0 / math.sqrt(hd), tile_q=nq)
         out = out.double().cpu().reshape(nq, nh, hd)
         # the plain attention over the whole sequence, from the values the pages hold
         qs = torch.zeros(L, nh, hd, dtype=torch.float64)

@@ -518,9 +518,12 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
         for t0 in range(0, L, 64):
             t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(64, L - t0))
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
-    out = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
-    ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale)
-    close(out, ref, dtype, "tiled attention")
+    from ferrox_amd import debug
+    for groups in (1, 2):      # of waves per block of the kernel for pages of 64 keys (it takes two where blocks are few)
+        out = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
+        with debug.kernel_switch("attention", "direct_groups", groups):
+            ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale)
+        close(out, ref, dtype, f"tiled attention, {groups} group(s) of waves")
     tq = ops.attention_tile_queries(dtype, hd, bs)
     assert tq == (128 if dtype == torch.bfloat16 and bs % 64 == 0 and hd in (64, 128) else 64)
     if tq > 64:       # larger items where the kernel takes them: blocks of eight waves
