@@ -1102,7 +1102,9 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
-        if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
+        if (tile_q == 128 && hd == 128 && two_groups) attn_mfma_direct_kernel<128, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
+        else if (tile_q == 128 && hd == 64 && two_groups) attn_mfma_direct_kernel<64, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
+        else if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
         else if (tile_q == 128) attn_mfma_direct_kernel<64, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
         else if (bs % 64 == 0 && hd == 128 && g_direct == 2 && two_groups) attn_mfma_direct_kernel<128, 2, 4, 2><<<grid_blocks, 512, 0, s>>>(a);
         else if (bs % 64 == 0 && hd == 64 && g_direct == 2 && two_groups) attn_mfma_direct_kernel<64, 2, 4, 2><<<grid_blocks, 512, 0, s>>>(a);

@@ -115,22 +115,29 @@ class PagedAttention(Mixer):
 
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
         """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many (a block
-        of eight waves then shares every tile of keys it brings in between twice as many queries) and the blocks
-        still number about one per CU.  Blocks of a portion that starts a prompt differ in work up to the portion's
-        length in keys, so they count by their mean share of the longest (measured at 16 and 28 heads of 128:
-        items of 128 gain up to 26 % from 448 such blocks on, are even at 256 and lose 8-13 % at 128)."""
+        of eight waves then shares every tile of keys it brings in between twice as many queries).  The kernel gives
+        a launch of no more blocks than the 256 CUs two groups of waves per block, which halves a block's chain of
+        tiles; so: items of 64 while they number no more than the CUs; else items of 128 if those do (a 2,048-token
+        portion deep in a prompt: 603 against 784 us at 16 heads); else items of 128 if they still number about
+        one evenly loaded block per CU (blocks of a portion that starts a prompt differ in work up to the portion's
+        length in keys and count by their mean share of the longest; +8-26 % from 448 such blocks on); else 64."""
         if ctx.recorded:
             return 64
         widest = ops.attention_tile_queries(dtype, self.head_dim, block_size)
         if widest == 64:
             return 64
+        small = large = 0
         even_blocks = 0.0
         for s in range(ctx.n_seqs):
             n = ctx.q_starts[s + 1] - ctx.q_starts[s]
             if n > 1:
                 before = ctx.kv_lens[s] - n
+                small += -(-n // 64) * self.n_heads
+                large += -(-n // widest) * self.n_heads
                 even_blocks += -(-n // widest) * self.n_heads * (before + n / 2) / (before + n)
-        return widest if even_blocks >= 250 else 64
+        if small <= 256:
+            return 64
+        return widest if large <= 256 or even_blocks >= 250 else 64
 
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         table = ctx.block_tables[cache.group]

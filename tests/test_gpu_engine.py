@@ -257,7 +257,7 @@ def test_far_key_and_window_edge_stand_out(model_folders):
 
 
 @pytest.mark.parametrize("hd,bs,nq,groups", [(64, 64, 64, 1), (128, 64, 64, 1), (64, 64, 64, 2), (128, 64, 64, 2), (32, 16, 64, 0),
-                                             (64, 64, 128, 0), (128, 64, 128, 0)])
+                                             (64, 64, 128, 1), (128, 64, 128, 1), (64, 64, 128, 2), (128, 64, 128, 2)])
 def test_window_edge_inside_a_tile_of_64_queries(hd, bs, nq, groups):
     """A full tile of 64 queries, or one item of 128 where the kernel takes them (the prefill kernels' fast path
     without per-element masks, and the per-row window edge inside a tile): for several rows the key at distance W-1 stands out and must be found, the key
@@ -407,19 +407,21 @@ def test_prompt_portions_in_items_of_128_queries(model_folders, name, monkeypatc
 
 
 def test_how_many_queries_an_item_of_a_prompt_portion_takes(model_folders):
-    """The attention part's choice between items of 64 and of 128 queries: by the number of evenly loaded blocks that
-    the step's portions give (a portion that starts a prompt counts half), never for recorded steps, and 64 where
-    the kernel has no larger items (float32, small heads)."""
+    """The attention part's choice between items of 64 and of 128 queries: by the number of blocks that the step's
+    portions give, against the CUs and evenly loaded (a portion that starts a prompt counts half); never for
+    recorded steps, and 64 where the kernel has no larger items (float32, small heads)."""
     from types import SimpleNamespace as NS
     folder, runner = runner_for(model_folders, "D", "bfloat16", block_size=64, num_pages=24)
     att = runner.model.blocks[0].mixer                       # 16 heads of 128
     ask = lambda portions, recorded=False, dtype=torch.bfloat16, bs=64: att.tile_queries(
         NS(recorded=recorded, n_seqs=len(portions), q_starts=[sum(n for n, _ in portions[:i]) for i in range(len(portions) + 1)],
            kv_lens=[before + n for n, before in portions]), dtype, bs)
-    assert ask([(2048, 0)]) == 64                            # 16 x 16 blocks, half-loaded on average: 128
+    assert ask([(1024, 0)]) == 64                            # 256 items of 64: two groups of waves each
+    assert ask([(2048, 0)]) == 128                           # 512 items of 64, 256 of 128: those get the two groups
+    assert ask([(2048, 22528)]) == 128
+    assert ask([(3072, 0)]) == 64                            # 384 items of 128, half-loaded on average: 192
     assert ask([(4096, 0)]) == 128                           # 32 x 16 x 0.5 = 256
-    assert ask([(2048, 22528)]) == 64                        # 16 x 16 x 0.96 = 245
-    assert ask([(2048, 22528), (512, 4096)]) == 128          # + 4 x 16 x 0.94
+    assert ask([(2048, 22528), (1024, 4096)]) == 128         # 384 items of 128, evenly loaded
     assert ask([(1, 500)] * 8) == 64                         # single tokens are no portions
     assert ask([(4096, 0)], recorded=True) == 64
     assert ask([(4096, 0)], dtype=torch.float32) == 64

@@ -531,10 +531,12 @@ def test_attention_kernels(dtype, nh, nkv, hd, bs, window):
         for s, L in enumerate(seq_lens):
             for t0 in range(0, L, tq):
                 t_seq.append(s); t_tok.append(starts[s] + t0); t_n.append(min(tq, L - t0))
-        wide = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
-        ops.attention_tiles(q_rot, wide, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window, scale,
-                            tile_q=tq)
-        close(wide, ref, dtype, f"tiled attention, items of {tq}")
+        for groups in (1, 2):
+            wide = torch.zeros(T, nh * hd, dtype=dtype, device=DEV)
+            with debug.kernel_switch("attention", "direct_groups", groups):
+                ops.attention_tiles(q_rot, wide, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window,
+                                    scale, tile_q=tq)
+            close(wide, ref, dtype, f"tiled attention, items of {tq}, {groups} group(s) of waves")
     else:
         with pytest.raises(ops.KernelError):
             ops.attention_tiles(q_rot, out, k_pages, v_pages, table, pos, i32(t_seq), i32(t_tok), i32(t_n), nh, nkv, hd, bs, window,
