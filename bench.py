@@ -154,14 +154,36 @@ class Bench:
         torch.cuda.synchronize()
         log(f"batch {batch}: prompts of {ctx} tokens prefilled in {time.time() - t0:.1f} s")
 
-        def one_step(toks):
+        pairs = [(i, i) for i in range(batch)]
+        read = []                                  # every id that came back to the host, step by step
+
+        def launch(known, on_device):
+            """One decode step of all requests, launched: its tokens are `known`, or the ids `on_device` that the
+            step before it sampled.  Returns (ids on the device, their copy in pinned memory, event after it)."""
             for rid in ids:
                 assert self.runner.reserve(rid, 1)
-            lg = self.runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)])
-            return ops.sample(lg).tolist()          # greedy, on the device; ids come back to the host
+            if on_device is None:
+                lg = self.runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, known)])
+            else:
+                lg = self.runner.step([StepEntry(rid, [0], [0]) for rid in ids], feed=(on_device, pairs))
+            out = ops.sample(lg)                   # greedy, on the device
+            host = torch.empty(batch, dtype=torch.int32, pin_memory=True)
+            host.copy_(out, non_blocking=True)
+            copied = torch.cuda.Event()
+            copied.record()
+            return out, host, copied
 
+        def collect(step):
+            step[2].synchronize()
+            read.append(step[1].tolist())
+
+        # as the engine generates: the host is one step ahead; a step is launched with the ids of the step before
+        # it still on the device, and those ids are read while it runs
+        flying = launch(cur, None)
         for _ in range(warmup):
-            cur = one_step(cur)
+            nxt = launch(None, flying[0])
+            collect(flying)
+            flying = nxt
         parts = max(1, min(parts, steps))
         sizes = [steps // parts + (1 if i < steps % parts else 0) for i in range(parts)]
         per_part = []
@@ -170,13 +192,17 @@ class Bench:
         for n in sizes:                            # exactly `steps` steps between the two synchronisations
             t0 = time.perf_counter()
             for _ in range(n):
-                cur = one_step(cur)                # (reading the ids back waits for the step)
+                nxt = launch(None, flying[0])
+                collect(flying)                    # (waits for the step before the one just launched)
+                flying = nxt
             per_part.append((time.perf_counter() - t0) / n)
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t_all) / steps
+        collect(flying)
+        assert all(0 <= t < self.cfg.vocab_size for row in read for t in row) and len(read) == warmup + steps + 1
         # one more, untimed, step that records which experts the router chose
         with debug.trace_routing() as trace:
-            one_step(cur)
+            collect(launch(read[-1], None))
             per_layer = [len({e for tok in layer for e in tok}) for layer in trace.read()]
         distinct = sum(per_layer) / max(1, len(per_layer))
         for rid in ids:

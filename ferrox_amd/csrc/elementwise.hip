@@ -461,3 +461,21 @@ FX_API int fx_fill_u32(void* stream, void* p, unsigned v, long n) {
     FX_CHECK_LAUNCH("fill");
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// token ids that are still on the device: tokens[pairs[i][0]] = ids[pairs[i][1]].
+// A step whose tokens were sampled by the step before it can be launched before the
+// host has read those ids; where it holds one of them, the host wrote a stand-in.
+// ---------------------------------------------------------------------------
+__global__ void feed_tokens_kernel(int* tokens, const int* ids, const int* pairs, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) tokens[pairs[2 * i]] = ids[pairs[2 * i + 1]];
+}
+
+FX_API int fx_feed_tokens(void* stream, int* tokens, const int* ids, const int* pairs, int n) {
+    FX_REQUIRE(n >= 0 && tokens && ids && pairs, "feed_tokens: bad arguments");
+    if (n == 0) return 0;
+    feed_tokens_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(tokens, ids, pairs, n);
+    FX_CHECK_LAUNCH("feed_tokens");
+    return 0;
+}

@@ -7,7 +7,9 @@
 Generation follows the reference's loop (ferrox-cli/src/run.rs:651-676,
 ferrox-server/src/batch_scheduler.rs:158-243): prefill, then sample -> append ->
 forward until EOS, the token limit or the context limit; here all requests share
-one continuously batched step.
+one continuously batched step.  The host runs one step ahead of the GPU: a step is
+launched with the tokens that the step before it sampled still on the device, and
+those ids are read while it runs (`Engine.overlap_steps`).
 """
 from __future__ import annotations
 
@@ -16,10 +18,10 @@ from dataclasses import dataclass
 
 import torch
 
-from ..sampling.sampler import SamplingParams, sample_rows
+from ..sampling.sampler import SamplingParams, launch_sample_rows
 from .loading import load_model, parse_dtype, random_model
 from .runner import ModelRunner, StepEntry
-from .scheduler import Request, Scheduler
+from .scheduler import UNKNOWN, Request, Scheduler
 
 
 @dataclass
@@ -59,6 +61,7 @@ class Engine:
         self.prefill_chunk = prefill_chunk
         self.eos_token_id = spec.eos_token_id
         self.last_stats: dict = {}
+        self.overlap_steps = True    # False: every step's ids are read before the next step is put together
         self.time_steps = False      # True: every step is bracketed by events and last_stats also says where the time went
 
     @property
@@ -102,29 +105,60 @@ class Engine:
         marks = []            # per step: [event at its first device operation, event after its last launch, all decodes?]
         if self.time_steps:
             self.runner.before_launch = lambda: marks[-1][0].record()
+        # the step whose sampled ids the host has not read yet: its batch, the requests of the rows, the ids on
+        # the device, their copy in pinned memory and the event after that copy
+        inflight = None
+
+        def settle() -> bool:
+            nonlocal inflight
+            if inflight is None:
+                return False
+            batch, rows, _, host_ids, copied = inflight
+            inflight = None
+            copied.synchronize()
+            sched.resolve(batch, {r.id: t for r, t in zip(rows, host_ids.tolist())})
+            return True
+
+        sched.settle = settle
         try:
-            while sched.has_work():
-                batch = sched.schedule()
+            while True:
+                batch = sched.schedule() if sched.has_work() else []
                 if not batch:
+                    if settle():              # the last ids may end a request and free what another waits for
+                        continue
                     if sched.has_work():
                         raise RuntimeError("scheduler made no progress")
                     break
-                entries = [StepEntry(s.request.id, sched.step_tokens(s), [s.n_tokens - 1] if s.samples else [])
-                           for s in batch]
+                row_of = {r.id: i for i, r in enumerate(inflight[1])} if inflight is not None else {}
+                entries, pairs, first = [], [], 0
+                for s in batch:
+                    toks = sched.step_tokens(s)
+                    if toks[-1] == UNKNOWN:         # sampled by the step in flight: taken from the device
+                        pairs.append((first + len(toks) - 1, row_of[s.request.id]))
+                        toks[-1] = 0
+                    entries.append(StepEntry(s.request.id, toks, [s.n_tokens - 1] if s.samples else []))
+                    first += len(toks)
                 if self.time_steps:
                     marks.append([torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True),
                                   all(s.n_tokens == 1 for s in batch)])
-                logits = self.runner.step(entries)
-                sampled = {}
+                logits = self.runner.step(entries, feed=(inflight[2], pairs) if pairs else None)
                 rows = [s.request for s in batch if s.samples]
-                done = marks[-1][1].record if self.time_steps else None
+                launched = None
                 if rows:
-                    toks = sample_rows(logits, [r.params for r in rows], [r.rng for r in rows],
-                                       [r.generated for r in rows], launched=done)
-                    sampled = {r.id: t for r, t in zip(rows, toks)}
-                elif done is not None:
-                    done()
-                sched.commit(batch, sampled)
+                    ids = launch_sample_rows(logits, [r.params for r in rows], [r.rng for r in rows],
+                                             [r.generated for r in rows])
+                    host_ids = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
+                    host_ids.copy_(ids, non_blocking=True)
+                    copied = torch.cuda.Event()
+                    copied.record()
+                    launched = (batch, rows, ids, host_ids, copied)
+                if self.time_steps:
+                    marks[-1][1].record()
+                settle()                      # the ids of the step before this one: they come while this one runs
+                sched.commit_launched(batch)
+                inflight = launched
+                if not self.overlap_steps or any(r.params.uses_history for r in rows):
+                    settle()                  # penalties over what was generated need every token on the host
                 n_steps += 1
                 n_tokens += sum(s.n_tokens for s in batch)
         finally:

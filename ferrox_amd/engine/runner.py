@@ -17,7 +17,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from .. import debug
+from .. import debug, ops
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..csrc.build import ensure_built
@@ -47,9 +47,11 @@ class DecodeGraph:
         self.keys = list(mgr.groups)
         total = mgr.step_words(n_seqs, n_seqs, n_seqs, self.max_blocks)
         dev = runner.device
-        self.meta = torch.zeros(total, dtype=torch.int32, device=dev)
-        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        # behind the step's own words: room for one (place, row) pair per token that is fed from the device
+        self.meta = torch.zeros(total + 2 * n_seqs, dtype=torch.int32, device=dev)
+        self.host = torch.zeros(total + 2 * n_seqs, dtype=torch.int32, pin_memory=True)
         self._host_ptr, self._host_words = self.host.data_ptr(), total
+        self._host_np = self.host.numpy()
         self.copied = torch.cuda.Event()
         self.copied.record()
         self.graph = None
@@ -69,9 +71,10 @@ class DecodeGraph:
                           logit_rows=m[4 * n:5 * n], recorded=True, kv_bound=self.kv_bound)
         return ctx
 
-    def run(self, entries) -> torch.Tensor:
+    def run(self, entries, feed=None) -> torch.Tensor:
         """The logits of the entries' tokens (one each).  Fewer entries than the step was recorded for are
-        filled up with stand-in rows, which write to a page and a slot that no request owns."""
+        filled up with stand-in rows, which write to a page and a slot that no request owns.  `feed` as in
+        `ModelRunner.step`."""
         self.copied.synchronize()                  # the last upload has left the staging buffer
         for e in entries:
             if e.want[0] != 0:
@@ -82,7 +85,16 @@ class DecodeGraph:
                                         pad_pages=storage.pad_pages, pad_slot=storage.pad_slot)
         if self.runner.before_launch is not None:
             self.runner.before_launch()
-        self.meta.copy_(self.host, non_blocking=True)
+        words = self._host_words
+        if feed:
+            ids, pairs = feed
+            flat = check_feed(ids, pairs, len(entries))
+            self._host_np[words:words + len(flat)] = flat
+            self.meta[:words + len(flat)].copy_(self.host[:words + len(flat)], non_blocking=True)
+            ops.feed_tokens(self.meta[:self.n], ids, self.meta[words:words + len(flat)].view(-1, 2),
+                            len(entries), ids.numel())
+        else:
+            self.meta[:words].copy_(self.host[:words], non_blocking=True)
         self.copied.record()
         model, caches = self.runner.model, self.runner.storage.caches
         if self.graph is None:
@@ -118,6 +130,16 @@ class DecodeGraph:
         if debug.routing_trace is not None:
             debug.routing_trace.replayed(self.trace_calls)
         return self.logits[:len(entries)]
+
+
+def check_feed(ids: torch.Tensor, pairs: list, n_tokens: int) -> list:
+    """`pairs` flattened, after a check that every place lies among the step's tokens and every row among `ids`."""
+    flat = []
+    for place, row in pairs:
+        if not (0 <= place < n_tokens and 0 <= row < ids.numel()):
+            raise ValueError(f"token {place} of {n_tokens} cannot be fed from row {row} of {ids.numel()} sampled ids")
+        flat += (place, row)
+    return flat
 
 
 class ModelRunner:
@@ -167,10 +189,15 @@ class ModelRunner:
             self._uploaded.synchronize()
         return self._host
 
-    def step(self, entries: list) -> torch.Tensor | None:
+    def step(self, entries: list, feed=None) -> torch.Tensor | None:
         """Logits [number of wanted places, vocab] in the order of the entries and of each
         entry's `want`, or None if nothing is wanted.  Every entry's request must hold pages
-        for its tokens already (`reserve`)."""
+        for its tokens already (`reserve`).
+
+        `feed = (ids, [(place, row), ...])` names tokens of this step that the host does not know yet: token
+        number `place` (counted through all entries) is `ids[row]`, an int32 tensor on the device that an
+        earlier step's sampling wrote; the entry holds any valid id in its stead.  So a step can be launched
+        while the one before it still runs."""
         mgr = self.manager
         n_seqs = len(entries)
         reqs = [e.req for e in entries]
@@ -191,7 +218,7 @@ class ModelRunner:
                     self._graphs.pop(next(iter(self._graphs)))
                 self._graphs[key] = DecodeGraph(self, n_rec, bound)
             try:
-                logits = self._graphs[key].run(entries)
+                logits = self._graphs[key].run(entries, feed)
             except RuntimeError as err:
                 # recording is an optimisation of how kernels are launched, not another code path:
                 # if the runtime refuses it, the same kernels are launched one by one from here on
@@ -206,13 +233,19 @@ class ModelRunner:
                 return logits
         longest = max((mgr.length(r) for r in reqs if r in mgr), default=0)
         max_blocks = max(1, mgr.blocks_for(longest))
-        host = self._staging(mgr.step_words(T, n_seqs, R, max_blocks))
+        flat = check_feed(feed[0], feed[1], T) if feed else []
+        host = self._staging(mgr.step_words(T, n_seqs, R, max_blocks) + len(flat))
         packed = mgr.pack_step(reqs, token_lists, wants, self.vocab_size, host.data_ptr(), host.numel())
-        dev = torch.empty(packed.total, dtype=torch.int32, device=self.device)
+        words = packed.total + len(flat)
+        if flat:
+            host[packed.total:words] = torch.tensor(flat, dtype=torch.int32)
+        dev = torch.empty(words, dtype=torch.int32, device=self.device)
         if self.before_launch is not None:
             self.before_launch()
-        dev.copy_(host[:packed.total], non_blocking=True)
+        dev.copy_(host[:words], non_blocking=True)
         self._uploaded.record()
+        if flat:
+            ops.feed_tokens(dev[:T], feed[0], dev[packed.total:words].view(-1, 2), T, feed[0].numel())
         o = 0
 
         def take(n):

@@ -20,6 +20,14 @@ Order of a request's life, as in the reference (batch_scheduler.rs:195-237):
 logits of its last position are sampled; EOS finishes it ("stop") without being
 appended; otherwise the token is appended; reaching max_new_tokens or the
 context limit finishes it ("length") without a forward pass for the last token.
+
+A step's sampled ids may be read one step late, so that the next step is launched
+while this one still runs: `commit_launched` advances the requests with a stand-in
+(`UNKNOWN`) for each sampled token, which the next step takes from the device;
+`resolve` puts the ids in once the host has them and finishes the requests whose
+token was EOS (their part of the step launched meanwhile is thrown away).  What a
+request generates is the same either way.  Before it preempts or gives up on a
+request the scheduler calls `settle`, so such decisions are made on known tokens.
 """
 from __future__ import annotations
 
@@ -27,6 +35,8 @@ from collections import deque
 from dataclasses import dataclass, field
 
 from ..sampling.sampler import SamplingParams, XorShift64
+
+UNKNOWN = -1          # in `Request.generated`: a token that is sampled but not read back yet
 
 
 @dataclass
@@ -64,6 +74,7 @@ class Scheduled:
     request: Request
     n_tokens: int
     samples: bool          # the portion reaches the request's last token: its logits are sampled
+    place: int = -1        # where in `request.generated` the sampled token goes (set by `commit_launched`)
 
 
 class Scheduler:
@@ -83,6 +94,7 @@ class Scheduler:
         self.finished: list = []
         self._arrivals = 0
         self.n_preemptions = 0
+        self.settle = None        # callable -> bool: read the ids still in flight and `resolve` them; True if any were
 
     # ---- arrival -----------------------------------------------------------
     def add(self, req: Request) -> None:
@@ -117,6 +129,12 @@ class Scheduler:
                 continue
             n = min(req.n_pending, budget, self.prefill_chunk if req.n_pending > 1 else 1)
             while not self.cache.reserve(req.id, n):
+                if self.settle is not None and self.settle():
+                    # ids that were in flight are known now: a request may have ended and given pages back
+                    if req.status != "running":
+                        n = 0
+                        break
+                    continue
                 victim = self._youngest_running(exclude=scheduled_ids)
                 if victim is None or victim is req:
                     if len(self.running) == 1 or victim is None:
@@ -140,6 +158,8 @@ class Scheduler:
                 break
             if not self.cache.reserve(req.id, n):
                 self.cache.release(req.id)
+                if self.settle is not None and self.settle():
+                    continue
                 if not self.running:          # nothing will ever free pages for it
                     self.waiting.popleft()
                     self._finish(req, "cache_full")
@@ -150,7 +170,8 @@ class Scheduler:
             self.running.append(req)
             out.append(Scheduled(req, n, n == req.n_pending))
             budget -= n
-        return out
+        # a request that `settle` ended after it was put on the list holds no pages any more
+        return [s for s in out if s.request.status == "running"]
 
     def step_tokens(self, s: Scheduled) -> list:
         toks = s.request.tokens
@@ -159,20 +180,46 @@ class Scheduler:
     def commit(self, scheduled: list, sampled: dict) -> None:
         """After the step: advance every scheduled request; `sampled[id]` is the token drawn from
         the logits of a request whose portion reached its end."""
+        self.commit_launched(scheduled)
+        self.resolve(scheduled, sampled)
+
+    def commit_launched(self, scheduled: list) -> None:
+        """The step is launched: advance every scheduled request that is still running, with `UNKNOWN` in the
+        place of each sampled token.  Whether a request ends for its length does not depend on the token."""
         for s in scheduled:
             req = s.request
+            if req.status != "running":          # ended by an id that was read after the step was put together
+                s.samples = False
+                continue
             req.n_computed += s.n_tokens
             if not s.samples:
                 continue
-            tok = int(sampled[req.id])
-            if req.eos_token_id is not None and tok == req.eos_token_id and not req.ignore_eos:
-                self._finish(req, "stop")
-                continue
-            req.generated.append(tok)
+            s.place = len(req.generated)
+            req.generated.append(UNKNOWN)
             if len(req.generated) >= req.max_new_tokens:
                 self._finish(req, "length")
             elif self.context_limit is not None and len(req.prompt) + len(req.generated) >= self.context_limit:
                 self._finish(req, "length")
+
+    def resolve(self, scheduled: list, sampled: dict) -> None:
+        """The ids of a step that `commit_launched` advanced are known: `sampled[id]` for every request it
+        sampled.  EOS ends the request without being appended, also where its length ended it already."""
+        for s in scheduled:
+            if not s.samples:
+                continue
+            req, tok = s.request, int(sampled[s.request.id])
+            if req.generated[s.place] != UNKNOWN:
+                raise RuntimeError(f"request {req.id!r}: token {s.place} was resolved twice")
+            if req.eos_token_id is not None and tok == req.eos_token_id and not req.ignore_eos:
+                del req.generated[s.place:]
+                if req.status == "waiting":          # preempted meanwhile
+                    self.waiting.remove(req)
+                if req.status == "finished":
+                    req.finish_reason = "stop"
+                else:
+                    self._finish(req, "stop")
+            else:
+                req.generated[s.place] = tok
 
     # ---- internals -----------------------------------------------------------
     def _youngest_running(self, exclude=()):

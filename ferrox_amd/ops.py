@@ -54,6 +54,7 @@ _sigs = {
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     ("elementwise", "fx_fill_u32"): [c_void_p, c_void_p, ctypes.c_uint, c_long],
+    ("elementwise", "fx_feed_tokens"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
@@ -184,6 +185,19 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
     if not t.is_contiguous() or t.element_size() * t.numel() % 4:
         raise KernelError("fill_u32 wants a contiguous buffer of whole 32-bit words")
     _call("elementwise", "fx_fill_u32", _stream(), _p(t), value, t.element_size() * t.numel() // 4)
+
+
+def feed_tokens(tokens: torch.Tensor, ids: torch.Tensor, pairs: torch.Tensor, n_tokens: int, n_ids: int) -> None:
+    """tokens[pairs[i, 0]] = ids[pairs[i, 1]], all int32 on the device.  `pairs` [n, 2] was written by the host,
+    which has checked it against `n_tokens` and `n_ids`; the ids come from the sampling kernel."""
+    for t, name in ((tokens, "tokens"), (ids, "ids"), (pairs, "pairs")):
+        if t.dtype != torch.int32 or not t.is_contiguous() or not t.is_cuda:
+            raise KernelError(f"feed_tokens: {name} must be contiguous int32 on the GPU")
+    if pairs.dim() != 2 or pairs.shape[1] != 2:
+        raise KernelError("feed_tokens: pairs must be [n, 2]")
+    if tokens.numel() < n_tokens or ids.numel() < n_ids:
+        raise KernelError("feed_tokens: a buffer is shorter than the bound its pairs were checked against")
+    _call("elementwise", "fx_feed_tokens", _stream(), _p(tokens), _p(ids), _p(pairs), pairs.shape[0])
 
 
 class ScaleLater:

@@ -59,40 +59,52 @@ class XorShift64:
         return (self.next_u64() >> 40) / float(1 << 24)
 
 
-def sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list, launched=None) -> list:
-    """One token id per row of `logits` [R, V] (float32, on the GPU).  `params[r]`,
-    `rngs[r]`, `histories[r]` (the tokens generated so far) belong to row r.  A generator is
-    advanced only for rows that draw.  `launched()` is called after the kernel is launched and
-    before the host waits for the ids (for measurement)."""
-    R = logits.shape[0]
-    dev = logits.device
+def _upload(dev, floats: dict, ints: dict) -> dict:
+    """All per-row parameters of one sampling call in one pinned buffer and one copy that the host does not wait
+    for: name -> float32 or int32 tensor on `dev`."""
+    n = sum(len(v) for v in floats.values()) + sum(len(v) for v in ints.values())
+    host = torch.empty(n, dtype=torch.float32, pin_memory=True)
+    as_f, as_i = host.numpy(), host.view(torch.int32).numpy()
+    spans, o = {}, 0
+    for group, view, integer in ((floats, as_f, False), (ints, as_i, True)):
+        for name, vals in group.items():
+            view[o:o + len(vals)] = vals
+            spans[name] = (o, o + len(vals), integer)
+            o += len(vals)
+    there = host.to(dev, non_blocking=True)
+    there_i = there.view(torch.int32)
+    return {name: (there_i if integer else there)[a:b] for name, (a, b, integer) in spans.items()}
 
-    def ids_of(out):
-        if launched is not None:
-            launched()
-        return out.tolist()
 
+def launch_sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list) -> torch.Tensor:
+    """One token id per row of `logits` [R, V] (float32, on the GPU), as an int32 tensor on the GPU; the host
+    waits for nothing.  `params[r]`, `rngs[r]`, `histories[r]` (the tokens generated so far) belong to row r.
+    A generator is advanced only for rows that draw."""
     if all(p.greedy and not p.uses_history for p in params):
-        return ids_of(ops.sample(logits))
-
-    def f32(vals):
-        return torch.tensor(vals, dtype=torch.float32, device=dev)
-
+        return ops.sample(logits)
     draws = [0.0 if p.greedy else rng.next_f32() for p, rng in zip(params, rngs)]
-    kw = dict(temperature=f32([p.temperature for p in params]), draw=f32(draws))
+    floats, ints = dict(temperature=[p.temperature for p in params], draw=draws), {}
     if any(p.top_k > 0 for p in params):
-        kw["top_k"] = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=dev)
+        ints["top_k"] = [p.top_k for p in params]
     if any(p.top_p < 1.0 for p in params):
-        kw["top_p"] = f32([p.top_p for p in params])
+        floats["top_p"] = [p.top_p for p in params]
     if any(p.uses_history for p in params):
         flat, starts = [], [0]
         for p, h in zip(params, histories):
             if p.uses_history:
                 flat.extend(h)
             starts.append(len(flat))
-        kw["hist"] = torch.tensor(flat or [0], dtype=torch.int32, device=dev)
-        kw["hist_start"] = torch.tensor(starts, dtype=torch.int32, device=dev)
-        kw["rep_penalty"] = f32([p.repetition_penalty for p in params])
-        kw["presence"] = f32([p.presence_penalty for p in params])
-        kw["frequency"] = f32([p.frequency_penalty for p in params])
-    return ids_of(ops.sample(logits, **kw))
+        ints["hist"], ints["hist_start"] = flat or [0], starts
+        floats["rep_penalty"] = [p.repetition_penalty for p in params]
+        floats["presence"] = [p.presence_penalty for p in params]
+        floats["frequency"] = [p.frequency_penalty for p in params]
+    return ops.sample(logits, **_upload(logits.device, floats, ints))
+
+
+def sample_rows(logits: torch.Tensor, params: list, rngs: list, histories: list, launched=None) -> list:
+    """`launch_sample_rows`, read back: a list of token ids.  `launched()` is called after the kernel is
+    launched and before the host waits for the ids (for measurement)."""
+    out = launch_sample_rows(logits, params, rngs, histories)
+    if launched is not None:
+        launched()
+    return out.tolist()

@@ -582,3 +582,66 @@ def test_generation_of_a_batch_that_shrinks(model_folders):
     assert 16 in sizes and any(n <= 8 for n in sizes), f"recorded sizes {sorted(sizes)}"
     for p, n, g in zip(prompts, lengths, got):
         assert g.token_ids == plain.greedy_generate(cfg, w, p, n) and g.finish_reason == "length"
+
+
+def test_a_step_takes_tokens_that_are_still_on_the_device(model_folders):
+    """`step(entries, feed=...)`: tokens named by (place, row) come from a device tensor of sampled ids; the
+    logits are those of the same step with the tokens given by the host (on requests with the same contents),
+    in recorded decode steps and in mixed steps launched kernel by kernel; a place or row out of range is
+    refused on the host"""
+    from ferrox_amd.engine.runner import StepEntry
+    folder, runner = runner_for(model_folders, "B", "bfloat16", block_size=16, num_pages=40, max_seqs=8)
+    vocab = runner.vocab_size
+    ids = torch.tensor([5, vocab - 1, 17, 3], dtype=torch.int32, device="cuda")
+    for k, rid in enumerate(["a", "b", "c", "a'", "b'", "c'"]):
+        assert runner.admit(rid) and runner.reserve(rid, 21)
+        runner.step([StepEntry(rid, [(7 * (k % 3) + j) % vocab for j in range(21)], [])])
+
+    def step(entries, feed=None):
+        for e in entries:
+            assert runner.reserve(e.req, len(e.tokens))
+        return runner.step(entries, feed=feed).clone()
+
+    # a recorded decode step: the tokens of b and c come from rows 1 and 3
+    known = step([StepEntry("a", [9], [0]), StepEntry("b", [vocab - 1], [0]), StepEntry("c", [3], [0])])
+    fed = step([StepEntry("a'", [9], [0]), StepEntry("b'", [0], [0]), StepEntry("c'", [0], [0])], (ids, [(1, 1), (2, 3)]))
+    assert runner._graphs and torch.equal(known, fed)
+    # a mixed step: a portion of four tokens whose last is fed, beside a decoded token that is fed
+    known = step([StepEntry("a", [1, 2, 3, 17], [3]), StepEntry("b", [5], [0])])
+    fed = step([StepEntry("a'", [1, 2, 3, 0], [3]), StepEntry("b'", [0], [0])], (ids, [(3, 2), (4, 0)]))
+    assert torch.equal(known, fed)
+    assert runner.reserve("c", 1)
+    for bad in ([(1, 0)], [(0, 4)], [(-1, 0)]):
+        with pytest.raises(ValueError, match="cannot be fed"):
+            runner.step([StepEntry("c", [0], [0])], feed=(ids, bad))
+
+
+def test_reading_ids_one_step_late_generates_the_same(model_folders):
+    """the engine launches a step before it has read the ids that the step before it sampled; requests that stop at
+    an EOS in the middle of the batch, a pool small enough for preemptions, and seeded temperature sampling give
+    the same tokens and reasons as with every step's ids read at once, and as the plain model"""
+    import plain_qwen2moe as plain
+    from ferrox_amd.engine.api import Engine
+    from ferrox_amd.sampling import SamplingParams
+    folder = model_folders("A", "float32")
+    cfg, w = plain.load_folder(folder)
+    prompts = list(ru.make_requests(cfg["vocab_size"], [5, 12, 3, 30, 9, 17], 33).values())
+    engine = Engine(folder, dtype="float32", block_size=8, num_pages=30, max_seqs=6, max_tokens_per_step=40, prefill_chunk=16)
+    free = engine.generate(prompts, max_new_tokens=20, ignore_eos=True)
+    # an EOS that request 1 produces as its 6th token: the others stop where they produce it, if they do
+    eos = free[1][5]
+    expect = []
+    for g in free:
+        expect.append((g[:g.index(eos)], "stop") if eos in g else (g, "length"))
+    assert expect[1][1] == "stop" and any(r == "length" for _, r in expect)
+    assert expect[1][0] == plain.greedy_generate(cfg, w, prompts[1], 20)[:len(expect[1][0])]
+    params = [SamplingParams(temperature=0.7, seed=40 + i) for i in range(6)]
+    outcomes = {}
+    for late in (True, False):
+        engine.overlap_steps = late
+        got = engine.generate_detailed(prompts, 20, eos_token_id=eos)
+        assert [(c.token_ids, c.finish_reason) for c in got] == expect, f"ids read late: {late}"
+        drawn = engine.generate_detailed(prompts, 20, params, eos_token_id=eos)
+        outcomes[late] = [(c.token_ids, c.finish_reason) for c in drawn]
+        assert engine.runner.manager.n_free_pages() == 30
+    assert outcomes[True] == outcomes[False]

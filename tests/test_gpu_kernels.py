@@ -763,3 +763,22 @@ def test_route_in_one_launch_equals_two(T, E, k):
     two = (ids, w, gate) + ops.moe_align(ids, E)
     for a, b in zip(fused, two):
         assert torch.equal(a, b)
+
+
+def test_tokens_fed_from_sampled_ids():
+    """tokens[place] = ids[row] for the pairs given, everything else untouched; buffers of the wrong kind are refused"""
+    from ferrox_amd import ops
+    g = torch.Generator().manual_seed(3)
+    tokens = torch.randint(0, 1000, (777,), generator=g, dtype=torch.int32)
+    ids = torch.randint(0, 1000, (300,), generator=g, dtype=torch.int32)
+    places = torch.randperm(777, generator=g)[:300]
+    rows = torch.randint(0, 300, (300,), generator=g)
+    expect = tokens.clone()
+    expect[places] = ids[rows]
+    d_tokens, pairs = tokens.cuda(), torch.stack([places, rows], 1).to(torch.int32).cuda()
+    ops.feed_tokens(d_tokens, ids.cuda(), pairs, 777, 300)
+    assert torch.equal(d_tokens.cpu(), expect)
+    with pytest.raises(ops.KernelError):
+        ops.feed_tokens(d_tokens, ids.cuda().long(), pairs, 777, 300)
+    with pytest.raises(ops.KernelError):
+        ops.feed_tokens(d_tokens, ids.cuda(), pairs, 778, 300)

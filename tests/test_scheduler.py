@@ -139,3 +139,77 @@ def test_each_request_has_its_own_seeded_generator():
     xs = [a.rng.next_f32() for _ in range(3)]
     assert xs == [b.rng.next_f32() for _ in range(3)] == [XorShift64(7).next_f32() for _ in range(1)] + xs[1:]
     assert XorShift64(1).next_u64() == 0x40822041 and XorShift64(0).state == 0x9E3779B97F4A7C15
+
+
+def run_late(sched, next_token, max_steps=10_000):
+    """Drives the scheduler as the engine does when it reads a step's ids one step late: the next step is put
+    together and launched (here: its pages checked) before the ids of the one before are resolved."""
+    from ferrox_amd.engine.scheduler import UNKNOWN
+    inflight = []
+
+    def settle():
+        if not inflight:
+            return False
+        batch, ids = inflight.pop()
+        sched.resolve(batch, ids)
+        sched.cache.m.check_invariants()
+        return True
+
+    sched.settle = settle
+    n_steps = n_fed = 0
+    while True:
+        batch = sched.schedule() if sched.has_work() else []
+        if not batch:
+            if settle():
+                continue
+            assert not sched.has_work()
+            break
+        for s in batch:
+            toks = sched.step_tokens(s)
+            assert sched.cache.m.length(s.request.id) == s.request.n_computed + s.n_tokens
+            assert UNKNOWN not in toks[:-1]                      # only a request's newest token can be on the way
+            if toks[-1] == UNKNOWN:
+                assert inflight and any(x.request is s.request and x.samples for x in inflight[0][0])
+                n_fed += 1
+        # the ids are what the model would give: a function of the request and of how much it has generated
+        ids = {s.request.id: next_token(s.request) for s in batch if s.samples}
+        settle()
+        sched.commit_launched(batch)
+        inflight.append((batch, ids))
+        sched.cache.m.check_invariants()
+        n_steps += 1
+        assert n_steps < max_steps
+    return n_fed
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_reading_the_ids_one_step_late_changes_nothing_that_is_generated(seed):
+    import random
+    rnd = random.Random(seed)
+    n_req = rnd.randint(2, 7)
+    spec = [(rnd.randint(1, 30), rnd.randint(1, 25)) for _ in range(n_req)]
+    pages, budget, chunk = rnd.randint(10, 24), rnd.randint(4, 40), rnd.randint(2, 16)
+    eos = 7
+
+    def nxt(req):          # the position decides: the same token whenever and with whomever it is computed
+        return (req.id * 131 + (len(req.prompt) + len(req.generated)) * 17) % 11
+
+    outcomes = []
+    for late in (False, True):
+        sched = Scheduler(Cache(pages, block_size=4), max_tokens_per_step=budget, prefill_chunk=chunk, context_limit=48)
+        for i, (n_prompt, n_new) in enumerate(spec):
+            sched.add(Request(i, [((i + j) % 5) for j in range(n_prompt)], n_new, eos_token_id=eos, ignore_eos=(i % 3 == 2)))
+        fed = run_late(sched, nxt) if late else run(sched, nxt)
+        assert sched.cache.m.n_free_pages() == pages and len(sched.finished) == n_req
+        assert all(t >= 0 for r in sched.finished for t in r.generated)
+        outcomes.append({r.id: (r.generated, r.finish_reason) for r in sched.finished})
+    assert fed > 0
+    # a request that ends because the cache is full ends where the pages ran out, which may differ by the one
+    # step that a request that has stopped already still holds its pages; everything else is the same
+    for rid, (gen, reason) in outcomes[0].items():
+        gen_late, reason_late = outcomes[1][rid]
+        if "cache_full" in (reason, reason_late):
+            n = min(len(gen), len(gen_late))
+            assert gen[:n] == gen_late[:n]
+        else:
+            assert (gen, reason) == (gen_late, reason_late)
