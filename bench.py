@@ -224,7 +224,7 @@ class Bench:
         from ferrox_amd.engine.api import Engine
         per_seq = -(-(ctx + new_tokens + 1) // self.block_size)
         eng = Engine(model=self.model, block_size=self.block_size, num_pages=per_seq * batch + 8, max_seqs=batch,
-                     max_tokens_per_step=2048, prefill_chunk=2048, ctx_size=ctx + new_tokens + 8)
+                     max_tokens_per_step=4096, prefill_chunk=4096, ctx_size=ctx + new_tokens + 8)
         eng.time_steps = True
         prompts = self.prompts(batch, ctx)
         # once untimed: decode steps are recorded (a HIP graph per number of sequences and length bound) the first
@@ -354,15 +354,15 @@ def run_workload(name: str, args) -> int:
     if name == "config3":
         for B in (8, 64):
             L = [2048] * B
-            serve(prompts_of(L), 256, 2048, 2048, B, pages_for(L, 256), f"B={B}")
+            serve(prompts_of(L), 256, 4096, 4096, B, pages_for(L, 256), f"B={B}")
     elif name == "config4":
         L = [rng.randint(512, 16384) for _ in range(32)]
         serve(prompts_of(L), 128, 512, 512 + 32, 32, pages_for(L, 128), "32 requests, 512-token portions")
     else:
         L = [24576] * 8
-        serve(prompts_of(L), 256, 2048, 2048, 8, pages_for(L, 256), "8 x 24,576-token prompts, 256 new tokens")
+        serve(prompts_of(L), 256, 4096, 4096, 8, pages_for(L, 256), "8 x 24,576-token prompts, 256 new tokens")
         L = [rng.randint(1024, 24576) for _ in range(64)]
-        serve(prompts_of(L), 32, 2048, 2048 + 64, 64, pages_for(L, 32), "64 requests at depths 1k..24k, 32 new tokens")
+        serve(prompts_of(L), 32, 4096, 4096 + 64, 64, pages_for(L, 32), "64 requests at depths 1k..24k, 32 new tokens")
     print(json.dumps({"workload": name, "model": shape_name, "layers": cfg["num_hidden_layers"], "dtype": args.dtype,
                       "results": results}), flush=True)
     return 0

@@ -39,8 +39,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "bfloat16", "fp32", "float32"])
     ap.add_argument("--block-size", type=int, default=64)
     ap.add_argument("--num-pages", type=int, default=0, help="cache pages per layer group (0 = from the context)")
-    ap.add_argument("--max-tokens-per-step", type=int, default=2048)
-    ap.add_argument("--prefill-chunk", type=int, default=2048,
+    ap.add_argument("--max-tokens-per-step", type=int, default=4096)
+    ap.add_argument("--prefill-chunk", type=int, default=4096,
                     help="most tokens of one prompt in a step (a step streams every expert it uses once, so large portions pay)")
     return ap
 

@@ -35,7 +35,7 @@ class Completion:
 class Engine:
     def __init__(self, model_dir: str | None = None, *, config=None, random_weights: int | None = None,
                  model=None, dtype="bfloat16", device="cuda:0", block_size: int = 64, num_pages: int | None = None,
-                 max_seqs: int = 64, max_tokens_per_step: int = 2048, prefill_chunk: int = 2048,
+                 max_seqs: int = 64, max_tokens_per_step: int = 4096, prefill_chunk: int = 4096,
                  ctx_size: int = 0):
         """One of: `model_dir` (config.json + safetensors), `config` with `random_weights=<seed>`, or `model`,
         a model that is loaded already (its dtype and device are taken)."""

@@ -78,7 +78,7 @@ class Scheduled:
 
 
 class Scheduler:
-    def __init__(self, cache, *, max_tokens_per_step: int = 2048, prefill_chunk: int = 2048,
+    def __init__(self, cache, *, max_tokens_per_step: int = 4096, prefill_chunk: int = 4096,
                  max_seqs: int | None = None, context_limit: int | None = None, vocab_size: int | None = None):
         """`cache` offers admit(id) -> bool, reserve(id, n) -> bool, release(id)."""
         if max_tokens_per_step < 1 or prefill_chunk < 1:
