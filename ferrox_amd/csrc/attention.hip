@@ -596,17 +596,31 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int p = a.positions[tok];
-    // the page ids of the whole chunk are copied, whatever part of it the position and the window leave: the copy
-    // then does not wait for the position to arrive (entries past the sequence's pages are read and never used)
+    // The keys this query sees, from the tile of 64 that holds the first of them on, go to the splits in equal
+    // chunks of whole tiles: a sequence shorter than the launch's bound, or a window far into a long sequence,
+    // still keeps every split busy.  (a.chunk is the longest chunk any sequence of the launch can have.)
     __shared__ int page_copy[PAGE_COPY];
     int first_blk, last_blk, unused;
-    page_slot(a, split * a.chunk, first_blk, unused);
-    page_slot(a, (split + 1) * a.chunk - 1, last_blk, unused);
-    first_blk = min(first_blk, a.max_blocks - 1);
-    last_blk = min(last_blk, a.max_blocks - 1);
-    const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
-    const int kv_begin = max(a.window > 0 ? max(0, p - a.window + 1) : 0, split * a.chunk);
-    const int kv_end = min(p + 1, (split + 1) * a.chunk);
+    PageLookup pl;
+    if (a.window <= 0) {
+        // the page ids that the split can need, whatever the position turns out to be, are copied before the
+        // position has arrived (entries past the sequence's pages are read and never used)
+        page_slot(a, (split + 1) * a.chunk - 1, last_blk, unused);
+        last_blk = min(last_blk, a.max_blocks - 1);
+        pl = stage_pages(bt, page_copy, max(0, last_blk - PAGE_COPY + 1), last_blk);
+    }
+    const int first_key = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const int base = first_key & ~63;
+    const int chunk = (((p + 1 - base + a.splits - 1) / a.splits) + 63) & ~63;
+    const int kv_begin = max(first_key, base + split * chunk);
+    const int kv_end = min(p + 1, base + (split + 1) * chunk);
+    if (a.window > 0) {
+        page_slot(a, min(kv_begin, p), first_blk, unused);
+        page_slot(a, max(kv_end - 1, 0), last_blk, unused);
+        first_blk = min(first_blk, a.max_blocks - 1);
+        last_blk = min(last_blk, a.max_blocks - 1);
+        pl = stage_pages(bt, page_copy, first_blk, last_blk);
+    }
     const int n = min(16, group - hb * 16);        // query heads in this block
     const int h0 = kvh * group + hb * 16;
     const bool empty = kv_begin >= kv_end;

@@ -410,10 +410,11 @@ def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, 
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
                      waves=0) -> None:
-    """Single queries.  The keys are cut into chunks of `chunk` positions that are merged in
-    ascending order; by default float32 uses 256 always (so that a result does not depend on the
-    batch) and bfloat16, whose blocks of eight waves share a chunk, takes the fewest chunks that
-    still put about two thousand waves on the GPU: one chunk, and no merge launch, from 256
+    """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
+    order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
+    batch); bfloat16, whose blocks of eight waves share a chunk, cuts every sequence's own range of keys (from its
+    window's first key to its position) into that many equal chunks of whole tiles of 64, and by default takes the
+    fewest chunks that still put about two thousand waves on the GPU: one chunk, and no merge launch, from 256
     (sequence, kv head) pairs on."""
     n = item_seq.numel()
     if chunk is None:
