@@ -173,8 +173,11 @@ class Bench:
             copied.record()
             return out, host, copied
 
+        done_at = []                               # when the host saw each step's ids
+
         def collect(step):
             step[2].synchronize()
+            done_at.append(time.perf_counter())
             read.append(step[1].tolist())
 
         # as the engine generates: the host is one step ahead; a step is launched with the ids of the step before
@@ -186,19 +189,25 @@ class Bench:
             flying = nxt
         parts = max(1, min(parts, steps))
         sizes = [steps // parts + (1 if i < steps % parts else 0) for i in range(parts)]
-        per_part = []
         torch.cuda.synchronize()
+        collect(flying)                            # (it has ended; only its ids are read here)
+        on_device, flying = flying[0], None
+        first = len(done_at)
         t_all = time.perf_counter()
-        for n in sizes:                            # exactly `steps` steps between the two synchronisations
-            t0 = time.perf_counter()
-            for _ in range(n):
-                nxt = launch(None, flying[0])
+        for _ in range(steps):                     # exactly `steps` steps between the two synchronisations
+            nxt = launch(None, on_device)
+            if flying is not None:
                 collect(flying)                    # (waits for the step before the one just launched)
-                flying = nxt
-            per_part.append((time.perf_counter() - t0) / n)
+            flying, on_device = nxt, nxt[0]
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t_all) / steps
         collect(flying)
+        # a part's time per step, from when the host saw the last step before it end to when it saw its own last
+        ends = [t_all] + done_at[first:]
+        per_part, at = [], 0
+        for n in sizes:
+            per_part.append((ends[at + n] - ends[at]) / n)
+            at += n
         assert all(0 <= t < self.cfg.vocab_size for row in read for t in row) and len(read) == warmup + steps + 1
         # one more, untimed, step that records which experts the router chose
         with debug.trace_routing() as trace:
