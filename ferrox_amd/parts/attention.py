@@ -40,7 +40,8 @@ def attention_items(ctx, tile_q: int = 64):
                 t_tok.append(t0)
                 t_n.append(min(tile_q, e - t0))
     flat = dec_seq + dec_tok + t_seq + t_tok + t_n
-    dev = torch.tensor(flat, dtype=torch.int32, device=ctx.device) if flat else None
+    # through pinned memory, so that the host does not wait here for the kernels launched before
+    dev = torch.tensor(flat, dtype=torch.int32).pin_memory().to(ctx.device, non_blocking=True) if flat else None
     nd, nt = len(dec_seq), len(t_seq)
     items = {"n_decode": nd, "n_tiles": nt, "max_kv": max_kv}
     if nd:
