@@ -1127,14 +1127,16 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per wave of the product for few rows (0: by the sizes)
 static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
 static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
+static int g_few_rows = 4;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
 static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "skinny_sets")) { g_skinny_nw = value; return 0; }
     if (!strcmp(key, "skinny_row_tiles")) { g_skinny_mt = value; return 0; }
     if (!strcmp(key, "skinny_waves")) { g_skinny_waves = value; return 0; }
+    if (!strcmp(key, "few_rows")) { g_few_rows = value < 0 ? 0 : (value > 64 ? 64 : value); return 0; }
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
-    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, wide)", key);
+    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, wide)", key);
     return 1;
 }
 
@@ -1304,12 +1306,20 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                ((K % 8 == 0) && (lda % 8 == 0) && (w_stride % 8 == 0) && (up_offset % 8 == 0) &&
                 (((uintptr_t)A | (uintptr_t)W) % 16 == 0));
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
+    const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
     FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
     // 33..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights faster
     // than four row tiles per block of the kernel for few rows
     const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > 32 && K % 64 == 0 &&
                               !g_no_wide && ceil_div(N, 128) >= 512;
-    if (g.vec_ok && (per_group <= 64 || pair_ids) && !many_columns) {
+    // Rows sorted by expert: the product for few rows only up to four rows an expert on average.  Its waves fetch
+    // every row tile's operands themselves, so its time grows with the rows (512 tokens of the larger model, 64 rows
+    // an expert: 1,107 us for the gate/up product at 2.1 TB/s), while the tiled product, whose tile of 192 rows
+    // holds an expert's share, streams the weights at the same speed whatever the rows (400 us at 5.9 TB/s); decode
+    // steps of 48 and 64 sequences 10.3 -> 10.0 and 12.0 -> 11.4 ms, of 17 to 64 of the larger model's sizes 8-24 %
+    // less, and with three or four rows an expert the product for few rows is still 2-6 % ahead.
+    const long few_limit = expert_offsets && wide_ok ? g_few_rows : 64;
+    if (g.vec_ok && (per_group <= few_limit || pair_ids) && !many_columns) {
         int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
         if (g_skinny_mt && !pair_ids) mt = g_skinny_mt;
         const int m_tiles = pair_ids ? (M < E ? M : E) + M / 16 + n_always
@@ -1334,9 +1344,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
         return 0;
     }
-    const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
-    FX_REQUIRE(!g.kb_stride || (per_group > 64 && wide_ok), "gemm: no kernel for weights in slabs of 64 k at these sizes");
-    if (per_group <= 64 && !many_columns) {
+    FX_REQUIRE(!g.kb_stride || wide_ok, "gemm: no kernel for weights in slabs of 64 k at these sizes");
+    if (per_group <= 64 && !many_columns && !wide_ok) {
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else if (g.vec_ok && K % 64 == 0 && !g_no_wide) {

@@ -782,3 +782,32 @@ def test_tokens_fed_from_sampled_ids():
         ops.feed_tokens(d_tokens, ids.cuda().long(), pairs, 777, 300)
     with pytest.raises(ops.KernelError):
         ops.feed_tokens(d_tokens, ids.cuda(), pairs, 778, 300)
+
+
+@pytest.mark.parametrize("T,E,k,I,H", [(40, 4, 2, 64, 128), (100, 4, 2, 128, 192), (24, 6, 3, 64, 64)])
+def test_sorted_experts_through_either_product(T, E, k, I, H):
+    """rows sorted by expert, more than four an expert: the tiled product takes them by itself; the product for few
+    rows, told to (it takes up to 64 rows an expert), gives the same activations and outputs up to rounding, and
+    both agree with per-token loops"""
+    from ferrox_amd import debug, ops
+    dtype = torch.bfloat16
+    x = rnd(T, H, dtype=dtype)
+    w_gu, w_dn = rnd(E, 2 * I, H, dtype=dtype, seed=1, scale=0.3), rnd(E, H, I, dtype=dtype, seed=2, scale=0.3)
+    g = torch.Generator().manual_seed(7)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
+    xd, gud, dnd = x.double().cpu(), w_gu.double().cpu(), w_dn.double().cpu()
+    ref = torch.zeros(T * k, H, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            a = (plain.silu(xd[t] @ gud[e, :I].T) * (xd[t] @ gud[e, I:].T)).to(torch.bfloat16).double()
+            ref[t * k + j] = a @ dnd[e].T
+    outs = []
+    for few in (4, 64):
+        with debug.kernel_switch("gemm", "few_rows", few):
+            act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+            y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
+        close(y, ref, dtype, f"sorted experts, few_rows {few}", k=I)
+        outs.append(y)
+    assert float((outs[0] - outs[1]).abs().max()) <= 2e-2 * float(ref.abs().max())
