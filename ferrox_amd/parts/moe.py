@@ -17,6 +17,8 @@ from .linear import matmul, same_dtype
 from .mlp import SwiGLU
 
 GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
+PIECES_MAX_PAIRS = 1024      # up to so many (token, slot) pairs the shared expert's pieces run as experts that every token takes
+                             # (measured at both models' sizes: ahead up to here, behind from 1,536 pairs on)
 OVERLAP_MAX_TOKENS = 8192    # up to here the shared expert runs beside the routed ones on a second stream
 _side_streams: dict = {}
 
@@ -169,6 +171,23 @@ class SparseMoE(FeedForward):
                          w_kblocked=self.kblocked)
             debug.region("combine")
             ctx.carry = ops.moe_combine(residual, y[:n], None, weights, self.top_k, shared=y[n:].view(S, T, -1), gate=gate, **then)
+            return
+        if (routed is None and self.shared_pieces and 64 < T and T * self.top_k <= PIECES_MAX_PAIRS and self.kblocked
+                and x.dtype == self.w_gate_up_all.dtype):
+            # A step of a few hundred tokens: the shared expert's pieces ride along behind the sorted pairs as they
+            # do for up to 64 tokens.  Its own two products would run on tiles too few for the GPU (its down
+            # product's 2,048 weight rows give 16 tiles of 128 columns) beside launches that the host cannot
+            # issue faster than the GPU runs them.
+            debug.region("router")
+            if self.router.shape[0] <= 64 and self.router.dtype == x.dtype:      # (as below: the router's rows as the short side)
+                logits = ops.gemm(self.router, x, epilogue=ops.EPI_STORE_F32).t()
+            else:
+                logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
+            ids, weights, gate = ops.router_select(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
+                                                   self.has_shared_gate)
+            S = self.shared_pieces
+            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts, always=S),
+                         then_norm=then_norm, sorted_pieces=S)
             return
         overlap = self.shared is not None and T <= OVERLAP_MAX_TOKENS
         if overlap:
