@@ -36,7 +36,7 @@ def _p(t):
         return None
     if not t.is_cuda:
         raise KernelError("kernel called with a tensor that is not on the GPU")
-    return c_void_p(t.data_ptr())
+    return t.data_ptr()           # (a plain integer: ctypes turns it into the pointer argument itself)
 
 
 # the current stream's handle, asked for before every launch: straight from the runtime's binding where this torch
@@ -47,8 +47,8 @@ _device_index = getattr(torch._C, "_cuda_getDevice", None)
 
 def _stream():
     if _raw_stream is not None and _device_index is not None:
-        return c_void_p(_raw_stream(_device_index()))
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(_device_index())
+    return torch.cuda.current_stream().cuda_stream
 
 
 _sigs = {
