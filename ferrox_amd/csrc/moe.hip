@@ -72,7 +72,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
             wsum += best;
         }
         if (lane < k) {
-            ids[t * k + lane] = my_id;
+            store_shared(ids + t * k + lane, my_id);      // (at device scope: a block of this launch may sort them)
             if (ids_copy) ids_copy[t * k + lane] = my_id;
             weights[t * k + lane] = renorm ? my_w / wsum : my_w;
         }
@@ -119,7 +119,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         }
         if (lane == j) my_w = best;
         if (lane == 0) {
-            ids[t * k + j] = bi;
+            store_shared(ids + t * k + j, bi);
             if (ids_copy) ids_copy[t * k + j] = bi;
             score[bi] = -2.f;  // scores are >= 0; taken out of the race
         }
@@ -184,6 +184,7 @@ __device__ __forceinline__ unsigned long long same_expert_lanes(int e, int bits)
 
 // the sort itself, by one block of whole waves; `offs` (E+1 ints) and `cnt` (rows*E ints) are LDS;
 // a row is `per_row` consecutive groups, rows = ceil(ceil(n/64) / per_row)
+template <bool SHARED_IDS = false>       // SHARED_IDS: other blocks of this launch wrote the ids with store_shared()
 __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E, int per_row, int* offs, int* cnt,
                                             int* __restrict__ expert_offsets, int* __restrict__ sorted_token,
                                             int* __restrict__ sorted_pair, int* __restrict__ inv) {
@@ -196,7 +197,7 @@ __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E,
     for (int r = wave; r < R; r += n_waves) {          // a row belongs to one wave, its groups in order
         for (int g = r * per_row; g < min(G, (r + 1) * per_row); ++g) {
             const int i = g * 64 + lane;
-            int e = i < n ? ids[i] : -1;
+            int e = i < n ? (SHARED_IDS ? load_shared(ids + i) : ids[i]) : -1;
             if (e >= E) e = -1;
             const unsigned long long same = same_expert_lanes(e, bits);
             if (e >= 0 && lane == __ffsll((long long)same) - 1) cnt[r * E + e] += __popcll(same);
@@ -241,7 +242,7 @@ __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E,
     for (int r = wave; r < R; r += n_waves) {
         for (int g = r * per_row; g < min(G, (r + 1) * per_row); ++g) {
             const int i = g * 64 + lane;
-            int e = i < n ? ids[i] : -1;
+            int e = i < n ? (SHARED_IDS ? load_shared(ids + i) : ids[i]) : -1;
             if (e >= E) e = -1;
             const unsigned long long same = same_expert_lanes(e, bits);
             int before = 0;
@@ -271,6 +272,16 @@ static int align_groups_per_row(long n, int E, size_t bytes, size_t* shm) {
     return (int)per_row;
 }
 
+__device__ __forceinline__ void align_always(int n, int k, int E, int* __restrict__ expert_offsets,
+                                             int* __restrict__ sorted_token, int* __restrict__ sorted_pair, int n_always) {
+    const int T = n / k;
+    for (int i = threadIdx.x; i < n_always * T; i += blockDim.x) {
+        sorted_token[n + i] = i % T;
+        if (sorted_pair) sorted_pair[n + i] = n + i;
+    }
+    for (int s = threadIdx.x; s < n_always; s += blockDim.x) expert_offsets[E + 1 + s] = n + (s + 1) * T;
+}
+
 // After the experts, `n_always` further ones that each of the n / k tokens takes (a shared expert cut into pieces):
 // piece s owns the sorted rows n + s T .. n + (s + 1) T, row n + s T + t being token t, and its output row has the
 // same number.
@@ -280,12 +291,7 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
                                                         int* __restrict__ inv, int n_always) {
     extern __shared__ int lds[];
     align_block(ids, n, k, E, per_row, lds, lds + E + 1, expert_offsets, sorted_token, sorted_pair, inv);
-    const int T = n / k;
-    for (int i = threadIdx.x; i < n_always * T; i += blockDim.x) {
-        sorted_token[n + i] = i % T;
-        if (sorted_pair) sorted_pair[n + i] = n + i;
-    }
-    for (int s = threadIdx.x; s < n_always; s += blockDim.x) expert_offsets[E + 1 + s] = n + (s + 1) * T;
+    align_always(n, k, E, expert_offsets, sorted_token, sorted_pair, n_always);
 }
 
 // Many pairs: the same sort by many blocks, in two launches.  First every wave counts the experts of its
@@ -440,8 +446,9 @@ __device__ __forceinline__ float dot8(uint4 w, const float* x) {
 __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
     const float* __restrict__ h, long ldh, const void* __restrict__ gamma, int gamma_dtype, float eps,
     bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm,
-    int gating, float* logits, int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ gate_out,
-    unsigned* counters) {
+    int gating, float* logits, int* ids, float* __restrict__ weights, float* __restrict__ gate_out,
+    unsigned* counters, int* __restrict__ expert_offsets, int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
+    int* __restrict__ inv, int n_always, int per_row) {
     extern __shared__ int lds[];
     __shared__ float red[FRONT_WAVES];
     float* xs = (float*)lds;            // H: the normed row as the experts will read it
@@ -545,15 +552,23 @@ __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
         __builtin_amdgcn_wave_barrier();
         select_token(mine, mine + n_rows, t, E, k, renorm, gating, ids, weights, has_gate ? gate_out : nullptr, nullptr);
     }
+    // with a place for the sorted layout: the block that selects the last token sorts all pairs by expert
+    if (!expert_offsets) return;
+    if (!last_block_arrives(counters + T, T)) return;
+    align_block<true>(ids, T * k, k, E, per_row, lds, lds + E + 1, expert_offsets, sorted_token, sorted_pair, inv);
+    align_always(T * k, k, E, expert_offsets, sorted_token, sorted_pair, n_always);
 }
 
 // Returns 2 (and launches nothing) for sizes this kernel does not take; the caller then runs the
 // norm, the router product and the two routing kernels one after the other.  `logits` holds
-// T x (E + has_gate) floats; `counters` are T zeroed unsigned in device memory, left at zero, that
-// launches on one stream may share.
+// T x (E + has_gate) floats; `counters` are T + 1 zeroed unsigned in device memory, left at zero, that
+// launches on one stream may share.  With `expert_offsets` (E + 1 + n_always ints), `sorted_token`, `sorted_pair`
+// (T k + n_always T ints) and `inv` (T k, or null) the same launch also sorts the pairs by expert, as
+// fx_moe_align does.
 FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamma, int gamma_dtype, float eps,
                         void* x_out, const void* W, int H, int T, int E, int has_gate, int k, int renorm, int gating,
-                        float* logits, int* ids, float* weights, float* gate_out, unsigned* counters) {
+                        float* logits, int* ids, float* weights, float* gate_out, unsigned* counters,
+                        int* expert_offsets, int* sorted_token, int* sorted_pair, int* inv, int n_always) {
     FX_REQUIRE(T >= 0 && H > 0, "moe_front: bad sizes T=%d H=%d", T, H);
     FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
     FX_REQUIRE(k >= 1 && k <= E && k <= K_MAX, "router: top-k %d must lie in 1..min(E, %d)", k, K_MAX);
@@ -562,13 +577,21 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
     FX_REQUIRE(ldh >= H, "moe_front: rows of %ld hold fewer than %d columns", ldh, H);
     FX_REQUIRE(!has_gate || gate_out, "moe_front: a gate row needs a place for its output");
     const size_t front = (size_t)H * 4, back = (size_t)(2 * E + 1) * 4;
-    const size_t shm = front > back ? front : back;
+    size_t shm = front > back ? front : back, sort = 0;
+    int per_row = 1;
+    if (expert_offsets) {       // the sort's counters share the block's LDS
+        FX_REQUIRE(sorted_token && n_always >= 0, "moe_front: the sorted layout needs its arrays");
+        per_row = align_groups_per_row((long)T * k, E, 40 * 1024, &sort);
+        if (sort > shm) shm = sort;
+    }
     if (T > 64 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
     dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
     moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out,
                                                                         (const bf16*)W, H, T, E, has_gate, k, renorm,
-                                                                        gating, logits, ids, weights, gate_out, counters);
+                                                                        gating, logits, ids, weights, gate_out, counters,
+                                                                        expert_offsets, sorted_token, sorted_pair, inv,
+                                                                        n_always, per_row);
     FX_CHECK_LAUNCH("moe_front");
     return 0;
 }

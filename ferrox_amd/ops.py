@@ -82,7 +82,7 @@ _sigs = {
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
-                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 5,
+                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 9 + [c_int],
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
@@ -499,10 +499,12 @@ def _counter(device, n: int = 1) -> torch.Tensor:
     return held[-1]
 
 
-def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False,
+              align: int | None = None):
     """For up to 64 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
     products and selection.  Returns None for sizes the kernel does not take, else
-    (x, ids, weights, gate)."""
+    (x, ids, weights, gate, aligned).  `align` = S asks the same launch for what `moe_align(ids, n_experts,
+    always=S)` returns (its last block sorts the pairs): `aligned`, else None."""
     T, H = h.shape
     if (T > 64 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
             or not router.is_contiguous() or router.shape != (n_experts + (1 if has_gate else 0), H)
@@ -514,15 +516,22 @@ def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE
     weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
     gate = torch.empty((T,), dtype=torch.float32, device=dev) if has_gate else None
     logits = torch.empty((T, router.shape[0]), dtype=torch.float32, device=dev)
+    offsets = buf = None
+    if align is not None:
+        offsets = torch.empty((n_experts + 1 + align,), dtype=torch.int32, device=dev)
+        buf = torch.empty((3, T * top_k + align * T), dtype=torch.int32, device=dev)
     f, handle = _fn("moe", "fx_moe_front")
     rc = f(_stream(), _p(h), h.stride(0), _p(norm_weight), dtype_code(norm_weight.dtype), float(eps), _p(x), _p(router),
            H, T, n_experts, 1 if has_gate else 0, top_k, 1 if renorm else 0, gating, _p(logits), _p(ids), _p(weights),
-           _p(gate), _p(_counter(dev, T)))
+           _p(gate), _p(_counter(dev, T + 1)), _p(offsets), _p(buf[0]) if buf is not None else None,
+           _p(buf[1]) if buf is not None else None, _p(buf[2]) if buf is not None else None, int(align or 0))
+    if rc == 2 and align is not None:      # the sort's counters do not fit beside the front's: without it
+        return moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating, has_gate)
     if rc == 2:
         return None
     if rc:
         raise KernelError(handle.fx_last_error().decode())
-    return x, ids, weights, gate
+    return x, ids, weights, gate, (offsets, buf[0], buf[1], buf[2]) if buf is not None else None
 
 
 def moe_align(ids: torch.Tensor, n_experts: int, always: int = 0):

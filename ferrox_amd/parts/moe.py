@@ -122,19 +122,22 @@ class SparseMoE(FeedForward):
         if T > 64 or ctx.act_dtype != torch.bfloat16 or rms is None:
             return False
         debug.region("router")
+        rows_ok = self.hidden_size % 8 == 0 and self.expert_intermediate_size % 8 == 0
+        unsorted = T <= 16 and T * self.top_k <= 64 and rows_ok       # the expert products take the pairs unsorted
+        # otherwise the shared expert's pieces ride along as experts that every token takes, behind the sorted
+        # pairs, and the launch that selects the experts also sorts the pairs by expert
+        S = self.shared_pieces if ctx.act_dtype == self.w_gate_up_all.dtype and T * self.top_k <= 2048 else 0
         front = ops.moe_front(residual, rms[0], rms[1], self.router, self.n_experts, self.top_k,
-                              self.norm_topk_prob, self.gating, self.has_shared_gate)
+                              self.norm_topk_prob, self.gating, self.has_shared_gate, align=None if unsorted else S)
         if front is None:
             return False
-        x, ids, weights, gate = front
-        aligned = self.hidden_size % 8 == 0 and self.expert_intermediate_size % 8 == 0
-        if T <= 16 and ids.numel() <= 64 and aligned:       # the expert products take the pairs unsorted
+        x, ids, weights, gate, sort = front
+        if unsorted:
             self.forward(x, ctx, residual, routed=(ids, weights, gate, None, None, None, None), then_norm=then_norm)
         else:
-            # the shared expert's pieces ride along as experts that every token takes, behind the sorted pairs
-            S = self.shared_pieces if x.dtype == self.w_gate_up_all.dtype and ids.numel() <= 2048 else 0
-            self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts, always=S),
-                         then_norm=then_norm, sorted_pieces=S)
+            if sort is None:
+                sort = ops.moe_align(ids, self.n_experts, always=S)
+            self.forward(x, ctx, residual, routed=(ids, weights, gate) + sort, then_norm=then_norm, sorted_pieces=S)
         return True
 
     def forward(self, x, ctx, residual, routed=None, then_norm=None, sorted_pieces: int = 0) -> None:

@@ -686,10 +686,16 @@ def test_moe_front(T, H, E, k, renorm, has_gate):
     router = rnd(E + (1 if has_gate else 0), H, dtype=torch.bfloat16, seed=4, scale=0.3)
     eps = 1e-5
     x_sep = ops.rmsnorm(h.contiguous(), gamma, eps, torch.bfloat16)
-    for rep in range(2):
-        got = ops.moe_front(h, gamma, eps, router, E, k, renorm, has_gate=has_gate)
+    for rep in range(3):
+        # the third time with the sort by expert in the same launch, and two pieces behind the experts
+        got = ops.moe_front(h, gamma, eps, router, E, k, renorm, has_gate=has_gate, align=2 if rep == 2 else None)
         assert got is not None
-        x, ids, w, gate = got
+        x, ids, w, gate, sort = got
+        assert (sort is None) == (rep < 2)
+        if sort is not None:
+            for i, (mine, theirs) in enumerate(zip(sort, ops.moe_align(ids, E, always=2))):
+                n_set = T * k if i == 3 else mine.numel()           # the inverse map covers the pairs only
+                assert torch.equal(mine[:n_set], theirs[:n_set]), "the launch's own sort is that of moe_align"
         # the same formula as the norm kernel: at most the last float32 bit differs, which moves a
         # bfloat16 result only where it stands on a rounding boundary
         differ = x != x_sep
