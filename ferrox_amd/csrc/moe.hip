@@ -443,6 +443,7 @@ __device__ __forceinline__ float dot8(uint4 w, const float* x) {
     return a;
 }
 
+#define FRONT_MAX_TOKENS 256
 __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
     const float* __restrict__ h, long ldh, const void* __restrict__ gamma, int gamma_dtype, float eps,
     bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm,
@@ -584,7 +585,7 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
         per_row = align_groups_per_row((long)T * k, E, 40 * 1024, &sort);
         if (sort > shm) shm = sort;
     }
-    if (T > 64 || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
+    if (T > FRONT_MAX_TOKENS || H % 8 != 0 || ((uintptr_t)W % 16) != 0 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
     dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
     moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out,

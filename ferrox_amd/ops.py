@@ -501,12 +501,12 @@ def _counter(device, n: int = 1) -> torch.Tensor:
 
 def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False,
               align: int | None = None):
-    """For up to 64 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
+    """For up to 256 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
     products and selection.  Returns None for sizes the kernel does not take, else
     (x, ids, weights, gate, aligned).  `align` = S asks the same launch for what `moe_align(ids, n_experts,
     always=S)` returns (its last block sorts the pairs): `aligned`, else None."""
     T, H = h.shape
-    if (T > 64 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
+    if (T > 256 or h.dtype != torch.float32 or h.stride(1) != 1 or router.dtype != torch.bfloat16
             or not router.is_contiguous() or router.shape != (n_experts + (1 if has_gate else 0), H)
             or norm_weight.numel() != H):
         return None

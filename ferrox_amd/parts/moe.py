@@ -17,6 +17,8 @@ from .linear import matmul, same_dtype
 from .mlp import SwiGLU
 
 GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
+FRONT_MAX_TOKENS = 128       # up to so many tokens the norm, the router, the selection and the sort are one launch (the
+                             # kernel takes 256; from 192 on its blocks, which all read the router's rows, fall behind)
 PIECES_MAX_PAIRS = 1024      # up to so many (token, slot) pairs the shared expert's pieces run as experts that every token takes
                              # (measured at both models' sizes: ahead up to here, behind from 1,536 pairs on)
 OVERLAP_MAX_TOKENS = 8192    # up to here the shared expert runs beside the routed ones on a second stream
@@ -115,12 +117,15 @@ class SparseMoE(FeedForward):
         return {}
 
     def forward_from_residual(self, norm, ctx, residual, then_norm=None) -> bool:
-        """Few tokens: the norm and the router are one launch, and the expert products group the
-        (token, slot) pairs themselves instead of reading a sorted layout."""
+        """Few tokens: the norm and the router are one launch; up to 16 tokens the expert products group the
+        (token, slot) pairs themselves instead of reading a sorted layout, for more that launch also sorts them."""
         T = residual.shape[0]
         rms = norm.rms_params()
-        if T > 64 or ctx.act_dtype != torch.bfloat16 or rms is None:
+        if T > FRONT_MAX_TOKENS or ctx.act_dtype != torch.bfloat16 or rms is None:
             return False
+        if T > 64 and not (self.shared_pieces and T * self.top_k <= PIECES_MAX_PAIRS and self.kblocked
+                           and ctx.act_dtype == self.w_gate_up_all.dtype):
+            return False        # (more than 64 tokens: only where the shared expert's pieces ride along, see forward)
         debug.region("router")
         rows_ok = self.hidden_size % 8 == 0 and self.expert_intermediate_size % 8 == 0
         unsorted = T <= 16 and T * self.top_k <= 64 and rows_ok       # the expert products take the pairs unsorted

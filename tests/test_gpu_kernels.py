@@ -676,7 +676,8 @@ def test_gemm_with_fused_norm(M, N, K, gamma_dtype):
 @pytest.mark.parametrize("T,H,E,k,renorm,has_gate", [(1, 2048, 60, 4, False, True), (8, 2048, 60, 4, False, True),
                                                       (16, 264, 7, 3, True, False), (5, 1792, 130, 8, True, True), (16, 2048, 60, 4, False, True),
                                                       (64, 2048, 60, 4, False, True), (33, 96, 6, 3, True, True),
-                                                      (3, 64, 4, 4, False, True)])
+                                                      (3, 64, 4, 4, False, True), (130, 1792, 60, 4, False, True),
+                                                      (256, 264, 64, 8, True, True)])
 def test_moe_front(T, H, E, k, renorm, has_gate):
     """norm + router products + selection + sort in one launch, twice in a row (the kernel's counter
     must be back at zero), against the plain norm and router on the rounded activations"""
@@ -711,7 +712,7 @@ def test_moe_front(T, H, E, k, renorm, has_gate):
         if has_gate:
             close(gate, torch.sigmoid(logits[E]), torch.float32, "shared gate")
     assert int(ops._counter(DEV).abs().sum()) == 0
-    assert ops.moe_front(rnd(65, H), gamma, eps, router, E, k, renorm, has_gate=has_gate) is None     # too many rows
+    assert ops.moe_front(rnd(257, H), gamma, eps, router, E, k, renorm, has_gate=has_gate) is None     # too many rows
 
 
 @pytest.mark.parametrize("T,E,k", [(5000, 60, 4), (3000, 700, 2), (1, 3, 1), (130, 1, 1), (2048, 60, 4), (701, 7, 3), (683, 5, 3)])
