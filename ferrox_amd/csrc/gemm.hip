@@ -1128,6 +1128,7 @@ static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per 
 static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
 static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
 static int g_few_rows = 4;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
+static int g_head_rows = 8;    // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
 static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
@@ -1135,8 +1136,9 @@ FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "skinny_row_tiles")) { g_skinny_mt = value; return 0; }
     if (!strcmp(key, "skinny_waves")) { g_skinny_waves = value; return 0; }
     if (!strcmp(key, "few_rows")) { g_few_rows = value < 0 ? 0 : (value > 64 ? 64 : value); return 0; }
+    if (!strcmp(key, "head_rows")) { g_head_rows = value; return 0; }
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
-    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, wide)", key);
+    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, head_rows, wide)", key);
     return 1;
 }
 
@@ -1308,9 +1310,10 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
     const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
     FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
-    // 33..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights faster
-    // than four row tiles per block of the kernel for few rows
-    const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > 32 && K % 64 == 0 &&
+    // 9..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights at the same
+    // speed whatever the rows (151,936 weight rows: 131-136 us from 1 to 33 rows), the kernel for few rows slows
+    // down with them (108 us at 1 row, 134 at 8, 150 at 16, 182 at 32)
+    const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > g_head_rows && K % 64 == 0 &&
                               !g_no_wide && ceil_div(N, 128) >= 512;
     // Rows sorted by expert: the product for few rows only up to four rows an expert on average.  Its waves fetch
     // every row tile's operands themselves, so its time grows with the rows (512 tokens of the larger model, 64 rows
