@@ -514,10 +514,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     const int na = (nblk - wm + 1) >> 1;         // this wave's active row blocks
 #define FX_LOOP(NA) \
     wide_k_loop<NA, MT, NT, TM, TN, NSA, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride)
-    if (na > 3 * MT / 4) FX_LOOP(MT);
-    else if (na > MT / 2) FX_LOOP(3 * MT / 4);
-    else if (na > MT / 4) FX_LOOP(MT / 2);
-    else FX_LOOP(MT / 4);
+    if constexpr (MT >= 4) {
+        if (na > 3 * MT / 4) FX_LOOP(MT);
+        else if (na > MT / 2) FX_LOOP(3 * MT / 4);
+        else if (na > MT / 4) FX_LOOP(MT / 2);
+        else FX_LOOP(MT / 4);
+    } else {
+        if (na > MT / 2) FX_LOOP(MT);
+        else FX_LOOP((MT + 1) / 2);
+    }
 #undef FX_LOOP
 
     // epilogue: lane holds rows 4*(lane/16)+r, column lane%16 of each 16x16 tile
@@ -1129,13 +1134,15 @@ static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows
 static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
 static int g_few_rows = 4;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
 static int g_head_rows = 8;    // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
+static int g_tile64_rows = 20; // "tile64_rows": experts with up to this many rows on average take tiles of 64 rows
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
-static int g_wide_force = 0;   //         256, 192, 128, 64 or 12 picks that tile of the LDS-tiled kernel
+static int g_wide_force = 0;   //         256, 192, 128, 64, 12 or 4 (tiles of 64 rows) picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "skinny_sets")) { g_skinny_nw = value; return 0; }
     if (!strcmp(key, "skinny_row_tiles")) { g_skinny_mt = value; return 0; }
     if (!strcmp(key, "skinny_waves")) { g_skinny_waves = value; return 0; }
     if (!strcmp(key, "few_rows")) { g_few_rows = value < 0 ? 0 : (value > 64 ? 64 : value); return 0; }
+    if (!strcmp(key, "tile64_rows")) { g_tile64_rows = value; return 0; }
     if (!strcmp(key, "head_rows")) { g_head_rows = value; return 0; }
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
     FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, head_rows, wide)", key);
@@ -1382,7 +1389,13 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         const double s12 = expert_offsets ? 0.0 : score(192, 256, 0.92);
         const bool few_rows = g_wide_force ? g_wide_force == 12
                                            : (expert_offsets ? per_group <= 176 : (s12 > s256 && s12 > s192 && s12 > s128 && s12 > s64));
-        if (few_rows)
+        // an expert's share of up to 20 rows on average: a tile of 64 rows leaves LDS for a ring of four weight tiles
+        // beside two of the rows (2-5 % less time than tiles of 192 rows with a ring of three, the same bits: decode
+        // at 64 sequences 11.2 -> 11.0 ms, a 192-token step 6.8 -> 6.4 ms; from 25 rows on average on, steps of 384
+        // tokens, more and more experts need a second tile and it falls behind)
+        if (g_wide_force == 4 || (!g_wide_force && expert_offsets && per_group <= g_tile64_rows))
+            launch_wide<4, 256, 4, 2>(g, epi, M / 64 + (expert_offsets ? nonempty : (M % 64 != 0)), s);
+        else if (few_rows)
             launch_wide<12, 256, 3, 2>(g, epi, M / 192 + (expert_offsets ? nonempty : (M % 192 != 0)), s);
         else if (s192 > s256 && s192 >= s128 && s192 >= s64)
             launch_wide<16, 192, 2>(g, epi, M / 256 + (expert_offsets ? nonempty : (M % 256 != 0)), s);

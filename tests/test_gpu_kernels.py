@@ -97,7 +97,7 @@ def test_combine_of_many_rows_equals_that_of_few(T, H, k, S, sorted_rows):
     close(h_all, want, torch.float32, "combined rows")
 
 
-@pytest.mark.parametrize("tile", [256, 192, 128, 64, 12])      # 12: tiles of 192 rows x 256 weight rows
+@pytest.mark.parametrize("tile", [256, 192, 128, 64, 12, 4])      # 12, 4: tiles of 192 and of 64 rows x 256 weight rows
 @pytest.mark.parametrize("M,N,K", [(300, 400, 192), (513, 200, 64), (70, 520, 448)])
 def test_gemm_every_wide_tile(tile, M, N, K):
     """The many-row kernel picks its tile by the sizes; here each tile shape is made to run the same products."""
@@ -117,9 +117,10 @@ def test_gemm_every_wide_tile(tile, M, N, K):
     close(act, plain.silu(a.double() @ w2[:N].double().T) * (a.double() @ w2[N:].double().T), dtype, "silu(gate)*up")
 
 
-@pytest.mark.parametrize("tile", [12, 256])
+@pytest.mark.parametrize("tile", [12, 256, 4])
 def test_grouped_gemm_tiles_agree(tile):
-    """An expert's rows in tiles of 192 (weights three steps deep) and of 256 give the same sums."""
+    """An expert's rows in tiles of 192 (weights three steps deep), of 256 and of 64 (weights four steps deep) give
+    the same sums."""
     from ferrox_amd import debug, ops
     T, E, k, I, H = 900, 6, 2, 64, 256
     x = rnd(T, H, dtype=torch.bfloat16)
