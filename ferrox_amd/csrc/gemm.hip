@@ -1132,7 +1132,7 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
 static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per wave of the product for few rows (0: by the sizes)
 static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
 static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
-static int g_few_rows = 4;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
+static int g_few_rows = 3;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
 static int g_head_rows = 8;    // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
 static int g_tile64_rows = 20; // "tile64_rows": experts with up to this many rows on average take tiles of 64 rows
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
@@ -1322,12 +1322,12 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     // down with them (108 us at 1 row, 134 at 8, 150 at 16, 182 at 32)
     const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > g_head_rows && K % 64 == 0 &&
                               !g_no_wide && ceil_div(N, 128) >= 512;
-    // Rows sorted by expert: the product for few rows only up to four rows an expert on average.  Its waves fetch
+    // Rows sorted by expert: the product for few rows only up to three rows an expert on average.  Its waves fetch
     // every row tile's operands themselves, so its time grows with the rows (512 tokens of the larger model, 64 rows
     // an expert: 1,107 us for the gate/up product at 2.1 TB/s), while the tiled product, whose tile of 192 rows
     // holds an expert's share, streams the weights at the same speed whatever the rows (400 us at 5.9 TB/s); decode
     // steps of 48 and 64 sequences 10.3 -> 10.0 and 12.0 -> 11.4 ms, of 17 to 64 of the larger model's sizes 8-24 %
-    // less, and with three or four rows an expert the product for few rows is still 2-6 % ahead.
+    // less; with three rows an expert the product for few rows is still 1-2 % ahead of the tiles of 64 rows.
     const long few_limit = expert_offsets && wide_ok ? g_few_rows : 64;
     if (g.vec_ok && (per_group <= few_limit || pair_ids) && !many_columns) {
         int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
