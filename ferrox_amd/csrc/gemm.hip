@@ -1377,7 +1377,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
             const double rows = expert_offsets ? 1.0 : (double)M / (double)((long)ceil_div(M, tm) * tm);
             return quality * rows * (double)t / (double)(ceil_div(t, 256) * 256L);
         };
-        double s256 = score(256, 256, 1.0), s192 = dual ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
+        double s256 = score(256, 256, 1.0), s192 = dual || expert_offsets ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
                s64 = score(128, 128, 0.7);
         if (g_wide_force) {
             s256 = g_wide_force == 256; s192 = g_wide_force == 192 && !dual; s128 = g_wide_force == 128; s64 = 0.5 * (g_wide_force == 64);
@@ -1387,8 +1387,13 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         // plain rows: tiles of 192 x 256 where they divide the work more evenly (2,048 rows against 11,264 weight
         // rows: 484 tiles for two rounds of the 256 CUs instead of 352 tiles of 256 x 256)
         const double s12 = expert_offsets ? 0.0 : score(192, 256, 0.92);
+        // (an expert's share beyond 192 rows: tiles of 192 rows too where they leave fewer empty rows than tiles of
+        // 256 do, 273 rows an expert as 2 x 192 instead of 2 x 256: the down product of a 4,096-token step 173
+        // against 190 us)
+        const long pad192 = ceil_div(per_group, 192) * 192L, pad256 = ceil_div(per_group, 256) * 256L;
         const bool few_rows = g_wide_force ? g_wide_force == 12
-                                           : (expert_offsets ? per_group <= 176 : (s12 > s256 && s12 > s192 && s12 > s128 && s12 > s64));
+                                           : (expert_offsets ? (per_group <= 176 || pad192 < pad256)
+                                                             : (s12 > s256 && s12 > s192 && s12 > s128 && s12 > s64));
         // an expert's share of up to 20 rows on average: a tile of 64 rows leaves LDS for a ring of four weight tiles
         // beside two of the rows (2-5 % less time than tiles of 192 rows with a ring of three, the same bits: decode
         // at 64 sequences 11.2 -> 11.0 ms, a 192-token step 6.8 -> 6.4 ms; from 25 rows on average on, steps of 384
