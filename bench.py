@@ -11,7 +11,9 @@ N(0, 0.02) made on the GPU, seeded random token ids.  A "step" is one decode
 step of the whole batch through the engine's own step function and sampling
 kernel (greedy).  Default: batch 8, 2,048-token prompts prefilled through the
 same step function, then W untimed and K timed decode steps (timed in three
-consecutive parts, whose spread is reported beside the whole).  The line also
+consecutive parts, whose spread is reported beside the whole), driven as the
+engine generates: the host a step ahead, a step launched with the ids of the
+step before it still on the device, every id read by the host one step late.  The line also
 carries: a 2,048-token prefill (one discarded run, median of three); decode at
 batch 1 and 64; the decode step's memory roofline for all three batch sizes:
 bytes it has to read (every weight it uses once, the distinct experts counted
@@ -19,8 +21,8 @@ from the router's own choices in an untimed step, plus the cache of the live
 requests) / time, against the published 8 TB/s; the ceilings measured on this
 GPU by the simplest kernels (a streaming read, a copy, a loop of MFMA
 products); and the same batch served through `Engine.generate` (scheduler,
-sampling, ids read back each step), with the share of the time that the GPU
-waited for the host.
+sampling, ids read back), with the share of the time that the GPU waited for
+the host.
 (The reference measures pp<N> / tg<N> the same way on synthetic ids with one
 discarded warm-up and the median of three runs, ferrox-cli/src/bench_model.rs:35-60, 239-302.)
 """
