@@ -1,3 +1,3 @@
-from .sampler import SamplingParams, XorShift64, sample_rows
+from .sampler import SamplingParams, XorShift64, launch_sample_rows, sample_rows
 
-__all__ = ["SamplingParams", "XorShift64", "sample_rows"]
+__all__ = ["SamplingParams", "XorShift64", "launch_sample_rows", "sample_rows"]
