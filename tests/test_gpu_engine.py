@@ -645,3 +645,38 @@ def test_reading_ids_one_step_late_generates_the_same(model_folders):
         outcomes[late] = [(c.token_ids, c.finish_reason) for c in drawn]
         assert engine.runner.manager.n_free_pages() == 30
     assert outcomes[True] == outcomes[False]
+
+
+@pytest.mark.parametrize("trial", range(4))
+def test_random_workloads_generate_the_same_with_ids_read_late_or_at_once(model_folders, trial):
+    """requests of random lengths, token limits and sampling parameters (some greedy, some drawing, some with a
+    repetition penalty) through engines of random pool sizes, budgets and portions, with an EOS that many of them
+    reach: the generation loop that reads a step's ids one step late gives what the loop that reads them at once
+    gives, token for token and reason for reason, and no page is lost"""
+    import random
+    from conftest import TINY
+    from ferrox_amd.engine.api import Engine
+    from ferrox_amd.sampling import SamplingParams
+    name = "AB"[trial % 2]
+    cfg = TINY[name][0]
+    folder = model_folders(name, "float32")
+    rnd = random.Random(4000 + trial)
+    n, V, ctx = rnd.randint(5, 30), cfg["vocab_size"], cfg["max_position_embeddings"]
+    prompts = [[rnd.randrange(V) for _ in range(rnd.randint(1, min(120, ctx - 2)))] for _ in range(n)]
+    new = [rnd.randint(1, 30) for _ in range(n)]
+    params = [SamplingParams(temperature=rnd.choice([0.0, 0.0, 0.8]), seed=rnd.randrange(1 << 30),
+                             repetition_penalty=rnd.choice([1.0, 1.0, 1.0, 1.2])) for _ in range(n)]
+    pages = rnd.randint(45, 100)
+    engine = Engine(folder, dtype="float32", block_size=8, num_pages=pages, max_seqs=rnd.randint(3, 16),
+                    max_tokens_per_step=rnd.randint(16, 96), prefill_chunk=rnd.randint(4, 64))
+    free = engine.generate_detailed(prompts, new, params, ignore_eos=True)
+    flat = [t for c in free for t in c.token_ids]
+    eos = max(set(flat), key=flat.count)          # the token generated most often: many requests stop early
+    outcomes = {}
+    for late in (True, False):
+        engine.overlap_steps = late
+        got = engine.generate_detailed(prompts, new, params, eos_token_id=eos)
+        outcomes[late] = [(c.token_ids, c.finish_reason) for c in got]
+        assert engine.runner.manager.n_free_pages() == pages
+    assert outcomes[True] == outcomes[False]
+    assert any(reason == "stop" for _, reason in outcomes[True])
