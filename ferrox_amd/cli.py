@@ -114,15 +114,29 @@ def main(argv=None) -> int:
         params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
                                 args.presence_penalty, args.frequency_penalty, seed)
         t1 = time.time()
-        out = engine.generate_detailed([prompt_ids], args.n_predict, params, ignore_eos=args.ignore_eos)[0]
+        shown = {"ids": [], "text": ""}
+
+        def show(_, token):                 # printed as it is generated (run.rs:651-676)
+            shown["ids"].append(token)
+            if tokenizer is None:
+                sys.stdout.write(("," if len(shown["ids"]) > 1 else "") + str(token))
+            else:
+                text = tokenizer.decode(shown["ids"])
+                if text.endswith("\ufffd"):        # half of a character: wait for the rest
+                    return
+                sys.stdout.write(text[len(shown["text"]):])
+                shown["text"] = text
+            sys.stdout.flush()
+
+        out = engine.generate_detailed([prompt_ids], args.n_predict, params, ignore_eos=args.ignore_eos, on_token=show)[0]
     except (ValueError, OSError, KernelBuildError) as e:     # ConfigError, CheckpointError, SafetensorsError are ValueErrors
         print(f"error: {e}", file=sys.stderr)
         return 2
     dt = time.time() - t1
     if tokenizer is not None:
-        print(tokenizer.decode(out.token_ids))
+        print(tokenizer.decode(out.token_ids)[len(shown["text"]):])
     else:
-        print(",".join(str(t) for t in out.token_ids))
+        print()
     n = len(out.token_ids)
     print(f"prompt {len(prompt_ids)} tokens; predict {n} tokens in {dt:.2f} s, {n / dt if dt > 0 else 0:.1f} t/s; "
           f"finish: {out.finish_reason}", file=sys.stderr)

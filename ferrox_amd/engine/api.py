@@ -83,9 +83,11 @@ class Engine:
             ignore_eos=ignore_eos, eos_token_id=eos_token_id)]
 
     def generate_detailed(self, prompts: list, max_new_tokens, params: SamplingParams | list | None = None,
-                          ignore_eos: bool = False, eos_token_id: int | None = None) -> list:
+                          ignore_eos: bool = False, eos_token_id: int | None = None, on_token=None) -> list:
         """`params` may be one `SamplingParams` for all or one per prompt; `max_new_tokens` likewise.
-        Request i draws from a generator seeded with its own params.seed."""
+        Request i draws from a generator seeded with its own params.seed.  `on_token(i, token)` is called for
+        every token that request i generates, in order, as soon as the host has read it (the reference prints
+        as it generates, ferrox-cli/src/run.rs:651-676)."""
         eos = eos_token_id if eos_token_id is not None else self.eos_token_id
         sched = Scheduler(self.runner, max_tokens_per_step=self.max_tokens_per_step,
                           prefill_chunk=self.prefill_chunk, max_seqs=self.max_seqs,
@@ -108,6 +110,7 @@ class Engine:
         # the step whose sampled ids the host has not read yet: its batch, the requests of the rows, the ids on
         # the device, their copy in pinned memory and the event after that copy
         inflight = None
+        told = [0] * len(reqs)        # how many of each request's tokens `on_token` has been given
 
         def settle() -> bool:
             nonlocal inflight
@@ -117,6 +120,11 @@ class Engine:
             inflight = None
             copied.synchronize()
             sched.resolve(batch, {r.id: t for r, t in zip(rows, host_ids.tolist())})
+            if on_token is not None:
+                for r in rows:           # a request's tokens that became known (an EOS is never among them)
+                    while told[r.id] < len(r.generated) and r.generated[told[r.id]] != UNKNOWN:
+                        on_token(r.id, r.generated[told[r.id]])
+                        told[r.id] += 1
             return True
 
         sched.settle = settle

@@ -639,8 +639,10 @@ def test_reading_ids_one_step_late_generates_the_same(model_folders):
     outcomes = {}
     for late in (True, False):
         engine.overlap_steps = late
-        got = engine.generate_detailed(prompts, 20, eos_token_id=eos)
+        told = [[] for _ in prompts]          # tokens are handed out as the host reads them, each once and in order
+        got = engine.generate_detailed(prompts, 20, eos_token_id=eos, on_token=lambda i, t: told[i].append(t))
         assert [(c.token_ids, c.finish_reason) for c in got] == expect, f"ids read late: {late}"
+        assert told == [c.token_ids for c in got]
         drawn = engine.generate_detailed(prompts, 20, params, eos_token_id=eos)
         outcomes[late] = [(c.token_ids, c.finish_reason) for c in drawn]
         assert engine.runner.manager.n_free_pages() == 30
