@@ -101,8 +101,10 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // ---------------------------------------------------------------------------
 // Rotary position encoding of q and k, and the write of k and v into the pages.
 //
-// Split-half pairing (i, i + rot/2), angle = pos * theta^(-2i/rot)
-// (ferrox-core/src/attention.rs:20-32); `interleaved` pairs (2i, 2i+1) instead.
+// Split-half pairing (i, i + rot/2), angle = (float)pos * inv_freq[i] in float32, as the reference
+// multiplies them (ferrox-core/src/attention.rs:20-32); the caller brings inv_freq[i] = theta^(-2i/rot)
+// as a table of rot/2 floats, so that the frequencies are the same numbers wherever they are made.
+// `interleaved` pairs (2i, 2i+1) instead.
 // `freq_factors` (rot/2 floats, or null): the angle of pair i is divided by freq_factors[i]
 // (per-band frequency correction, attention.rs:319-333).
 // rot = 0 rotates nothing.  v is never rotated.  Key pages hold
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta, int vec8,
+    int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, const float* __restrict__ inv_freq, int vec8,
     const float* __restrict__ freq_factors) {
     __shared__ float cs[128], sn[128];     // rot / 2 <= 128
     const int tid = threadIdx.x;
@@ -128,8 +130,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         const int t = blockIdx.x / split, part = blockIdx.x % split, step = 256 * split;
         const int pos = positions[t];
         for (int p = tid; p < half; p += 256) {
-            const float freq = 1.0f / powf(theta, (float)(2 * p) / (float)rot);
-            float angle = (float)pos * freq;
+            float angle = (float)pos * inv_freq[p];
             if (freq_factors) angle = angle / freq_factors[p];
             sincosf(angle, &sn[p], &cs[p]);
         }
@@ -223,11 +224,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
 FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const void* k, int ldk,
                             const void* v, int ldv, const int* positions, const int* token_seq,
                             const int* block_table, int max_blocks, void* k_pages, void* v_pages,
-                            int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, float theta,
+                            int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, const float* inv_freq,
                             const float* freq_factors) {
     FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
     FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
     FX_REQUIRE(rot <= 256, "rope_kv_write: rotary dim %d is more than this kernel's 256", rot);
+    FX_REQUIRE(inv_freq || rot == 0, "rope_kv_write: a rotation needs the table of its %d frequencies", rot / 2);
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -241,12 +243,12 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
         rope_kv_write_kernel<float><<<blocks, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
                                                            positions, token_seq, block_table, max_blocks,
                                                            (float*)k_pages, (float*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                           interleaved, theta, 0, freq_factors);
+                                                           interleaved, inv_freq, 0, freq_factors);
     else if (dtype == FX_BF16)
         rope_kv_write_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
                                                           positions, token_seq, block_table, max_blocks,
                                                           (bf16*)k_pages, (bf16*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                          interleaved, theta, vec8, freq_factors);
+                                                          interleaved, inv_freq, vec8, freq_factors);
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("rope_kv_write");

@@ -60,7 +60,7 @@ struct GemmArgs {
     void* rope_k_pages;     // null: nothing is written to pages (a layer that reads another's cache)
     void* rope_v_pages;
     int rope_nh, rope_nkv, rope_hd, rope_bs, rope_rot;
-    float rope_theta;
+    const float* rope_inv_freq;       // rot/2 floats: pair i turns by (float)pos * rope_inv_freq[i]
     const float* rope_freq_factors;   // rot/2 floats or null: the angle of pair i is divided by rope_freq_factors[i]
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
@@ -829,14 +829,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         const int bias_dt = g.bias ? g.bias_dtype : FX_F32;
         const RawElement e0 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c0 + cc : 0);
         const RawElement e1 = fetch_element(bias_or, bias_dt, g.bias ? (size_t)rope_head * g.rope_hd + rope_c1 + cc : 0);
+        // the pair's frequency from the table (columns that are not rotated read entry 0 and do not use it)
+        const int p = rope_rotated ? 16 * rope_j + cc : 0;
+        const float freq = g.rope_inv_freq[p];
+        const float freq_div = g.rope_freq_factors ? g.rope_freq_factors[p] : 1.f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
             total[mt] = g.row_ss ? sum_in_order(g.row_ss + (size_t)row_of[mt] * g.row_ss_n, g.row_ss_n) : 0.f;
         rope_b0 = element_as_float(e0);
         rope_b1 = element_as_float(e1);
-        const int p = 16 * rope_j + cc;
-        const float freq = rope_rotated ? 1.0f / powf(g.rope_theta, (float)(2 * p) / (float)g.rope_rot) : 0.f;
-        const float freq_div = rope_rotated && g.rope_freq_factors ? g.rope_freq_factors[p] : 1.f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             rope_page[mt] = 0;
@@ -1225,7 +1226,7 @@ static void launch_skinny(const GemmArgs& g, int epi, int mt, int nw, int waves,
 FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, long kb_rows, const void* bias, int bias_dtype,
                        void* C, long ldc, int M, int K, const float* row_ss, int row_ss_n, float eps,
                        const int* positions, const int* token_seq, const int* table, int max_blocks,
-                       void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, float theta,
+                       void* k_pages, void* v_pages, int nh, int nkv, int hd, int bs, int rot, const float* inv_freq,
                        const float* freq_factors) {
     FX_REQUIRE(M >= 1 && M <= 64 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K, "qkv_rope: 1..64 rows of a multiple of 8 elements");
     FX_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 32 == 0 && rot >= 0 && rot <= hd && rot % 32 == 0 && bs > 0,
@@ -1234,6 +1235,7 @@ FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, lon
     FX_REQUIRE(ldc >= N && (((uintptr_t)A | (uintptr_t)W) % 16) == 0, "qkv_rope: output rows too short or operands not aligned");
     FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "qkv_rope: key and value pages must come together");
     FX_REQUIRE(positions && token_seq && (!k_pages || (table && max_blocks > 0)), "qkv_rope: positions, sequences and block table");
+    FX_REQUIRE(inv_freq || rot == 0, "qkv_rope: a rotation needs the table of its %d frequencies", rot / 2);
     FX_REQUIRE(!bias || bias_dtype == FX_F32 || bias_dtype == FX_BF16, "qkv_rope: unknown bias dtype %d", bias_dtype);
     FX_REQUIRE(kb_rows == 0 || (kb_rows == N && K % 64 == 0), "qkv_rope: weights in slabs of 64 k hold all %d rows", N);
     FX_REQUIRE(!row_ss || row_ss_n >= 1, "qkv_rope: sums of squares without their count");
@@ -1243,7 +1245,8 @@ FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, lon
     g.row_ss = row_ss; g.row_ss_n = row_ss_n; g.norm_eps = eps;
     g.rope_positions = positions; g.rope_token_seq = token_seq; g.rope_table = table; g.rope_max_blocks = max_blocks;
     g.rope_k_pages = k_pages; g.rope_v_pages = v_pages;
-    g.rope_nh = nh; g.rope_nkv = nkv; g.rope_hd = hd; g.rope_bs = bs; g.rope_rot = rot; g.rope_theta = theta;
+    g.rope_nh = nh; g.rope_nkv = nkv; g.rope_hd = hd; g.rope_bs = bs; g.rope_rot = rot;
+    g.rope_inv_freq = inv_freq ? inv_freq : (const float*)positions;      // (rot == 0: read, never used)
     g.rope_freq_factors = freq_factors;
     dim3 grid((nh + 2 * nkv) * (hd / 32), 1);
     if (M <= 16) gemm_bf16_skinny_kernel<1, 4, 2, false, EPI_STORE, false, true><<<grid, 256, 0, (hipStream_t)stream>>>(g);

@@ -50,8 +50,10 @@ def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: floa
     return model
 
 
-def write_random_model(config, folder: str, seed: int, dtype="bfloat16", std: float = 0.02) -> None:
-    """Writes config.json and model.safetensors with the same tensors `random_model` makes."""
+def write_random_model(config, folder: str, seed: int, dtype="bfloat16", std: float = 0.02, device="cpu") -> None:
+    """Writes config.json and model.safetensors with the same tensors `random_model` makes.  `device`: where the
+    values are worked out before they are written (the same numbers on the CPU and on the GPU up to the last bit
+    of either's logarithm and cosine; a GPU makes a billion of them in seconds)."""
     if isinstance(config, dict):
         arch = resolve(config)
         config = arch.config_class.from_dict(config)
@@ -61,7 +63,7 @@ def write_random_model(config, folder: str, seed: int, dtype="bfloat16", std: fl
     os.makedirs(folder, exist_ok=True)
     model = Model(arch.build_spec(config, None))
     specs = model.named_params()
-    src = RandomSource(seed, store, "cpu", std)
+    src = RandomSource(seed, store, device, std)
     src.expect(specs)
     items = [(name, LazyTensor(torch.int32 if spec.integer else store, spec.shape,
                                lambda n=name: src.tensor(n))) for name, spec in specs.items()]

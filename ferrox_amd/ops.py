@@ -56,7 +56,7 @@ _sigs = {
     ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float],
     ("elementwise", "fx_rope_kv_write"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -68,7 +68,7 @@ _sigs = {
                           c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
     ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
                               c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                              c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                              c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
@@ -149,6 +149,24 @@ def _freq_factors(freq_factors, rotary_dim):
     return freq_factors
 
 
+_inv_freq_tables: dict = {}
+
+
+def rotary_frequencies(device, rotary_dim: int, theta: float) -> torch.Tensor | None:
+    """float32 [rotary_dim / 2] on the device: theta^(-2i/rotary_dim), worked out in float64 on the host and
+    rounded once, so that the numbers do not depend on whose `powf` made them (the reference makes them in
+    float32, ferrox-core/src/attention.rs:26: the last bit is its libm's).  The kernels multiply them by the
+    position in float32, as the reference does (attention.rs:27).  Tables are kept for the life of the process:
+    recorded steps hold their addresses."""
+    if rotary_dim <= 0:
+        return None
+    key = (torch.device(device), int(rotary_dim), float(theta))
+    if key not in _inv_freq_tables:
+        values = [1.0 / float(theta) ** (2.0 * i / rotary_dim) for i in range(rotary_dim // 2)]
+        _inv_freq_tables[key] = torch.tensor(values, dtype=torch.float64).to(torch.float32).to(device)
+    return _inv_freq_tables[key]
+
+
 def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads,
                   head_dim, block_size, rotary_dim, theta, interleaved=False, freq_factors=None) -> None:
     """Rotate q in place; rotate k and write it and v into the pages (skipped when k_pages is None).
@@ -170,7 +188,7 @@ def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, 
           _p(v), v.stride(0), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
           _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
           _p(k_pages), _p(v_pages), T, n_heads, n_kv_heads, head_dim, block_size, rotary_dim,
-          1 if interleaved else 0, float(theta), _p(freq_factors))
+          1 if interleaved else 0, _p(rotary_frequencies(q.device, rotary_dim, theta)), _p(freq_factors))
 
 
 def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:
@@ -375,7 +393,7 @@ def qkv_rope(x, w, bias, positions, token_seq, block_table, k_pages, v_pages, n_
           _p(later.ss) if later else None, later.ss.shape[1] if later else 0, float(later.eps) if later else 0.0,
           _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")), _p(_i32(block_table, "block_table")),
           block_table.shape[1] if block_table is not None else 0, _p(k_pages), _p(v_pages),
-          n_heads, n_kv_heads, head_dim, block_size, rotary_dim, float(theta),
+          n_heads, n_kv_heads, head_dim, block_size, rotary_dim, _p(rotary_frequencies(xt.device, rotary_dim, theta)),
           _p(_freq_factors(freq_factors, rotary_dim)))
     return out
 

@@ -84,7 +84,9 @@ WIDE_G = {
     "max_position_embeddings": 8192, "use_sliding_window": False, "sliding_window": 4096,
     "max_window_layers": 1, "tie_word_embeddings": False,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5),
+# one layer of the smaller model's sizes under its real vocabulary: the head and the sampling at 151,936 columns
+WIDE_DV = dict(WIDE_D, vocab_size=151936)
+TINY = {"DV": (WIDE_DV, 7), "A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5),
         "G": (WIDE_G, 6)}
 
 
@@ -93,13 +95,28 @@ def model_folders(tmp_path_factory):
     """name, dtype -> folder with config.json and model.safetensors (made once a session)."""
     made = {}
 
-    def get(name: str, dtype: str = "float32") -> str:
-        key = (name, dtype)
+    def get(name: str, dtype: str = "float32", std: float = 0.02, qk_scale: float = 1.0, **overrides) -> str:
+        """`std`: spread of the random weights (0.2 gives logits that single out tokens).  `qk_scale`: the query and
+        key projections (weights and biases) are multiplied by it after they are drawn, which makes attention
+        peaked, so that where a key lies and how exactly it is rotated shows in the logits.  `overrides` replace
+        keys of the configuration."""
+        key = (name, dtype, std, qk_scale, tuple(sorted(overrides.items())))
         if key not in made:
             from ferrox_amd.engine.loading import write_random_model
             cfg, seed = TINY[name]
             folder = str(tmp_path_factory.mktemp(f"tiny{name}_{dtype}"))
-            write_random_model(dict(cfg), folder, seed, dtype)
+            import torch
+            # (whoever reads the folder reads what was written; the GPU makes the large models in seconds)
+            device = "cuda:0" if torch.cuda.is_available() else "cpu"
+            write_random_model(dict(cfg, **overrides), folder, seed, dtype, std=std, device=device)
+            if qk_scale != 1.0:
+                from safetensors.torch import load_file, save_file
+                path = os.path.join(folder, "model.safetensors")
+                tensors = load_file(path)
+                for n in tensors:
+                    if ".q_proj." in n or ".k_proj." in n:
+                        tensors[n] = (tensors[n].double() * qk_scale).to(tensors[n].dtype)
+                save_file(tensors, path)
             made[key] = folder
         return made[key]
 

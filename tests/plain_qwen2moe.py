@@ -46,17 +46,35 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return x * scale * weight
 
 
-def rope_neox(vec: torch.Tensor, pos: int, theta: float) -> torch.Tensor:
+def rope_angle(pos: int, i: int, dim: int, theta: float, angles: str = "exact") -> float:
+    """The angle of pair i at position pos: pos / theta^(2i/dim) (ferrox-core/src/attention.rs:26-27).
+
+    The reference works it out in float32: `freq = 1.0 / theta.powf(2i / dim)`, `angle = pos as f32 * freq`.
+    angles="float32" does the same: the frequency rounded to float32, times the position in float32 (one rounded
+    product); deep in a sequence that angle is off the exact one by up to half a unit in its last place, 1e-4 rad
+    at position 2,000, which is part of what the reference computes.  (The frequency is rounded from its exact
+    value here; the reference's is whatever its float32 `powf` returns, which may differ in the last bit.)
+    angles="exact" keeps float64 throughout.
+    """
+    freq = 1.0 / (theta ** ((2 * i) / dim))
+    if angles == "exact":
+        return pos * freq
+    assert angles == "float32", angles
+    import numpy as np
+    return float(np.float32(pos) * np.float32(freq))
+
+
+def rope_neox(vec: torch.Tensor, pos: int, theta: float, angles: str = "exact") -> torch.Tensor:
     """Split-half rotary on one head vector (ferrox-core/src/attention.rs:20-32).
 
-    Pair (i, i + half) is rotated by angle pos / theta^(2i/dim).
+    Pair (i, i + half) is rotated by `rope_angle(pos, i, dim, theta, angles)`; sine and cosine of that angle
+    are taken in float64.
     """
     dim = vec.shape[-1]
     half = dim // 2
     out = vec.clone()
     for i in range(half):
-        freq = 1.0 / (theta ** ((2 * i) / dim))
-        angle = pos * freq
+        angle = rope_angle(pos, i, dim, theta, angles)
         s, c = math.sin(angle), math.cos(angle)
         a, b = vec[..., i], vec[..., i + half]
         out[..., i] = a * c - b * s
@@ -64,12 +82,12 @@ def rope_neox(vec: torch.Tensor, pos: int, theta: float) -> torch.Tensor:
     return out
 
 
-def rope_neox_rows(x: torch.Tensor, positions, theta: float) -> torch.Tensor:
+def rope_neox_rows(x: torch.Tensor, positions, theta: float, angles: str = "exact") -> torch.Tensor:
     """`rope_neox` on x[T, n_heads, head_dim], row t at positions[t]
     (ferrox-models/src/decoder.rs:3489-3507: every q head and k head, full head_dim)."""
     out = torch.empty_like(x)
     for t in range(x.shape[0]):
-        out[t] = rope_neox(x[t], int(positions[t]), theta)
+        out[t] = rope_neox(x[t], int(positions[t]), theta, angles)
     return out
 
 
@@ -233,7 +251,7 @@ def load_folder(folder: str, dtype=torch.float64):
 
 
 def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0, margins=None, routing=None,
-            chosen=None, router_probs=None, stored=None) -> torch.Tensor:
+            chosen=None, router_probs=None, stored=None, angles: str = "float32") -> torch.Tensor:
     """Logits[T, V] of one whole sequence (ferrox-models/src/decoder.rs:3014-3678
     followed by the head on every row, decoder.rs:2952-2973).
 
@@ -242,7 +260,8 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
     `router_margin` over the sparse layers.  `routing[t][j]` forces the experts of position t in the
     j-th sparse layer; `chosen`, a list, receives the experts used in the same shape, and
     `router_probs`, a list, the router's probabilities of all experts as [position][sparse layer][expert].
-    `stored`: see the head of this file.
+    `stored`: see the head of this file.  `angles`: how the rotation's angles are worked out, see `rope_angle`;
+    the default is the reference's float32 product.
     """
     keep = stored if stored is not None else (lambda t: t)
     T = len(tokens)
@@ -272,8 +291,8 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, start_pos: int = 0,
             k = k + w[p + "self_attn.k_proj.bias"]                                   # decoder.rs:3234-3254
             v = v + w[p + "self_attn.v_proj.bias"]
         q, k, v = keep(q), keep(k), keep(v)
-        q = keep(rope_neox_rows(q.reshape(T, nh, hd), positions, theta))
-        k = keep(rope_neox_rows(k.reshape(T, nkv, hd), positions, theta))
+        q = keep(rope_neox_rows(q.reshape(T, nh, hd), positions, theta, angles))
+        k = keep(rope_neox_rows(k.reshape(T, nkv, hd), positions, theta, angles))
         v = v.reshape(T, nkv, hd)                                                    # v is not rotated
         a = keep(causal_attention(q, k, v, nh, nkv, layer_window(cfg, l), stored=stored))
         h = h + a.reshape(T, nh * hd) @ w[p + "self_attn.o_proj.weight"].T          # no bias: decoder.rs:3549-3560

@@ -361,21 +361,17 @@ def test_rope_and_cache_write_of_long_prompts(dtype, nh, nkv, hd, bs, rot, seq_l
     T = len(toks)
     p = pos.double().cpu()
     freq = 1.0 / theta ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot)
-    ang = p[:, None] * freq[None, :]                                   # plain.rope_neox, all tokens at once
+    # plain.rope_neox(..., "float32"), all tokens at once: the float32 product of position and float32 frequency
+    ang = (p.float()[:, None] * freq.float()[None, :]).double()
     def rotated(x, heads):
         x = x.double().cpu().reshape(T, heads, hd)
         a, b = x[..., :rot // 2], x[..., rot // 2:rot]
         c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
         return torch.cat([a * c - b * s_, a * s_ + b * c, x[..., rot:]], dim=-1)
-    assert torch.allclose(plain.rope_neox(q[5].double().cpu().reshape(nh, hd)[:, :rot], int(pos[5]), theta),
-                          rotated(q, nh)[5, :, :rot])                  # the formula above is the plain one
-    # the angle is position x frequency in float32 (ferrox-core/src/attention.rs:20-32): at position p it is known to
-    # about p x 2^-23, and so are the rotated values (times their size); bfloat16 rounds coarser than that anyway
-    def near(got, want, what):
-        got, want = got.double().cpu(), want.double().cpu()
-        bound = float(want.abs().max()) * ((1e-5 if dtype == torch.float32 else 1e-2) + float(p.max()) * 2.0 ** -22)
-        err = float((got - want).abs().max())
-        assert err <= bound, f"{what}: max error {err:.3e} > {bound:.3e}"
+    for t in (5, T - 1):
+        assert torch.allclose(plain.rope_neox(q[t].double().cpu().reshape(nh, hd)[:, :rot], int(pos[t]), theta, "float32"),
+                              rotated(q, nh)[t, :, :rot], atol=1e-12)  # the formula above is the plain one
+    near = lambda got, want, what: close(got, want, dtype, what)
     near(q_rot.reshape(T, nh, hd), rotated(q, nh), "rotated queries")
     page_of = table.cpu()[seq.cpu().long(), (pos.cpu() // bs).long()].long()
     slot = (pos.cpu() % bs).long()
@@ -384,6 +380,84 @@ def test_rope_and_cache_write_of_long_prompts(dtype, nh, nkv, hd, bs, rot, seq_l
     used = torch.zeros(n_pages, bs, dtype=torch.bool)
     used[page_of, slot] = True
     assert bool(torch.isnan(v_pages.cpu().float().permute(0, 3, 1, 2)[~used]).all()), "slots past the sequences stay untouched"
+
+
+DEEP_POSITIONS = [0, 1, 511, 2047, 2048, 4097, 8191, 16384, 20000, 32766, 32767]
+
+
+def rotated_by_float32_angles(x, positions, rot, theta, angles="float32"):
+    """x [T, heads, hd] in float64 with its first `rot` dimensions turned, split halves, by the plain model's angles"""
+    out = x.clone()
+    for t, p in enumerate(positions):
+        out[t, :, :rot] = plain.rope_neox(x[t, :, :rot], int(p), theta, angles)
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,bs,rot,theta", [(2, 1, 128, 64, 128, 1e6), (3, 3, 64, 16, 32, 1e4), (2, 2, 16, 16, 16, 1e6)])
+def test_rope_deep_in_a_sequence(dtype, nh, nkv, hd, bs, rot, theta):
+    """Rotation and cache write at positions up to 32,767.  The angle is the float32 product of the position and
+    the float32 frequency (ferrox-core/src/attention.rs:26-27); against float64 sines and cosines of exactly that
+    angle the float32 kernel is right to rounding, and would be off by a thousand times that against exact angles."""
+    from ferrox_amd import ops
+    T = len(DEEP_POSITIONS)
+    blocks = -(-32768 // bs)
+    table = torch.zeros(1, blocks, dtype=torch.int32)
+    used = sorted({p // bs for p in DEEP_POSITIONS})
+    order = torch.randperm(len(used), generator=torch.Generator().manual_seed(bs)).tolist()
+    for b, page in zip(used, order):
+        table[0, b] = page + 1                             # page 0 stays empty
+    q, k, v = rnd(T, nh * hd, dtype=dtype), rnd(T, nkv * hd, dtype=dtype, seed=1), rnd(T, nkv * hd, dtype=dtype, seed=2)
+    k_pages = torch.full((len(used) + 1, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
+    v_pages = torch.full((len(used) + 1, nkv, hd, bs), float("nan"), dtype=dtype, device=DEV)
+    pos = torch.tensor(DEEP_POSITIONS, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    q_rot = q.clone()
+    ops.rope_kv_write(q_rot, k, v, pos, seq, table.to(DEV), k_pages, v_pages, nh, nkv, hd, bs, rot, theta)
+    want_q = rotated_by_float32_angles(q.double().cpu().reshape(T, nh, hd), DEEP_POSITIONS, rot, theta)
+    want_k = rotated_by_float32_angles(k.double().cpu().reshape(T, nkv, hd), DEEP_POSITIONS, rot, theta)
+    page_of = table[0, (pos.cpu() // bs).long()].long()
+    slot = (pos.cpu() % bs).long()
+    got_q, got_k = q_rot.reshape(T, nh, hd), k_pages.cpu()[page_of, :, slot, :]
+    close(got_q, want_q, dtype, "rotated queries")
+    close(got_k, want_k, dtype, "key pages")
+    assert torch.equal(v_pages.cpu()[page_of, :, :, slot], v.cpu().reshape(T, nkv, hd)), "value pages"
+    assert bool(torch.isnan(k_pages[0].float()).all()), "a page that no position maps to was written"
+    if dtype == torch.float32:
+        exact = rotated_by_float32_angles(q.double().cpu().reshape(T, nh, hd), DEEP_POSITIONS, rot, theta, "exact")
+        off = float((got_q.double().cpu() - exact).abs().max()) / float(exact.abs().max())
+        assert off > 1e-4, f"exact angles are only {off:.2e} away: the test does not tell the two apart"
+
+
+def test_qkv_product_that_rotates_deep_in_a_sequence():
+    """the rotating product's epilogue at positions up to 32,767: the bits of the product followed by rope_kv_write,
+    which the test above holds against the plain rotation"""
+    from ferrox_amd import ops
+    T, H, nh, nkv, hd, bs, rot, theta = len(DEEP_POSITIONS), 264, 4, 2, 64, 64, 64, 1e6
+    N = (nh + 2 * nkv) * hd
+    w = rnd(N, H, dtype=torch.bfloat16, seed=1, scale=0.05)
+    b = rnd(N, dtype=torch.bfloat16, seed=2)
+    x = rnd(T, H, dtype=torch.bfloat16, seed=3)
+    blocks = 32768 // bs
+    used = sorted({p // bs for p in DEEP_POSITIONS})
+    table = torch.zeros(1, blocks, dtype=torch.int32)
+    for i, blk in enumerate(used):
+        table[0, blk] = len(used) - i
+    table = table.to(DEV)
+    pos = torch.tensor(DEEP_POSITIONS, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    pages = lambda: (torch.zeros(len(used) + 1, nkv, bs, hd, dtype=torch.bfloat16, device=DEV),
+                     torch.zeros(len(used) + 1, nkv, hd, bs, dtype=torch.bfloat16, device=DEV))
+    assert ops.can_qkv_rope(x, w, T, hd, rot, False)
+    k1, v1 = pages()
+    got = ops.qkv_rope(x, w, b, pos, seq, table, k1, v1, nh, nkv, hd, bs, rot, theta)
+    k2, v2 = pages()
+    ref = ops.gemm(x, w, bias=b)
+    qw, kvw = nh * hd, nkv * hd
+    ops.rope_kv_write(ref[:, :qw], ref[:, qw:qw + kvw], ref[:, qw + kvw:], pos, seq, table, k2, v2, nh, nkv, hd, bs, rot, theta)
+    assert torch.equal(got[:, :qw], ref[:, :qw]), "rotated queries"
+    assert torch.equal(k1, k2) and float(k1.abs().sum()) > 0, "key pages"
+    assert torch.equal(v1, v2), "value pages"
 
 
 @pytest.mark.parametrize("later", [False, True])
@@ -626,6 +700,11 @@ def test_router_golden_vector():
     assert ids[0].tolist() == [1, 3]                               # ferrox-moe/src/lib.rs:834-841
 
 
+# xorshift64 started from a small number returns small numbers at first (the first uniform draw is 0, which picks
+# the first token that has any probability whatever the logits say); the sampling tests start it high
+SEED = 0x2545F4914F6CDD1D
+
+
 def test_sampling_kernel():
     from ferrox_amd import ops
     V = 1000
@@ -640,11 +719,14 @@ def test_sampling_kernel():
              dict(temperature=0.0, repetition_penalty=2.0, presence_penalty=0.5, frequency_penalty=0.25),
              dict(temperature=0.9, top_k=1)]
     hist = [int(logits[0].argmax()), 3, 3, 999, int(logits[0].argmax())]
+    draws = []
     for case in cases:
+        picked = set()
         for trial in range(12):
-            rng_a = plain.XorShift64(trial + 1)
-            want = plain.sample(logits[0].double().cpu().tolist(), rng_a, history=hist, **case)
-            u = plain.XorShift64(trial + 1).next_f32()
+            seed = SEED + (trial << 45)
+            want = plain.sample(logits[0].double().cpu().tolist(), plain.XorShift64(seed), history=hist, **case)
+            u = plain.XorShift64(seed).next_f32()
+            draws.append(u)
             f = lambda v: torch.tensor([v], dtype=torch.float32, device=DEV)
             got = ops.sample(logits[:1], temperature=f(case.get("temperature", 0.0)), draw=f(u),
                              top_k=torch.tensor([case.get("top_k", 0)], dtype=torch.int32, device=DEV),
@@ -653,6 +735,48 @@ def test_sampling_kernel():
                              hist=torch.tensor(hist, dtype=torch.int32, device=DEV),
                              hist_start=torch.tensor([0, len(hist)], dtype=torch.int32, device=DEV)).tolist()[0]
             assert got == want, f"{case} trial {trial}: kernel {got}, plain {want}"
+            picked.add(got)
+        if case["temperature"] > 0 and case.get("top_k", 0) != 1:
+            assert len(picked) >= 3, f"{case}: twelve draws picked {sorted(picked)} only"
+    assert min(draws) > 0.0 and max(draws) - min(draws) > 0.5, "the draws do not spread over (0, 1)"
+
+
+def test_sampling_kernel_at_the_real_vocabulary():
+    """V = 151,936, three rows in one call, eight draws each: the command line's defaults (top-k 40, top-p 0.95,
+    repetition penalty 1.1: ferrox-cli/src/run.rs:52-64) and temperature alone, against the plain sampler
+    (ferrox-models/src/sampling.rs:93-189).  A few dozen tokens stand out of the noise, as in a trained model, so
+    that the most likely token has a probability near 0.2 and top-p cuts inside the top-k."""
+    from ferrox_amd import ops
+    V, R = 151936, 3
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(R, V, generator=g) * 2.0
+    for r in range(R):
+        idx = torch.randperm(V, generator=g)[:30]
+        logits[r, idx] += 5.0 + 3.0 * torch.rand(30, generator=g)
+    rows = logits.double().tolist()
+    dev = logits.to(DEV)
+    assert ops.sample(dev).tolist() == logits.argmax(-1).tolist()
+    hists = [[int(logits[0].argmax()), 7, 7, V - 1], [], [int(logits[2].argmax())] * 3 + [int(logits[2].topk(2).indices[1])]]
+    flat = [t for h in hists for t in h]
+    starts = [0]
+    for h in hists:
+        starts.append(starts[-1] + len(h))
+    f = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    for case in (dict(temperature=0.8, top_k=40, top_p=0.95, repetition_penalty=1.1), dict(temperature=0.8)):
+        gens = [plain.XorShift64(SEED + ((r + 1) << 45)) for r in range(R)]
+        mirrors = [plain.XorShift64(SEED + ((r + 1) << 45)) for r in range(R)]
+        picked = [set() for _ in range(R)]
+        for draw in range(8):
+            want = [plain.sample(rows[r], gens[r], history=hists[r], **case) for r in range(R)]
+            u = [m.next_f32() for m in mirrors]
+            got = ops.sample(dev, temperature=f([case["temperature"]] * R), draw=f(u), top_k=i32([case.get("top_k", 0)] * R),
+                             top_p=f([case.get("top_p", 1.0)] * R), rep_penalty=f([case.get("repetition_penalty", 1.0)] * R),
+                             presence=f([0.0] * R), frequency=f([0.0] * R), hist=i32(flat), hist_start=i32(starts)).tolist()
+            assert got == want, f"{case} draw {draw}: kernel {got}, plain {want}"
+            for r in range(R):
+                picked[r].add(got[r])
+        assert all(len(p) >= 3 for p in picked), f"{case}: eight draws picked {picked}"
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 2048), (8, 6144, 2048), (5, 100, 96), (16, 48, 264), (31, 257, 520),

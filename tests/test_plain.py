@@ -50,6 +50,26 @@ def test_rope_pairing_sign_and_frequencies():
     assert not torch.allclose(plain.rope_neox(x, 9, 1e4), inter, atol=1e-3)
 
 
+def test_rope_angle_in_float32_is_one_rounded_product():
+    """attention.rs:26-27: `angle = pos as f32 * freq` with a float32 frequency.  The float32 angle is the rounded
+    product of the rounded frequency, equal to the exact angle where nothing is rounded (pair 0, whose frequency
+    is 1) and within half a unit in the last place of the angle, plus the frequency's own rounding, elsewhere."""
+    import numpy as np
+    for theta, dim in ((1e4, 16), (1e6, 128)):
+        for pos in (0, 1, 7, 500, 2047, 2048, 32767):
+            assert plain.rope_angle(pos, 0, dim, theta, "float32") == float(pos)
+            for i in (1, 3, dim // 2 - 1):
+                exact, f32 = plain.rope_angle(pos, i, dim, theta), plain.rope_angle(pos, i, dim, theta, "float32")
+                assert f32 == float(np.float32(f32))                            # a float32 number
+                assert abs(f32 - exact) <= 2.0 ** -23 * abs(exact) + 1e-300
+    # deep in a sequence the two are apart by far more than the tests' float32 tolerance
+    assert max(abs(plain.rope_angle(2047, i, 16, 1e4, "float32") - plain.rope_angle(2047, i, 16, 1e4)) for i in range(8)) > 1e-6
+    x = randn(16)
+    near = plain.rope_neox(x, 2047, 1e4, "float32")
+    assert torch.allclose(near, plain.rope_neox(x, 2047, 1e4), atol=1e-3) and not torch.allclose(
+        near, plain.rope_neox(x, 2047, 1e4), atol=1e-7)
+
+
 def test_rope_scores_depend_on_distance_only():
     q, k = randn(16), randn(16)
     a = plain.rope_neox(q, 37, 1e6) @ plain.rope_neox(k, 30, 1e6)
@@ -164,9 +184,12 @@ def test_positions_shift_invariance(tiny):
     for name in ("A", "B"):
         cfg, w = tiny[name]
         toks = [5, 17, 3, 99, 42, 7, 7, 1, 250, 33, 12, 8, 90, 21, 60, 2, 4, 6, 19, 55]
-        a = plain.forward(cfg, w, toks)
-        b = plain.forward(cfg, w, toks, start_pos=37)
+        a = plain.forward(cfg, w, toks, angles="exact")
+        b = plain.forward(cfg, w, toks, start_pos=37, angles="exact")
         assert torch.allclose(a, b, atol=1e-9), name
+        # with the reference's float32 angles the shifted run differs by their rounding alone
+        c = plain.forward(cfg, w, toks, start_pos=37)
+        assert torch.allclose(a, c, atol=1e-6) and not torch.equal(b, c), name
 
 
 def test_prefix_property_and_bias_is_live(tiny):
