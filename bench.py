@@ -42,20 +42,12 @@ sys.path.insert(0, ROOT)
 PEAK_HBM = 8.0e12          # bytes/s, MI355X HBM3E
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-A27B = {
-    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
-    "num_hidden_layers": 24, "hidden_size": 2048, "num_attention_heads": 16, "num_key_value_heads": 16,
-    "num_experts": 60, "num_experts_per_tok": 4, "norm_topk_prob": False, "moe_intermediate_size": 1408,
-    "shared_expert_intermediate_size": 5632, "intermediate_size": 5632, "decoder_sparse_step": 1,
-    "mlp_only_layers": [], "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
-    "max_position_embeddings": 8192, "use_sliding_window": False, "sliding_window": 32768,
-    "max_window_layers": 21, "tie_word_embeddings": False, "qkv_bias": True,
-}
-FULL_LAYERS = 24
+from ferrox_amd.config import presets  # noqa: E402  (sizes are data: the config.json of each shape lies in the package)
+
+A27B = presets.load("qwen1.5-moe-a2.7b")
+FULL_LAYERS = A27B["num_hidden_layers"]
 # the other shape of the family (not the default run): Qwen2-57B-A14B
-A14B = dict(A27B, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
-            num_experts=64, num_experts_per_tok=8, moe_intermediate_size=2560, shared_expert_intermediate_size=20480,
-            intermediate_size=18944, max_position_embeddings=32768)
+A14B = presets.load("qwen2-57b-a14b")
 SHAPES = {"a2.7b": ("Qwen1.5-MoE-A2.7B shape", A27B), "57b-a14b": ("Qwen2-57B-A14B shape", A14B)}
 
 

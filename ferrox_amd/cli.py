@@ -1,10 +1,14 @@
 """Command line in the manner of the reference's `ferrox -m ... -p ... -n ...`
 (ferrox-cli/src/run.rs:19-125, main.rs:254-296): the same flag names and
 defaults where this engine has the feature.  The model is a folder with
-config.json and safetensors, not a GGUF file.  The prompt is text when the
-folder holds a tokenizer.json (read with the `tokenizers` package), else token
-ids through --tokens.  Generated text (or ids) goes to stdout, timings to stderr
-(run.rs:680-695).
+config.json and safetensors, not a GGUF file; or, with --random-weights, a
+configuration alone (--config FILE, or the name of one of the shapes that
+`ferrox_amd.config.presets` holds) whose weights are drawn from --seed, as the
+reference serves synthetic weights when it is given no model
+(ferrox-server/src/model.rs:228-243).  The prompt is text when the folder holds
+a tokenizer.json (or --tokenizer names one; read with the `tokenizers`
+package), else token ids through --tokens.  Generated text (or ids) goes to
+stdout, timings to stderr (run.rs:680-695).
 """
 from __future__ import annotations
 
@@ -13,10 +17,18 @@ import os
 import sys
 import time
 
+from .config import presets
+
 
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="ferrox-amd", description="Qwen2-MoE text generation on one MI355X")
-    ap.add_argument("-m", "--model", required=True, metavar="DIR", help="model folder (config.json + safetensors)")
+    ap.add_argument("-m", "--model", metavar="DIR", help="model folder (config.json + safetensors)")
+    ap.add_argument("--random-weights", action="store_true",
+                    help="no model folder: weights drawn from --seed for the configuration that --config names")
+    ap.add_argument("--config", metavar="FILE|NAME", default="qwen1.5-moe-a2.7b",
+                    help="with --random-weights: a config.json, or one of: " + ", ".join(presets.names()))
+    ap.add_argument("--layers", type=int, default=0, help="with --random-weights: build only so many layers (0 = all)")
+    ap.add_argument("--tokenizer", metavar="FILE", help="tokenizer.json (default: the one in the model folder)")
     ap.add_argument("-p", "--prompt", default="", help="prompt text (needs tokenizer.json in the model folder)")
     ap.add_argument("-f", "--file", metavar="FILE", help="read the prompt from a file")
     ap.add_argument("--tokens", metavar="IDS", help="prompt as comma-separated token ids")
@@ -60,9 +72,15 @@ def unescape(s: str) -> str:
 
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
+    if bool(args.model) == bool(args.random_weights):
+        print("error: give either a model folder (-m DIR) or --random-weights [--config FILE|NAME]", file=sys.stderr)
+        return 2
     tokenizer = None
-    tok_path = os.path.join(args.model, "tokenizer.json")
-    if os.path.isfile(tok_path):
+    tok_path = args.tokenizer or (os.path.join(args.model, "tokenizer.json") if args.model else "")
+    if args.tokenizer and not os.path.isfile(tok_path):
+        print(f"error: no tokenizer file at {tok_path}", file=sys.stderr)
+        return 2
+    if tok_path and os.path.isfile(tok_path):
         try:
             from tokenizers import Tokenizer
             tokenizer = Tokenizer.from_file(tok_path)
@@ -82,7 +100,8 @@ def main(argv=None) -> int:
         if args.escape:
             text = unescape(text)
         if tokenizer is None:
-            print("error: no tokenizer.json in the model folder; give the prompt as --tokens 1,2,3", file=sys.stderr)
+            print("error: no tokenizer.json (in the model folder or through --tokenizer); give the prompt as --tokens 1,2,3",
+                  file=sys.stderr)
             return 2
         prompt_ids = tokenizer.encode(text).ids
     if not prompt_ids:
@@ -103,14 +122,22 @@ def main(argv=None) -> int:
     # program with one message and exit code 2 (the reference bails the same way, run.rs:598-607)
     try:
         t0 = time.time()
-        engine = Engine(args.model, dtype=args.dtype, device=args.device, block_size=args.block_size,
+        seed = args.seed if args.seed >= 0 else (time.time_ns() & 0x7FFFFFFFFFFFFFFF)       # run.rs:462-471
+        source = dict(model_dir=args.model)
+        if args.random_weights:
+            from .config.base import read_config_json
+            raw = read_config_json(args.config) if os.path.exists(args.config) else presets.load(args.config)
+            if args.layers > 0:
+                raw = dict(raw, num_hidden_layers=args.layers)
+            source = dict(config=raw, random_weights=seed)
+            print(f"random weights: seed {seed}, configuration {args.config}", file=sys.stderr)
+        engine = Engine(**source, dtype=args.dtype, device=args.device, block_size=args.block_size,
                         num_pages=args.num_pages or None, max_seqs=4, ctx_size=args.ctx_size,
                         max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk)
         print(f"load time: {time.time() - t0:.2f} s", file=sys.stderr)
         defaulted = getattr(getattr(engine.model, "config", None), "defaulted_keys", ())
         if defaulted:                                                                    # run.rs:520-528
             print("config keys defaulted: " + ", ".join(defaulted), file=sys.stderr)
-        seed = args.seed if args.seed >= 0 else (time.time_ns() & 0x7FFFFFFFFFFFFFFF)       # run.rs:462-471
         params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
                                 args.presence_penalty, args.frequency_penalty, seed)
         t1 = time.time()

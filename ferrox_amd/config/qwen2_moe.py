@@ -40,7 +40,7 @@ class Qwen2MoeConfig:
     max_window_layers: int
     tie_word_embeddings: bool
     qkv_bias: bool | None      # None: decided by whether the checkpoint holds the bias tensors
-    eos_token_id: int | None = None
+    eos_token_id: int | tuple | None = None      # one id, or several (chat variants stop on either of two)
     bos_token_id: int | None = None
     defaulted_keys: tuple = field(default=(), compare=False)
 
@@ -64,7 +64,11 @@ class Qwen2MoeConfig:
         top_k = r.integer("num_experts_per_tok", 2 if experts else 0, minimum=0)  # default 2: loader.rs:248-256
         eos = raw.get("eos_token_id")
         if isinstance(eos, list):
-            eos = eos[0] if eos else None
+            if any(isinstance(i, bool) or not isinstance(i, int) for i in eos):
+                raise ConfigError(f"{where}: key 'eos_token_id' must be an integer or a list of integers, got {eos!r}")
+            eos = tuple(eos) if len(eos) > 1 else (eos[0] if eos else None)
+        elif eos is not None and (isinstance(eos, bool) or not isinstance(eos, int)):
+            raise ConfigError(f"{where}: key 'eos_token_id' must be an integer or a list of integers, got {eos!r}")
         cfg = cls(
             vocab_size=r.integer("vocab_size", minimum=1),
             hidden_size=hidden,
@@ -88,7 +92,7 @@ class Qwen2MoeConfig:
             max_window_layers=r.integer("max_window_layers", 0, minimum=0),
             tie_word_embeddings=r.boolean("tie_word_embeddings", False),
             qkv_bias=raw.get("qkv_bias") if isinstance(raw.get("qkv_bias"), bool) else None,
-            eos_token_id=eos if isinstance(eos, int) else None,
+            eos_token_id=eos,
             bos_token_id=raw.get("bos_token_id") if isinstance(raw.get("bos_token_id"), int) else None,
             defaulted_keys=tuple(r.defaulted),
         )
@@ -175,7 +179,7 @@ class Qwen2MoeConfig:
             d["qkv_bias"] = self.qkv_bias
         d["mlp_only_layers"] = list(self.mlp_only_layers)
         if self.eos_token_id is not None:
-            d["eos_token_id"] = self.eos_token_id
+            d["eos_token_id"] = list(self.eos_token_id) if isinstance(self.eos_token_id, tuple) else self.eos_token_id
         if self.bos_token_id is not None:
             d["bos_token_id"] = self.bos_token_id
         return d

@@ -19,7 +19,7 @@
 
 FX_DEFINE_LAST_ERROR()
 
-enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_RESID = 2, EPI_SILU_MUL = 3 };
+enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_RESID = 2, EPI_GATED = 3 };
 
 struct GemmArgs {
     const void* A;
@@ -62,6 +62,7 @@ struct GemmArgs {
     int rope_nh, rope_nkv, rope_hd, rope_bs, rope_rot;
     const float* rope_inv_freq;       // rot/2 floats: pair i turns by (float)pos * rope_inv_freq[i]
     const float* rope_freq_factors;   // rot/2 floats or null: the angle of pair i is divided by rope_freq_factors[i]
+    int act;     // EPI_GATED: which activation the gate goes through (ACT_*)
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
@@ -167,7 +168,24 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
     return true;
 }
 
+// The gated epilogue stores act(gate) * up; `act` is a parameter of the call (GemmArgs::act), uniform over the
+// launch, so another gated feed-forward needs no other kernel.
+//   ACT_SILU       x / (1 + exp(-x))                               (ferrox-core/src/matmul.rs:268-270)
+//   ACT_GELU_TANH  0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+//   ACT_GELU       0.5 x (1 + erf(x / sqrt(2)))
+//   ACT_RELU       max(x, 0)
+enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_GELU = 2, ACT_RELU = 3, ACT_COUNT = 4 };
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float gated_f(int act, float gate, float up) {
+    float a;
+    switch (act) {
+        case ACT_GELU_TANH: a = 0.5f * gate * (1.0f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate))); break;
+        case ACT_GELU: a = 0.5f * gate * (1.0f + erff(gate * 0.7071067811865476f)); break;
+        case ACT_RELU: a = fmaxf(gate, 0.0f); break;
+        default: a = silu_f(gate); break;
+    }
+    return a * up;
+}
 
 // ===========================================================================
 // bfloat16 on MFMA
@@ -318,7 +336,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                 for (int j = 0; j < NT; j += 2) {
                     const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
                     if (n < g.N)
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(acc[i][j][r]) * acc[i][j + 1][r]);
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, acc[i][j][r], acc[i][j + 1][r]));
                 }
             } else {
 #pragma unroll
@@ -565,7 +583,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
                 for (int j = 0; j < NT; j += 2) {
                     const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
                     if (n < g.N)
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(acc[i][j][r]) * acc[i][j + 1][r]);
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, acc[i][j][r], acc[i][j + 1][r]));
                 }
             } else {
 #pragma unroll
@@ -997,7 +1015,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             float o = v[r] * rstd;
             asm volatile("" : "+v"(o));          // the product is rounded before the bias is added (no fused multiply-add)
             if (DUAL) {
-                from_float((bf16*)g.C + (size_t)m * g.ldc + n, silu_f(o) * v2[r]);
+                from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, o, v2[r]));
                 continue;
             }
             if (g.bias) o += bias_v[r];
@@ -1093,7 +1111,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             float v = acc[i][j];
             float* out = (float*)g.C + (size_t)m * g.ldc + n;
             if (DUAL) {
-                *out = silu_f(v) * acc2[i][j];
+                *out = gated_f(g.act, v, acc2[i][j]);
             } else {
                 if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
                 if (EPI == EPI_RESID) {
@@ -1112,7 +1130,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
 // ===========================================================================
 template <int TM, int TN, int WM, int WN>
 static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
-    const bool dual = epi == EPI_SILU_MUL;
+    const bool dual = epi == EPI_GATED;
     g.n_col_tiles = ceil_div(g.N, dual ? TN / 2 : TN);
     g.n_row_tiles = m_tiles;
     dim3 grid(8 * ceil_div((long)g.n_col_tiles * g.n_row_tiles, 8));
@@ -1123,7 +1141,7 @@ static void launch_bf16(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
         case EPI_STORE: FX_TILED(false, EPI_STORE); break;
         case EPI_STORE_F32: FX_TILED(false, EPI_STORE_F32); break;
         case EPI_RESID: FX_TILED(false, EPI_RESID); break;
-        default: FX_TILED(true, EPI_SILU_MUL); break;
+        default: FX_TILED(true, EPI_GATED); break;
     }
 #undef FX_TILED
 }
@@ -1152,7 +1170,7 @@ FX_API int fx_debug_set(const char* key, int value) {
 
 template <int TMB, int TN, int NS, int NSA = NS>
 static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
-    g.n_col_tiles = ceil_div(g.N, epi == EPI_SILU_MUL ? TN / 2 : TN);
+    g.n_col_tiles = ceil_div(g.N, epi == EPI_GATED ? TN / 2 : TN);
     g.n_row_tiles = m_tiles;
     dim3 grid(g.expert_offsets ? 8 * ceil_div(m_tiles, 8) * g.n_col_tiles : 8 * ceil_div((long)g.n_col_tiles * m_tiles, 8));
     switch (epi) {
@@ -1160,14 +1178,14 @@ static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
         case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32, NSA><<<grid, 512, 0, s>>>(g); break;
         case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID, NSA><<<grid, 512, 0, s>>>(g); break;
         default:
-            if constexpr (TN % 128 == 0) gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_SILU_MUL, NSA><<<grid, 512, 0, s>>>(g);
+            if constexpr (TN % 128 == 0) gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_GATED, NSA><<<grid, 512, 0, s>>>(g);
             break;
     }
 }
 
 template <int MT, int WAVES, int NW>
 static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream_t s) {
-    dim3 grid(ceil_div(g.N, epi == EPI_SILU_MUL ? 8 * NW : 16 * NW), m_tiles);
+    dim3 grid(ceil_div(g.N, epi == EPI_GATED ? 8 * NW : 16 * NW), m_tiles);
     if constexpr (MT * NW * WAVES <= 32) {       // the partial sums of all waves fit in LDS
         if (g.norm_w) {
             gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE, true><<<grid, WAVES * 64, 0, s>>>(g);
@@ -1178,7 +1196,7 @@ static void launch_skinny_cfg(const GemmArgs& g, int epi, int m_tiles, hipStream
             case EPI_STORE_F32: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_STORE_F32><<<grid, WAVES * 64, 0, s>>>(g); break;
             case EPI_RESID: gemm_bf16_skinny_kernel<MT, WAVES, NW, false, EPI_RESID><<<grid, WAVES * 64, 0, s>>>(g); break;
             default:
-                if constexpr (NW % 2 == 0) gemm_bf16_skinny_kernel<MT, WAVES, NW, true, EPI_SILU_MUL><<<grid, WAVES * 64, 0, s>>>(g);
+                if constexpr (NW % 2 == 0) gemm_bf16_skinny_kernel<MT, WAVES, NW, true, EPI_GATED><<<grid, WAVES * 64, 0, s>>>(g);
                 break;
         }
     }
@@ -1262,19 +1280,20 @@ FX_API int fx_qkv_rope(void* stream, const void* A, long lda, const void* W, lon
     return 0;
 }
 
-// dtype: type of A and W.  C is: T for EPI_STORE and EPI_SILU_MUL, float32 otherwise.
+// dtype: type of A and W.  C is: T for EPI_STORE and EPI_GATED, float32 otherwise.
 // rows_hint: in grouped mode, the expected number of rows per expert (chooses the tile).
 FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, const void* W, long w_stride,
                    long up_offset, const void* bias, int bias_dtype, void* C, long ldc,
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
                    const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows,
-                   const float* row_ss, int row_ss_n) {
+                   const float* row_ss, int row_ss_n, int act) {
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
-    FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_SILU_MUL, "gemm: unknown epilogue %d", epi);
+    FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_GATED, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     FX_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%ld ldc=%ld too small for K=%d N=%d", lda, ldc, K, N);
-    FX_REQUIRE(!(epi == EPI_SILU_MUL && bias), "gemm: the gate/up epilogue takes no bias");
+    FX_REQUIRE(!(epi == EPI_GATED && bias), "gemm: the gate/up epilogue takes no bias");
+    FX_REQUIRE(act >= 0 && act < ACT_COUNT, "gemm: unknown activation %d", act);
     FX_REQUIRE(!(expert_offsets || pair_ids) || E > 0, "gemm: grouped mode needs E > 0");
     FX_REQUIRE(!pair_ids || (!expert_offsets && !a_rows && !c_rows && !row_scale && !norm_w && pair_div >= 1 && M <= 64 &&
                              dtype == FX_BF16),
@@ -1297,7 +1316,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
-    g.pair_ids = pair_ids; g.pair_div = pair_div;
+    g.pair_ids = pair_ids; g.pair_div = pair_div; g.act = act;
     g.kb_stride = kb_rows * 64;
     FX_REQUIRE(kb_rows >= 0 && (kb_rows == 0 || (dtype == FX_BF16 && K % 64 == 0 && ((uintptr_t)W % 16) == 0 && lda % 8 == 0 &&
                                                  ((uintptr_t)A % 16) == 0 && (up_offset % K) == 0)),
@@ -1315,7 +1334,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
             case EPI_STORE:
             case EPI_STORE_F32: gemm_f32_kernel<false, EPI_STORE_F32><<<grid, 256, 0, s>>>(g); break;
             case EPI_RESID: gemm_f32_kernel<false, EPI_RESID><<<grid, 256, 0, s>>>(g); break;
-            default: gemm_f32_kernel<true, EPI_SILU_MUL><<<grid, 256, 0, s>>>(g); break;
+            default: gemm_f32_kernel<true, EPI_GATED><<<grid, 256, 0, s>>>(g); break;
         }
         FX_CHECK_LAUNCH("gemm_f32");
         return 0;
@@ -1340,7 +1359,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     const long few_limit = expert_offsets && wide_ok ? g_few_rows : 64;
     if (g.vec_ok && (per_group <= few_limit || pair_ids) && !many_columns) {
         int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
-        const bool dual = epi == EPI_SILU_MUL;
+        const bool dual = epi == EPI_GATED;
         // 33 to 64 plain rows against few weight rows (the attention's output product: 2,048): four row tiles a
         // block leave 128 blocks; a block per row tile, with two sets of weight rows, gives 256 and every block a
         // quarter of the rows' operands to fetch (13.4 -> 9.1 us at 64 rows, 11.2 -> 9.0 at 40; with 6,144 weight
@@ -1376,7 +1395,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else if (g.vec_ok && K % 64 == 0 && !g_no_wide) {
         // the widest tile that still gives the 256 CUs (one block each) an even share of the work
-        const bool dual = epi == EPI_SILU_MUL;
+        const bool dual = epi == EPI_GATED;
         auto tiles = [&](int tm, int tn) {
             return (long)ceil_div(N, dual ? tn / 2 : tn) * (M / tm + (expert_offsets ? nonempty : (M % tm != 0)));
         };
@@ -1421,7 +1440,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
             launch_wide<8, 128, 4>(g, epi, M / 128 + (expert_offsets ? nonempty : (M % 128 != 0)), s);
     } else {
         const int m_tiles = M / 128 + (expert_offsets ? nonempty : (M % 128 != 0));
-        const bool dual = epi == EPI_SILU_MUL;
+        const bool dual = epi == EPI_GATED;
         // narrow outputs: tiles of 64 columns give the 256 CUs at least two blocks each
         if (!dual && (long)ceil_div(N, 128) * m_tiles < 512)
             launch_bf16<128, 64, 64, 32>(g, epi, m_tiles, s);

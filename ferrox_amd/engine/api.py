@@ -75,15 +75,16 @@ class Engine:
     def generate(self, prompts: list, max_new_tokens: int = 128, temperature: float = 0.0, top_k: int = 0,
                  top_p: float = 1.0, repetition_penalty: float = 1.0, presence_penalty: float = 0.0,
                  frequency_penalty: float = 0.0, seed: int = 0, ignore_eos: bool = False,
-                 eos_token_id: int | None = None) -> list:
-        """Token ids generated for each prompt (a list of token ids), in order."""
+                 eos_token_id=None) -> list:
+        """Token ids generated for each prompt (a list of token ids), in order.  `eos_token_id`: one id or a list
+        of ids that end a request (default: the model's own, which may be several)."""
         return [c.token_ids for c in self.generate_detailed(
             prompts, max_new_tokens, SamplingParams(temperature, top_k, top_p, repetition_penalty,
                                                     presence_penalty, frequency_penalty, seed),
             ignore_eos=ignore_eos, eos_token_id=eos_token_id)]
 
     def generate_detailed(self, prompts: list, max_new_tokens, params: SamplingParams | list | None = None,
-                          ignore_eos: bool = False, eos_token_id: int | None = None, on_token=None) -> list:
+                          ignore_eos: bool = False, eos_token_id=None, on_token=None) -> list:
         """`params` may be one `SamplingParams` for all or one per prompt; `max_new_tokens` likewise.
         Request i draws from a generator seeded with its own params.seed.  `on_token(i, token)` is called for
         every token that request i generates, in order, as soon as the host has read it (the reference prints

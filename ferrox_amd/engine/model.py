@@ -10,6 +10,22 @@ from ..parts.base import (BLOCKS, EMBEDDINGS, HEADS, NORMS, LayerCache, ModelSpe
 from ..weights.loader import check_names, upload
 
 
+class Fetcher:
+    """What a part's `load` receives: `fetch(local name)` for its own tensors, `fetch.shared(full name)` for one
+    that another part owns and this part has announced in `borrows()`."""
+
+    def __init__(self, get, prefix: str, shared: dict):
+        self._get, self._prefix, self._shared = get, prefix, shared
+
+    def __call__(self, local: str) -> torch.Tensor:
+        return self._get(self._prefix + local)
+
+    def shared(self, name: str) -> torch.Tensor:
+        if name not in self._shared:
+            raise KeyError(f"part '{self._prefix}' asks for '{name}' without having announced it in borrows()")
+        return self._get(name)
+
+
 class Model:
     def __init__(self, spec: ModelSpec):
         self.spec = spec
@@ -71,11 +87,26 @@ class Model:
             source.expect(self.named_params())
         check_names(self.named_params(), source, where)
         device = torch.device(device)
+        owned = self.named_params()
+        shared: dict = {}              # full name -> the one tensor that its owner and its borrowers get
         for prefix, root in self._roots():
             for pfx, part in walk_parts(root, prefix):
-                part.load(lambda local, _p=pfx: upload(source, _p + local, act_dtype, device))
-        if getattr(self.head, "tied", False):
-            self.head.tie(self.embedding)
+                for name in part.borrows():
+                    if name not in owned:
+                        raise ValueError(f"part '{pfx}' ({type(part).__name__}) reads the tensor '{name}', "
+                                         f"which no part of the model declares")
+                    shared[name] = None
+
+        def get(name: str) -> torch.Tensor:
+            if name not in shared:
+                return upload(source, name, act_dtype, device)
+            if shared[name] is None:
+                shared[name] = upload(source, name, act_dtype, device)
+            return shared[name]
+
+        for prefix, root in self._roots():
+            for pfx, part in walk_parts(root, prefix):
+                part.load(Fetcher(get, pfx, shared))
         self.act_dtype, self.device = act_dtype, device
 
     # ---- cache needs -----------------------------------------------------

@@ -45,7 +45,7 @@ class Request:
     prompt: list
     max_new_tokens: int
     params: SamplingParams = field(default_factory=SamplingParams)
-    eos_token_id: int | None = None
+    eos_token_id: object = None       # None, one token id, or several: each of them ends the request
     ignore_eos: bool = False
     # progress
     generated: list = field(default_factory=list)
@@ -59,6 +59,9 @@ class Request:
     def __post_init__(self):
         if self.rng is None:
             self.rng = XorShift64(self.params.seed)
+        eos = self.eos_token_id
+        self.stop_ids = frozenset() if eos is None else frozenset(
+            int(t) for t in (eos if isinstance(eos, (list, tuple, set, frozenset)) else (eos,)))
 
     @property
     def tokens(self) -> list:
@@ -210,7 +213,7 @@ class Scheduler:
             req, tok = s.request, int(sampled[s.request.id])
             if req.generated[s.place] != UNKNOWN:
                 raise RuntimeError(f"request {req.id!r}: token {s.place} was resolved twice")
-            if req.eos_token_id is not None and tok == req.eos_token_id and not req.ignore_eos:
+            if tok in req.stop_ids and not req.ignore_eos:
                 del req.generated[s.place:]
                 if req.status == "waiting":          # preempted meanwhile
                     self.waiting.remove(req)

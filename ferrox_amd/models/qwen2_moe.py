@@ -54,8 +54,9 @@ def build_spec(cfg: Qwen2MoeConfig, tensor_names=None) -> ModelSpec:
         layers=layers,
         schedule=[ScheduleEntry(l) for l in range(cfg.num_hidden_layers)],
         final_norm=PartSpec("rmsnorm", {"size": H, "eps": cfg.rms_norm_eps}, prefix="model.norm."),
-        head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "hidden_size": H,
-                                      "tied": cfg.tie_word_embeddings}, prefix="lm_head."),
+        head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "hidden_size": H,           # loader.rs:1433-1436
+                                      "tied_to": "model.embed_tokens.weight" if cfg.tie_word_embeddings else None},
+                      prefix="lm_head."),
         max_positions=cfg.max_position_embeddings,
         eos_token_id=cfg.eos_token_id,
     )

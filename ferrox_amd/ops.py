@@ -14,7 +14,9 @@ import torch
 from .csrc.build import load_library
 
 FX_F32, FX_BF16 = 0, 1
-EPI_STORE, EPI_STORE_F32, EPI_RESID, EPI_SILU_MUL = 0, 1, 2, 3
+EPI_STORE, EPI_STORE_F32, EPI_RESID, EPI_GATED = 0, 1, 2, 3
+# what the gate of a gated product goes through (EPI_GATED stores activation(gate) * up); ACT_* in csrc/gemm.hip
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}
 GATE_SOFTMAX, GATE_SIGMOID = 0, 1
 ROPE_NEOX, ROPE_INTERLEAVED = 0, 1
 
@@ -65,7 +67,7 @@ _sigs = {
     ("elementwise", "fx_feed_tokens"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int, c_int],
     ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
                               c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
@@ -268,13 +270,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          expert_offsets: torch.Tensor | None = None,
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
          norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
-         always: tuple | None = None, w_kblocked: bool = False, row_ss: tuple | None = None) -> torch.Tensor:
+         always: tuple | None = None, w_kblocked: bool = False, row_ss: tuple | None = None,
+         activation: str = "silu") -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
     EPI_STORE stores in a's dtype (+bias); EPI_STORE_F32 stores float32; EPI_RESID adds the
-    product (times row_scale[m]) into the float32 `out`; EPI_SILU_MUL multiplies two
-    matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores silu(gate)*up.
+    product (times row_scale[m]) into the float32 `out`; EPI_GATED multiplies two
+    matrices (rows [0, n_out) and [up_offset/K, ...) of w) and stores activation(gate) * up,
+    `activation` being one of ACTIVATIONS.
     `a_rows` gathers the rows of a; `n_rows` is the number of logical rows then.  `c_rows`
     scatters the rows of the output (row_scale stays indexed by the logical row).
     `pair_ids` (int32, up to 64 entries) replaces the sorted layout for
@@ -327,7 +331,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     if kw != K:
         raise KernelError(f"gemm: inner sizes differ, activations {K}, weights {kw}")
     M = n_rows if n_rows is not None else a.shape[0]
-    if epilogue == EPI_SILU_MUL:
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"gemm: activation '{activation}' is not one of {sorted(ACTIVATIONS)}")
+    if epilogue == EPI_GATED:
         N = n_out if n_out is not None else n_w // 2
         if up_offset == 0:
             up_offset = N * K
@@ -335,7 +341,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
             raise KernelError("gemm: gate/up rows exceed the weight matrix")
     else:
         N = n_out if n_out is not None else n_w
-    out_dtype = w.dtype if epilogue in (EPI_STORE, EPI_SILU_MUL) else torch.float32
+    out_dtype = w.dtype if epilogue in (EPI_STORE, EPI_GATED) else torch.float32
     out_rows = M + n_always * always_rows
     if out is None:
         if epilogue == EPI_RESID:
@@ -353,7 +359,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           float(norm[1]) if norm is not None else (float(row_ss[1]) if row_ss is not None else 0.0),
           _p(_i32(pair_ids, "pair_ids")), int(pair_div),
           n_always, always_rows, always_from_a, n_w if w_kblocked else 0,
-          _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0)
+          _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0,
+          ACTIVATIONS[activation])
     return out
 
 

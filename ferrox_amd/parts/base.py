@@ -20,7 +20,8 @@ Interfaces (all tensors on the GPU; `h` is the float32 residual stream [T, H],
                    forward(x, ctx, cache, residual) -> None   (adds its output into residual)
   FeedForward      forward(x, ctx, residual) -> None
   Block            forward(h, ctx, cache) -> None
-  every part       param_specs() -> {local name: ParamSpec}, load(fetch), kernel_libraries
+  every part       param_specs() -> {local name: ParamSpec}, load(fetch), kernel_libraries;
+                   borrows() -> [full names of tensors that other parts own and this one reads too]
 """
 from __future__ import annotations
 
@@ -70,7 +71,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_positions: int
-    eos_token_id: int | None = None
+    eos_token_id: int | tuple | None = None      # the id, or the ids, that end a generation
 
 
 # --------------------------------------------------------------------------
@@ -183,7 +184,14 @@ class Part:
 
     def load(self, fetch: Callable[[str], torch.Tensor]) -> None:
         """`fetch(local name)` returns the tensor on the device.  Floating tensors come
-        in the activation type, except those stored in float32, which stay float32."""
+        in the activation type, except those stored in float32, which stay float32.
+        `fetch.shared(full name)` returns a tensor that another part owns and `borrows()` has announced:
+        the same memory that its owner gets, uploaded once."""
+
+    def borrows(self) -> list:
+        """Full names of tensors that other parts declare and this part reads as well (a head tied to
+        the embedding table).  The model checks that someone owns them and uploads each once."""
+        return []
 
     def children(self) -> list:
         """Sub-parts as [(prefix, part)]; a child's tensors are named prefix + its local names."""

@@ -30,19 +30,24 @@ class TokenEmbedding(Part):
 class LinearHead(Part):
     kernel_libraries = ("gemm",)
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
-        self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: str | None = None):
+        """`tied_to`: the full name of another part's [vocab, hidden] tensor that serves as this head's matrix (the
+        embedding table of a model with tied embeddings); the head then has no tensor of its own."""
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tied_to = tied_to or None
         self.weight = None
 
     def param_specs(self):
-        return {} if self.tied else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {} if self.tied_to else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def borrows(self):
+        return [self.tied_to] if self.tied_to else []
 
     def load(self, fetch):
-        if not self.tied:
-            self.weight = fetch("weight").contiguous()
-
-    def tie(self, embedding: TokenEmbedding):
-        self.weight = embedding.weight
+        self.weight = (fetch.shared(self.tied_to) if self.tied_to else fetch("weight")).contiguous()
+        if tuple(self.weight.shape) != (self.vocab_size, self.hidden_size):
+            raise ValueError(f"the head's matrix {self.tied_to or 'weight'} has shape {tuple(self.weight.shape)}, "
+                             f"not [{self.vocab_size}, {self.hidden_size}]")
 
     def forward(self, x):
         """float32 logits [rows, vocab]."""

@@ -14,7 +14,7 @@ import torch
 from .. import debug, limits, ops
 from .base import FEED_FORWARDS, FeedForward, ParamSpec
 from .linear import matmul, same_dtype
-from .mlp import SwiGLU
+from .mlp import GatedMLP
 
 GATINGS = {"softmax": ops.GATE_SOFTMAX, "sigmoid": ops.GATE_SIGMOID}
 FRONT_MAX_TOKENS = 128       # up to so many tokens the norm, the router, the selection and the sort are one launch (the
@@ -40,7 +40,7 @@ class SparseMoE(FeedForward):
 
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
                  norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
-                 shared_gate: bool = True):
+                 shared_gate: bool = True, activation: str = "silu"):
         if not 1 <= top_k <= n_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{n_experts}")
         if n_experts > limits.MOE_MAX_EXPERTS or top_k > limits.MOE_MAX_TOP_K:
@@ -48,10 +48,13 @@ class SparseMoE(FeedForward):
                              f"{limits.MOE_MAX_EXPERTS} experts and {limits.MOE_MAX_TOP_K} per token")
         if gating not in GATINGS:
             raise ValueError(f"gating '{gating}' is not one of {sorted(GATINGS)}")
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation '{activation}' is not one of {sorted(ops.ACTIVATIONS)}")
+        self.activation = activation
         self.hidden_size, self.n_experts, self.top_k = int(hidden_size), int(n_experts), int(top_k)
         self.expert_intermediate_size = int(expert_intermediate_size)
         self.norm_topk_prob, self.gating = bool(norm_topk_prob), GATINGS[gating]
-        self.shared = SwiGLU(hidden_size, shared_intermediate_size) if shared_intermediate_size > 0 else None
+        self.shared = GatedMLP(hidden_size, shared_intermediate_size, activation) if shared_intermediate_size > 0 else None
         self.has_shared_gate = bool(shared_gate) and self.shared is not None
         self.router = self.w_gate_up = self.w_down = None
 
@@ -157,7 +160,7 @@ class SparseMoE(FeedForward):
             S, n = sorted_pieces, ids.numel()
             kb = dict(w_kblocked=True) if self.kblocked else {}
             debug.region("experts gate/up")
-            act = matmul(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets,
+            act = matmul(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, activation=self.activation, a_rows=sorted_token, expert_offsets=offsets,
                          n_rows=n + S * T, **kb)
             debug.region("experts down")
             y = matmul(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
@@ -172,7 +175,7 @@ class SparseMoE(FeedForward):
                 debug.routing_trace.put(ids)
             S, n = self.shared_pieces, ids.numel()
             debug.region("experts gate/up")
-            act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k,
+            act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, activation=self.activation, pair_ids=ids, pair_div=self.top_k,
                            always=(S, T, True), w_kblocked=self.kblocked)
             debug.region("experts down")
             y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False),
@@ -226,11 +229,11 @@ class SparseMoE(FeedForward):
         kb = dict(w_kblocked=True) if self.kblocked else {}
         debug.region("experts gate/up")
         if offsets is None:      # few pairs, unsorted: row p of `act` and of `y` is pair p
-            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=self.top_k, **kb)
+            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_GATED, activation=self.activation, pair_ids=ids, pair_div=self.top_k, **kb)
             debug.region("experts down")
             y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids, **kb)
         else:
-            act = matmul(x, self.w_gate_up, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token,
+            act = matmul(x, self.w_gate_up, epilogue=ops.EPI_GATED, activation=self.activation, a_rows=sorted_token,
                          expert_offsets=offsets, n_rows=T * self.top_k, **kb)
             debug.region("experts down")
             # each expert's rows go back to the place of their (token, slot) pair

@@ -1,16 +1,31 @@
 """Binding checkpoint tensors to a model's parameters by name.
 
 The model says which tensors it wants (name, shape); the source says which it
-has.  Everything that does not fit — missing tensors, tensors nobody asked for,
-wrong shapes, unusable dtypes — is collected into ONE `CheckpointError`
-(the reference stops at the first: ferrox-models/src/loader.rs:38-65).
+has.  Everything that does not fit — missing tensors, wrong shapes, unusable
+dtypes — is collected into ONE `CheckpointError` (the reference stops at the
+first: ferrox-models/src/loader.rs:38-65).  Tensors that the file holds and the
+model does not ask for are not an error (the reference never looks at them
+either: it fetches by name, loader.rs:564-629); they are listed in one
+`UnexpectedTensorsWarning`, and in the error if there is one.
 Floating tensors are uploaded in the activation type, except that a tensor the
 file stores in 32 bits stays float32 under bfloat16 activations; integer tables
 become int32.
 """
 from __future__ import annotations
 
+import warnings
+
 import torch
+
+
+class UnexpectedTensorsWarning(UserWarning):
+    """The checkpoint holds tensors that the model does not ask for; `names` lists them."""
+
+    def __init__(self, names, where=""):
+        self.names = list(names)
+        shown = ", ".join(self.names[:12]) + (f", ... and {len(self.names) - 12} more" if len(self.names) > 12 else "")
+        super().__init__(f"checkpoint {where} holds {len(self.names)} tensors that the model does not use: {shown}"
+                         .replace("  ", " "))
 
 
 class CheckpointError(ValueError):
@@ -38,8 +53,9 @@ FLOATS = (torch.float64, torch.float32, torch.float16, torch.bfloat16)
 INTS = (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8)
 
 
-def check_names(expected: dict, source, where: str = "") -> None:
-    """`expected`: full name -> ParamSpec."""
+def check_names(expected: dict, source, where: str = "") -> list:
+    """`expected`: full name -> ParamSpec.  Returns the names that the source holds beyond them (after a warning
+    that lists them)."""
     have = set(source.names())
     missing = sorted(n for n in expected if n not in have)
     unexpected = sorted(n for n in have if n not in expected)
@@ -54,8 +70,11 @@ def check_names(expected: dict, source, where: str = "") -> None:
             wrong_dtype.append((n, f"stored as {dt}, the model wants an integer table"))
         if not spec.integer and dt not in FLOATS:
             wrong_dtype.append((n, f"stored as {dt}, the model wants floating point"))
-    if missing or unexpected or wrong_shape or wrong_dtype:
+    if missing or wrong_shape or wrong_dtype:
         raise CheckpointError(missing, unexpected, wrong_shape, wrong_dtype, where)
+    if unexpected:
+        warnings.warn(UnexpectedTensorsWarning(unexpected, where), stacklevel=2)
+    return unexpected
 
 
 def resident_dtype(stored: torch.dtype, act_dtype: torch.dtype) -> torch.dtype:

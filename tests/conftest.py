@@ -100,7 +100,7 @@ def model_folders(tmp_path_factory):
         key projections (weights and biases) are multiplied by it after they are drawn, which makes attention
         peaked, so that where a key lies and how exactly it is rotated shows in the logits.  `overrides` replace
         keys of the configuration."""
-        key = (name, dtype, std, qk_scale, tuple(sorted(overrides.items())))
+        key = (name, dtype, std, qk_scale, repr(sorted(overrides.items())))
         if key not in made:
             from ferrox_amd.engine.loading import write_random_model
             cfg, seed = TINY[name]

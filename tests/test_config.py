@@ -57,6 +57,8 @@ def test_defaults_are_reported():
     ({"num_experts": 64, "num_experts_per_tok": 33}, "num_experts_per_tok"),
     ({"use_sliding_window": True, "sliding_window": 0, "max_window_layers": 0}, "sliding_window"),
     ({"rms_norm_eps": -1.0}, "rms_norm_eps"),
+    ({"eos_token_id": "stop"}, "eos_token_id"),
+    ({"eos_token_id": [3, 4.5]}, "eos_token_id"),
 ])
 def test_bad_configs_are_refused_with_the_key_named(patch, word):
     raw = dict(TINY_A)
@@ -65,6 +67,16 @@ def test_bad_configs_are_refused_with_the_key_named(patch, word):
     with pytest.raises(ConfigError) as e:
         Qwen2MoeConfig.from_dict(raw)
     assert word in str(e.value)
+
+
+def test_stop_ids_are_one_or_several():
+    one = Qwen2MoeConfig.from_dict(dict(TINY_A, eos_token_id=7))
+    two = Qwen2MoeConfig.from_dict(dict(TINY_A, eos_token_id=[7, 9]))
+    assert one.eos_token_id == 7 and two.eos_token_id == (7, 9)
+    assert Qwen2MoeConfig.from_dict(dict(TINY_A, eos_token_id=[7])).eos_token_id == 7
+    assert Qwen2MoeConfig.from_dict(dict(TINY_A)).eos_token_id is None
+    assert two.to_dict()["eos_token_id"] == [7, 9] and Qwen2MoeConfig.from_dict(two.to_dict()) == two
+    assert build_spec(two).eos_token_id == (7, 9)
 
 
 def test_registry_is_closed(tmp_path):
@@ -89,7 +101,7 @@ def test_spec_is_chosen_layer_by_layer():
     assert kinds == [("paged_attention", "swiglu", None), ("paged_attention", "sparse_moe", 16),
                      ("paged_attention", "swiglu", 16)]
     assert spec.layers[1].parts["ffn"].args["top_k"] == 3 and spec.layers[0].parts["ffn"].args["intermediate_size"] == 160
-    assert spec.head.args["tied"] is True and [e.layer for e in spec.schedule] == [0, 1, 2]
+    assert spec.head.args["tied_to"] == "model.embed_tokens.weight" and [e.layer for e in spec.schedule] == [0, 1, 2]
     # q/k/v bias not stated in the config: decided by what the checkpoint holds
     assert build_spec(Qwen2MoeConfig.from_dict(TINY_B), ["model.layers.0.self_attn.q_proj.weight"]) \
         .layers[0].parts["mixer"].args["bias"] is False

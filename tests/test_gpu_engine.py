@@ -736,6 +736,109 @@ def test_command_line_generates_and_refuses(model_folders, tmp_path):
     refused(run_cli("-m", folder, "--tokens", ",".join(["1"] * 300), "--dtype", "fp32"), "context")
 
 
+def test_command_line_text_prompts_and_random_weights(model_folders, tmp_path):
+    """The text path (ferrox-cli/src/run.rs:561-571, 651-676): -p, -f and -e with a tokenizer.json in the model
+    folder (a word-level tokenizer that the test builds), text streamed to stdout equal to the decoded tokens of
+    the plain model's greedy generation; and --random-weights --seed N with a configuration file, which makes the
+    weights that `write_random_model` writes for the same seed (the reference serves synthetic weights when no
+    model is given, ferrox-server/src/model.rs:228-243)."""
+    import shutil
+    import plain_qwen2moe as plain
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from ferrox_amd.engine.loading import write_random_model
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(model_folders("A", "float32"), folder)
+    cfg, w = plain.load_folder(folder)
+    words = ["<unk>", "the", "cat", "sat", "on", "a", "mat", "and", "purred"] + [f"w{i}" for i in range(9, cfg["vocab_size"])]
+    tok = Tokenizer(models.WordLevel({word: i for i, word in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    text = "the cat sat on a mat and purred w200 w77"
+    prompt = tok.encode(text).ids
+    assert prompt == [1, 2, 3, 4, 5, 6, 7, 8, 200, 77]
+    want = plain.greedy_generate(cfg, w, prompt, 12)
+    assert telling(want, 6), want
+    common = ["-n", "12", "--temp", "0", "--repeat-penalty", "1", "--dtype", "fp32", "--block-size", "16"]
+    by_p = run_cli("-m", folder, "-p", text, "--verbose-prompt", *common)
+    assert by_p.returncode == 0, by_p.stderr[-2000:]
+    assert by_p.stdout.rstrip("\n") == tok.decode(want), (by_p.stdout, tok.decode(want))
+    assert str(prompt) in by_p.stderr                                        # --verbose-prompt
+    (tmp_path / "prompt.txt").write_text(text + "\n")
+    by_f = run_cli("-m", folder, "-f", str(tmp_path / "prompt.txt"), *common)
+    assert by_f.returncode == 0 and by_f.stdout == by_p.stdout, by_f.stderr[-2000:]
+    escaped = run_cli("-m", folder, "-e", "-p", "the cat\\nsat on\\ta mat and purred w200 w77", *common)
+    assert escaped.returncode == 0 and escaped.stdout == by_p.stdout, escaped.stderr[-2000:]
+    raw = run_cli("-m", folder, "-p", "the cat\\nsat", *common)            # without -e the backslash stays: other tokens
+    assert raw.returncode == 0 and raw.stdout != by_p.stdout
+    # a tokenizer named on the command line, for a folder that has none
+    bare = model_folders("A", "float32")
+    named = run_cli("-m", bare, "--tokenizer", os.path.join(folder, "tokenizer.json"), "-p", text, *common)
+    assert named.returncode == 0 and named.stdout == by_p.stdout, named.stderr[-2000:]
+    none = run_cli("-m", bare, "-p", text, *common)
+    assert none.returncode == 2 and "tokenizer" in none.stderr and none.stdout == ""
+    # random weights from a seed: the tensors that write_random_model writes for that seed
+    cfg_file = tmp_path / "tiny_a.json"
+    cfg_file.write_text(json.dumps(TINY["A"][0]))
+    seeded = str(tmp_path / "seed_321")
+    write_random_model(dict(TINY["A"][0]), seeded, 321, "float32", device="cuda:0")
+    ids = ",".join(map(str, prompt))
+    from_folder = run_cli("-m", seeded, "--tokens", ids, *common)
+    from_seed = run_cli("--random-weights", "--seed", "321", "--config", str(cfg_file), "--tokens", ids, *common)
+    assert from_folder.returncode == 0 and from_seed.returncode == 0, from_seed.stderr[-2000:]
+    assert from_seed.stdout == from_folder.stdout and "seed 321" in from_seed.stderr
+    got = [int(t) for t in from_seed.stdout.strip().split(",")]
+    assert got == plain.greedy_generate(*plain.load_folder(seeded), prompt, 12) and got != want
+    other = run_cli("--random-weights", "--seed", "322", "--config", str(cfg_file), "--tokens", ids, *common)
+    assert other.returncode == 0 and other.stdout != from_seed.stdout
+    # a named shape, cut to one layer so that it is made in a moment
+    named_shape = run_cli("--random-weights", "--seed", "1", "--config", "qwen1.5-moe-a2.7b", "--layers", "1", "--tokens",
+                          "5,17,150000", "-n", "4", "--temp", "0")
+    assert named_shape.returncode == 0 and len(named_shape.stdout.strip().split(",")) == 4, named_shape.stderr[-2000:]
+    for bad, word in ((["--tokens", ids], "either"), (["-m", folder, "--random-weights", "--tokens", ids], "either"),
+                      (["--random-weights", "--config", "no-such-shape", "--tokens", ids], "no-such-shape")):
+        refused = run_cli(*bad)
+        assert refused.returncode == 2 and word in refused.stderr and "Traceback" not in refused.stderr, refused.stderr[-2000:]
+
+
+def test_a_checkpoint_with_tensors_nobody_asked_for_still_runs(model_folders, tmp_path):
+    """a folder whose file holds more tensors than the model wants loads with one warning that lists them, and
+    generates what the folder without them generates"""
+    from safetensors.torch import load_file, save_file
+    from ferrox_amd.engine.api import Engine
+    from ferrox_amd.weights import UnexpectedTensorsWarning
+    import shutil
+    folder = str(tmp_path / "more")
+    shutil.copytree(model_folders("A", "float32"), folder)
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, path)
+    prompts = [[5, 17, 3, 250, 9]]
+    with pytest.warns(UnexpectedTensorsWarning, match="rotary_emb.inv_freq"):
+        engine = Engine(folder, dtype="float32", block_size=16, num_pages=8, max_seqs=1)
+    clean = Engine(model_folders("A", "float32"), dtype="float32", block_size=16, num_pages=8, max_seqs=1)
+    assert engine.generate(prompts, max_new_tokens=8) == clean.generate(prompts, max_new_tokens=8)
+
+
+def test_generation_stops_on_any_of_the_models_stop_ids(model_folders):
+    """config.json may give several stop ids (`eos_token_id: [a, b]`): the request ends on whichever comes first"""
+    import plain_qwen2moe as plain
+    from ferrox_amd.engine.api import Engine
+    base = model_folders("A", "float32")
+    cfg, w = plain.load_folder(base)
+    prompt = [5, 17, 3, 250, 9]
+    free = plain.greedy_generate(cfg, w, prompt, 8)
+    assert len(set(free[:6])) == 6, free
+    folder = model_folders("A", "float32", eos_token_id=[free[5], free[3]])
+    engine = Engine(folder, dtype="float32", block_size=16, num_pages=8, max_seqs=2)
+    assert engine.eos_token_id == (free[5], free[3])
+    got = engine.generate_detailed([prompt, prompt], [8, 3])
+    assert (got[0].token_ids, got[0].finish_reason) == (free[:3], "stop")
+    assert (got[1].token_ids, got[1].finish_reason) == (free[:3], "length")
+    assert engine.generate([prompt], max_new_tokens=8, eos_token_id=free[5]) == [free[:5]]
+    assert engine.generate([prompt], max_new_tokens=8, ignore_eos=True) == [free]
+
+
 def test_generation_of_a_batch_that_shrinks(model_folders):
     """twelve requests that ask for different numbers of tokens, through the entry point: the decode batch shrinks one
     request at a time through the recorded sizes (16 with stand-in rows, then 8 and below as they are), and every

@@ -111,7 +111,7 @@ def test_gemm_every_wide_tile(tile, M, N, K):
         got = ops.gemm(a, w, bias=bias)
         ops.gemm(a, w, epilogue=ops.EPI_RESID, out=h)
         w2 = rnd(2 * N, K, dtype=dtype, seed=4, scale=0.5)
-        act = ops.gemm(a, w2, epilogue=ops.EPI_SILU_MUL)
+        act = ops.gemm(a, w2, epilogue=ops.EPI_GATED)
     close(got, ref + bias.double(), dtype, "store+bias")
     close(h, h0.double() + ref, dtype, "residual")
     close(act, plain.silu(a.double() @ w2[:N].double().T) * (a.double() @ w2[N:].double().T), dtype, "silu(gate)*up")
@@ -131,7 +131,7 @@ def test_grouped_gemm_tiles_agree(tile):
     ids = torch.stack([first, 2 + torch.randint(0, E - 2, (T,), generator=g)], dim=1).to(torch.int32).to(DEV)
     offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
     with debug.kernel_switch("gemm", "wide", tile):
-        act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+        act = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
     xs = x.double()[sorted_token.long()]
     off = offsets.cpu().tolist()
     assert off[1] - off[0] > 256
@@ -148,7 +148,16 @@ def test_gemm_gate_up(dtype, M, I, K):
     from ferrox_amd import ops
     a, w = rnd(M, K, dtype=dtype), rnd(2 * I, K, dtype=dtype, seed=1, scale=0.5)
     g, u = a.double() @ w[:I].double().T, a.double() @ w[I:].double().T
-    close(ops.gemm(a, w, epilogue=ops.EPI_SILU_MUL), plain.silu(g) * u, dtype, "silu(gate)*up")
+    close(ops.gemm(a, w, epilogue=ops.EPI_GATED), plain.silu(g) * u, dtype, "silu(gate)*up")
+    # the gate's activation is a parameter of the call: every kernel that has the epilogue takes every activation
+    others = {"gelu_tanh": lambda z: 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3))),
+              "gelu": lambda z: 0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0))), "relu": lambda z: z.clamp(min=0.0),
+              "silu": plain.silu}
+    assert set(others) == set(ops.ACTIVATIONS)
+    for name, f in others.items():
+        close(ops.gemm(a, w, epilogue=ops.EPI_GATED, activation=name), f(g) * u, dtype, f"{name}(gate)*up")
+    with pytest.raises(ops.KernelError, match="activation"):
+        ops.gemm(a, w, epilogue=ops.EPI_GATED, activation="swish2")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -175,7 +184,7 @@ def test_grouped_gemm_and_routing_buffers(dtype, T, E, k, I, H):
     for e in range(E):
         seg = [i for i in range(T * k) if int(ids_c.flatten()[i]) == e]
         assert [int(inv_c[i]) for i in seg] == list(range(int(offsets[e]), int(offsets[e + 1])))
-    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
     y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets)
     h = torch.zeros(T, H, device=DEV)
     ops.moe_combine(h, y, inv, wts, k)
@@ -210,9 +219,9 @@ def test_grouped_gemm_from_unsorted_pairs(T, E, k, I, H):
     if T >= 8 and E >= 8:
         ids[:, 0] = 5            # one expert with a row of every token
     offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
-    act_s = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    act_s = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
     y_s = ops.gemm(act_s, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
-    act_p = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k)
+    act_p = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=k)
     y_p = ops.gemm(act_p, w_dn, epilogue=ops.EPI_STORE_F32, pair_ids=ids)
     assert torch.equal(act_p, act_s[inv.long()])
     assert torch.equal(y_p, y_s)
@@ -240,11 +249,11 @@ def test_shared_expert_as_pieces_beside_unsorted_pairs(T, E, k, I, H, S):
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
     wts, gate = torch.rand(T, k, generator=g).to(DEV), torch.rand(T, generator=g).to(DEV)
     n = T * k
-    act = ops.gemm(x, gu_all, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k, always=(S, T, True))
+    act = ops.gemm(x, gu_all, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=k, always=(S, T, True))
     y = ops.gemm(act, dn_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False))
     assert act.shape == (n + S * T, I) and y.shape == (n + S * T, H)
     # the routed rows are what the products without the pieces give
-    assert torch.equal(act[:n], ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k))
+    assert torch.equal(act[:n], ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=k))
     h = torch.zeros(T, H, device=DEV)
     ops.moe_combine(h, y[:n], None, wts, k, shared=y[n:].view(S, T, H), gate=gate)
     xd = x.double().cpu()
@@ -273,16 +282,16 @@ def test_weights_in_slabs_of_64_k(T, E, k, I, H):
     g = torch.Generator().manual_seed(17)
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
     offsets, sorted_token, sorted_pair, inv = ops.moe_align(ids, E)
-    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
-    act_kb = ops.gemm(x, kb_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k,
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+    act_kb = ops.gemm(x, kb_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k,
                       w_kblocked=True)
     assert torch.equal(act, act_kb)
     y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
     y_kb = ops.gemm(act, kb_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, w_kblocked=True)
     assert torch.equal(y, y_kb)
     if T * k <= 64:
-        assert torch.equal(ops.gemm(x, kb_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k, w_kblocked=True),
-                           ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, pair_ids=ids, pair_div=k))
+        assert torch.equal(ops.gemm(x, kb_gu, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=k, w_kblocked=True),
+                           ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=k))
     # a plain matrix with bias, stored, and added into a residual
     bias = rnd(2 * I, dtype=dtype, seed=3)
     assert torch.equal(ops.gemm(x, kb_gu[0], bias=bias, w_kblocked=True), ops.gemm(x, w_gu[0], bias=bias))
@@ -871,7 +880,7 @@ def test_sort_by_expert_with_experts_that_every_token_takes(T, E, k, S):
     H, I = 64, 32
     x = rnd(T, H, dtype=torch.bfloat16)
     w_gu, w_dn = rnd(E + S, 2 * I, H, dtype=torch.bfloat16, seed=1, scale=0.3), rnd(E + S, H, I, dtype=torch.bfloat16, seed=2, scale=0.3)
-    act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=n + S * T)
+    act = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=n + S * T)
     y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
     assert y.shape == (n + S * T, H)
     xd = x.double().cpu()
@@ -938,7 +947,7 @@ def test_sorted_experts_through_either_product(T, E, k, I, H):
     outs = []
     for few in (3, 64):
         with debug.kernel_switch("gemm", "few_rows", few):
-            act = ops.gemm(x, w_gu, epilogue=ops.EPI_SILU_MUL, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
+            act = ops.gemm(x, w_gu, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets, n_rows=T * k)
             y = ops.gemm(act, w_dn, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair)
         close(y, ref, dtype, f"sorted experts, few_rows {few}", k=I)
         outs.append(y)

@@ -85,6 +85,19 @@ def test_eos_stops_without_being_appended_and_can_be_ignored():
     assert (a.finish_reason, a.generated) == ("stop", [4]) and (b.finish_reason, b.generated) == ("length", [4, 9, 9])
 
 
+def test_any_of_several_stop_ids_ends_a_request():
+    """chat variants of this family stop on either of two ids (config.json gives a list)"""
+    sched = Scheduler(Cache(64))
+    sched.add(Request("a", [1, 2], max_new_tokens=9, eos_token_id=[9, 11]))
+    sched.add(Request("b", [1, 2], max_new_tokens=9, eos_token_id=(11, 9)))
+    sched.add(Request("c", [1, 2], max_new_tokens=4, eos_token_id=[9, 11], ignore_eos=True))
+    sched.add(Request("d", [1, 2], max_new_tokens=4, eos_token_id=[]))            # no stop id at all
+    picks = {"a": [4, 5, 11, 4], "b": [4, 9, 4, 4], "c": [9, 11, 4, 4], "d": [9, 11, 4, 4]}
+    run(sched, lambda req: picks[req.id][len(req.generated)])
+    by = {r.id: (r.finish_reason, r.generated) for r in sched.finished}
+    assert by == {"a": ("stop", [4, 5]), "b": ("stop", [4]), "c": ("length", [9, 11, 4, 4]), "d": ("length", [9, 11, 4, 4])}
+
+
 def test_bad_requests_are_refused():
     sched = Scheduler(Cache(8), context_limit=10, vocab_size=50)
     with pytest.raises(ValueError):

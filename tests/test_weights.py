@@ -124,6 +124,32 @@ def test_one_error_lists_everything_that_does_not_fit(tmp_path):
         assert word in msg
 
 
+def test_tensors_nobody_asked_for_are_a_warning(tmp_path):
+    """A file that holds more than the model wants still loads (the reference fetches by name and never looks at
+    the rest, ferrox-models/src/loader.rs:564-629); one warning lists what is left over."""
+    import warnings
+    from ferrox_amd.weights import UnexpectedTensorsWarning
+    folder = str(tmp_path / "m")
+    write_random_model(dict(TINY_A), folder, 0, "float32")
+    ck = Checkpoint(folder)
+    model = Model(build_spec(Qwen2MoeConfig.from_dict(TINY_A), ck.names()))
+    tensors = {n: ck.tensor(n).clone() for n in ck.names()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    more = str(tmp_path / "more")
+    os.makedirs(more)
+    write_safetensors(more + "/model.safetensors", tensors)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        left = check_names(model.named_params(), Checkpoint(more), more)
+    assert left == ["model.layers.0.self_attn.rotary_emb.inv_freq", "model.layers.1.self_attn.rotary_emb.inv_freq"]
+    mine = [w for w in caught if issubclass(w.category, UnexpectedTensorsWarning)]
+    assert len(mine) == 1 and mine[0].message.names == left and "layers.1.self_attn.rotary_emb.inv_freq" in str(mine[0].message)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert check_names(model.named_params(), ck) == []          # nothing left over: no warning
+
+
 def test_resident_dtypes():
     bf, f32 = torch.bfloat16, torch.float32
     assert resident_dtype(bf, bf) == bf and resident_dtype(torch.float16, bf) == bf
