@@ -26,8 +26,10 @@ int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void* out, 
 // its inputs and its output, and neither it nor anything it calls allocates or frees.  It refuses shapes whose
 // partial results, n_items * nh * splits * (hd + 2) floats, exceed fx_attn_static_capacity().  All calls on one GPU
 // share that GPU's array: calls that overlap on one GPU race; calls in stream order do not.
-// fx_attn_static_init() looks the array's address up for the current device ahead of the first call (the first
-// call on a device does it otherwise).
+// The array used is that of the device that `stream` belongs to (null: the current device).
+// fx_attn_static_init() looks the array's address up for the current device ahead of the first call; the first
+// call on a device does it otherwise, except under stream capture, where the lookup is refused with an error:
+// call fx_attn_static_init() with the stream's device current before a capture that holds this call.
 int fx_attn_decode_static(void* stream, int dtype, const void* q, long ldq, void* out, long ldo, const void* k_pages,
                           const void* v_pages, const int* block_table, int max_blocks, const int* positions,
                           const int* item_seq, const int* item_tok, int n_items, int nh, int nkv, int hd, int bs, int window,

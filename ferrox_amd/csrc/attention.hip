@@ -1075,7 +1075,10 @@ static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const vo
 }
 
 // ---------------------------------------------------------------------------
-static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window) {
+static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale) {
+    // (the bfloat16 kernels take a row's maximum over the raw scores and scale it once, which is the maximum of
+    // the scaled scores only under a positive scale)
+    FX_REQUIRE(scale > 0.f && scale < INFINITY, "%s: the scale of the scores must be positive and finite, got %g", who, (double)scale);
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "%s: unknown dtype %d", who, dtype);
     FX_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: n_heads %d must be a multiple of n_kv_heads %d", who, nh, nkv);
     FX_REQUIRE(hd > 0 && hd <= HD_MAX, "%s: head_dim %d is outside 1..%d", who, hd, HD_MAX);
@@ -1096,7 +1099,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
                          int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q) {
-    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window)) return 1;
+    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale)) return 1;
     FX_REQUIRE(tile_q == 64 || (tile_q == 128 && wide_items_ok(dtype, hd, bs) && mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)),
                "attn_tiles: items of %d queries (64, or 128 where fx_attn_tile_queries says so)", tile_q);
     if (n_items <= 0) return 0;
@@ -1112,7 +1115,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     // no more blocks than CUs: a block's chain of tiles is what takes the time, and two groups of waves halve it
     // (measured: 512-token portions at depth 8k-24k 130 and 360 us against 214 and 616 us; from 448 blocks on, one
     // group and two blocks to a CU are as fast or faster)
-    const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= 256;
+    const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
@@ -1182,8 +1185,8 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     return 0;
 }
 
-static int attn_decode_check(int dtype, int nh, int nkv, int hd, int bs, int window, int splits, int chunk) {
-    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window)) return 1;
+static int attn_decode_check(int dtype, int nh, int nkv, int hd, int bs, int window, float scale, int splits, int chunk) {
+    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale)) return 1;
     FX_REQUIRE(splits > 0 && chunk > 0 && chunk % 64 == 0, "attn_decode: chunk %d must be a positive multiple of 64", chunk);
     FX_REQUIRE(splits <= 8192, "attn_decode: %d chunks are more than the merge kernel takes (8192)", splits);
     return 0;
@@ -1194,7 +1197,7 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
                           float* part_o, float* part_ml, int splits, int chunk, int waves) {
-    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, splits, chunk)) return 1;
+    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
@@ -1215,17 +1218,37 @@ static __device__ __align__(256) float fx_attn_scratch[FX_ATTN_STATIC_FLOATS];
 #define FX_MAX_DEVICES 64
 static float* g_attn_scratch_ptr[FX_MAX_DEVICES];    // per device: the address of that device's copy (null: not asked yet)
 
-// The array's name is only a host-side stand-in; its memory on the current device is found with
-// hipGetSymbolAddress, once per device, with that device current.
-static int attn_scratch_of_current_device(float** out) {
-    int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
+// The array's name is only a host-side stand-in; its memory on a device is found with hipGetSymbolAddress, once
+// per device, with that device current.  `stream`: the stream a call is for (its device is the one whose copy is
+// used; null: the current device).  While `stream` is being captured nothing is looked up: the address must be
+// known by then, through fx_attn_static_init() or an earlier call on that device.
+static int attn_scratch_of(hipStream_t stream, float** out) {
+    int current = -1, dev = -1;
+    hipError_t e = hipGetDevice(&current);
     FX_REQUIRE(e == hipSuccess, "attn_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+    dev = current;
+    if (stream) {
+        e = hipStreamGetDevice(stream, &dev);
+        FX_REQUIRE(e == hipSuccess, "attn_decode_static: hipStreamGetDevice: %s", hipGetErrorString(e));
+    }
     FX_REQUIRE(dev >= 0 && dev < FX_MAX_DEVICES, "attn_decode_static: device %d is beyond the %d this library keeps", dev, FX_MAX_DEVICES);
     float* p = __atomic_load_n(&g_attn_scratch_ptr[dev], __ATOMIC_ACQUIRE);
     if (!p) {
+        if (stream) {
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            e = hipStreamIsCapturing(stream, &capturing);
+            FX_REQUIRE(e == hipSuccess, "attn_decode_static: hipStreamIsCapturing: %s", hipGetErrorString(e));
+            FX_REQUIRE(capturing == hipStreamCaptureStatusNone,
+                       "attn_decode_static: the stream is being captured and device %d's array has not been looked up yet; "
+                       "call fx_attn_static_init() with that device current before the capture begins", dev);
+        }
+        if (dev != current) {
+            e = hipSetDevice(dev);
+            FX_REQUIRE(e == hipSuccess, "attn_decode_static: hipSetDevice(%d): %s", dev, hipGetErrorString(e));
+        }
         void* sym = nullptr;
         e = hipGetSymbolAddress(&sym, HIP_SYMBOL(fx_attn_scratch));
+        if (dev != current) (void)hipSetDevice(current);
         FX_REQUIRE(e == hipSuccess && sym, "attn_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
         p = (float*)sym;
         __atomic_store_n(&g_attn_scratch_ptr[dev], p, __ATOMIC_RELEASE);     // (two threads would store the same address)
@@ -1234,9 +1257,11 @@ static int attn_scratch_of_current_device(float** out) {
     return 0;
 }
 
+// The array's address on the current device, looked up now (no allocation; call it once per device before calls
+// that are captured into a graph).
 FX_API int fx_attn_static_init(void) {
     float* p;
-    return attn_scratch_of_current_device(&p);
+    return attn_scratch_of(nullptr, &p);
 }
 
 FX_API long fx_attn_static_capacity(void) { return (long)FX_ATTN_STATIC_FLOATS; }
@@ -1245,7 +1270,7 @@ FX_API int fx_attn_decode_static(void* stream, int dtype, const void* q, long ld
                                  const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                                  const int* positions, const int* item_seq, const int* item_tok, int n_items,
                                  int nh, int nkv, int hd, int bs, int window, float scale, int splits, int chunk, int waves) {
-    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, splits, chunk)) return 1;
+    if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
     if (n_items <= 0) return 0;
     const size_t n_o = (size_t)n_items * nh * splits * hd, n_ml = (size_t)n_items * nh * splits * 2;
     FX_REQUIRE(n_o + n_ml <= FX_ATTN_STATIC_FLOATS,
@@ -1253,7 +1278,7 @@ FX_API int fx_attn_decode_static(void* stream, int dtype, const void* q, long ld
                "point holds; use fewer chunks or fx_attn_decode with buffers of your own",
                n_items, nh, splits, hd, n_o + n_ml, FX_ATTN_STATIC_FLOATS);
     float* scratch = nullptr;
-    if (attn_scratch_of_current_device(&scratch)) return 1;
+    if (attn_scratch_of((hipStream_t)stream, &scratch)) return 1;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, scratch, scratch + n_o, splits,
                               chunk, waves);

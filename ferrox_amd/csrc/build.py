@@ -27,7 +27,11 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
 HOST_LIBRARIES = ("host_runtime",)
-LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling", "probe") + HOST_LIBRARIES
+KERNEL_LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling")      # what parts of a model may name
+# kernels for measurement only (a streaming read, a copy, a loop of MFMA products, a marker): bench.py loads them,
+# no model can ask for them; their sources lie in measure/
+MEASUREMENT_LIBRARIES = ("probe",)
+LIBRARIES = KERNEL_LIBRARIES + MEASUREMENT_LIBRARIES + HOST_LIBRARIES            # what `compile_all` builds
 HEADERS = ("common.h",)
 
 _loaded: dict[str, ctypes.CDLL] = {}
@@ -57,6 +61,8 @@ def _sources(name: str) -> tuple:
     """The file that is compiled first, then what it includes (all of it goes into the hash)."""
     if name in HOST_LIBRARIES:
         return (name + ".cpp",)
+    if name in MEASUREMENT_LIBRARIES:
+        return (os.path.join("measure", name + ".hip"),) + HEADERS
     own = (name + ".h",) if os.path.isfile(os.path.join(HERE, name + ".h")) else ()
     return (name + ".hip",) + HEADERS + own
 
@@ -116,7 +122,7 @@ def compile_library(name: str, verbose: bool = True) -> str:
     out_dir = _writable_dir()
     so = os.path.join(out_dir, name + ".so")
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [compiler] + (HOST_FLAGS if host else FLAGS) + [os.path.join(HERE, _sources(name)[0]), "-o", tmp]
+    cmd = [compiler] + (HOST_FLAGS if host else FLAGS + ["-I", HERE]) + [os.path.join(HERE, _sources(name)[0]), "-o", tmp]
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)   # hipcc wants a home for its temporary files
     t0 = time.time()
@@ -155,7 +161,12 @@ def compile_all(verbose: bool = True) -> None:
 
 
 def ensure_built(names, verbose: bool = True) -> None:
-    """Compile those of `names` that have no current object, several at a time."""
+    """Compile those of `names` (libraries that a model's parts name, and the host runtime) that have no current
+    object, several at a time."""
+    for n in names:
+        if n not in KERNEL_LIBRARIES + HOST_LIBRARIES:
+            raise KernelBuildError(f"'{n}' is not a kernel library that a part may name (those are: "
+                                   f"{', '.join(KERNEL_LIBRARIES)})")
     todo = [n for n in names if _find_built(n, _source_hash(n)) is None]
     if not todo:
         return

@@ -194,3 +194,18 @@ __device__ __forceinline__ bool last_block_arrives(unsigned* counter, unsigned t
 }
 
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
+
+// Compute units of the current device, asked for once per device.  Dispatch decisions that weigh a launch's
+// blocks against the CUs (tile shapes, one or two groups of waves) take the number from here; the measurements
+// behind their ratios were made on 256.
+static inline int fx_compute_units() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return n;
+}

@@ -1377,12 +1377,12 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         if (spread_rows) nw = 2;
         if ((g_skinny_nw == 1 && !dual) || (g_skinny_nw == 2 && !norm_w)) nw = g_skinny_nw;
         // Waves per block: four, a part of K each.  Unsorted pairs: one wave that runs through all four parts when
-        // the blocks number no more than the 3,072 waves that the GPU holds at a time, else two (a wave then spends
+        // the blocks number no more than the waves that the GPU holds at a time (twelve a CU: 3,072), else two (a wave then spends
         // less of its time finding its rows and more of it streaming; measured at the sizes of the engine, one
         // token's gate/up product 20.5 against 23.3 us, its down product 11.2 against 12.0, sixteen tokens' 96 and
         // 53 against 104 and 62 us, eight tokens' within 3 %).  The sums are the same bits either way.
         int waves = 4;
-        if (pair_ids) waves = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles <= 3072 ? 1 : 2;
+        if (pair_ids) waves = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles <= 12L * fx_compute_units() ? 1 : 2;
         else if (expert_offsets && mt == 1) waves = 2;      // sorted, up to 16 rows per expert: 152 against 159 us at 64 tokens
         if (g_skinny_waves == 8 || g_skinny_waves == 4 || g_skinny_waves == 2 || g_skinny_waves == 1) waves = g_skinny_waves;
         launch_skinny(g, epi, mt, nw, waves, m_tiles, s);
@@ -1394,8 +1394,9 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         const int m_tiles = M / 64 + (expert_offsets ? nonempty : (M % 64 != 0));
         launch_bf16<64, 64, 32, 32>(g, epi, m_tiles, s);
     } else if (g.vec_ok && K % 64 == 0 && !g_no_wide) {
-        // the widest tile that still gives the 256 CUs (one block each) an even share of the work
+        // the widest tile that still gives the CUs (one block each) an even share of the work
         const bool dual = epi == EPI_GATED;
+        const long cus = fx_compute_units();
         auto tiles = [&](int tm, int tn) {
             return (long)ceil_div(N, dual ? tn / 2 : tn) * (M / tm + (expert_offsets ? nonempty : (M % tm != 0)));
         };
@@ -1403,7 +1404,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
             const long t = tiles(tm, tn);
             // plain rows: the share of a tile's rows that exist (an expert's missing row blocks are skipped)
             const double rows = expert_offsets ? 1.0 : (double)M / (double)((long)ceil_div(M, tm) * tm);
-            return quality * rows * (double)t / (double)(ceil_div(t, 256) * 256L);
+            return quality * rows * (double)t / (double)(ceil_div(t, cus) * cus);
         };
         double s256 = score(256, 256, 1.0), s192 = dual || expert_offsets ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
                s64 = score(128, 128, 0.7);
@@ -1441,8 +1442,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     } else {
         const int m_tiles = M / 128 + (expert_offsets ? nonempty : (M % 128 != 0));
         const bool dual = epi == EPI_GATED;
-        // narrow outputs: tiles of 64 columns give the 256 CUs at least two blocks each
-        if (!dual && (long)ceil_div(N, 128) * m_tiles < 512)
+        // narrow outputs: tiles of 64 columns give the CUs at least two blocks each
+        if (!dual && (long)ceil_div(N, 128) * m_tiles < 2L * fx_compute_units())
             launch_bf16<128, 64, 64, 32>(g, epi, m_tiles, s);
         else
             launch_bf16<128, 128, 64, 64>(g, epi, m_tiles, s);

@@ -422,6 +422,17 @@ def can_fuse_norm(h: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:
             and h.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+_compute_units: dict = {}
+
+
+def compute_units(device) -> int:
+    """CUs of the device (asked for once)."""
+    key = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+    if key not in _compute_units:
+        _compute_units[key] = int(torch.cuda.get_device_properties(key).multi_processor_count)
+    return _compute_units[key]
+
+
 def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
     """The most consecutive queries of a sequence that one item of attention_tiles may cover at these sizes: 64,
     or 128 where the kernel has a block of eight waves for them."""

@@ -17,6 +17,7 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec, Rotary
 from .linear import Linear, same_dtype
 
 NO_ROTATION = Rotary(0, 1.0)
+EVEN_BLOCKS_PER_CU = 250 / 256     # items of 128 queries pay from about one evenly loaded block per CU on (measured on 256 CUs)
 
 
 def attention_items(ctx, tile_q: int = 64):
@@ -68,6 +69,8 @@ class PagedAttention(Mixer):
         self.bias = bool(bias)
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # attention.rs:433
+        if not 0.0 < self.scale < math.inf:
+            raise ValueError(f"the scale of the attention scores must be positive and finite, got {self.scale}")
         self.position = POSITION_ENCODINGS.build(position)
         self._position_prefix = position.prefix or ""       # where the encoding's own tensors (if any) are named
         self.qw, self.kvw = n_heads * head_dim, n_kv_heads * head_dim
@@ -117,7 +120,7 @@ class PagedAttention(Mixer):
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
         """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many (a block
         of eight waves then shares every tile of keys it brings in between twice as many queries).  The kernel gives
-        a launch of no more blocks than the 256 CUs two groups of waves per block, which halves a block's chain of
+        a launch of no more blocks than the GPU has CUs (256) two groups of waves per block, which halves a block's chain of
         tiles; so: items of 64 while they number no more than the CUs; else items of 128 if those do (a 2,048-token
         portion deep in a prompt: 603 against 784 us at 16 heads); else items of 128 if they still number about
         one evenly loaded block per CU (blocks of a portion that starts a prompt differ in work up to the portion's
@@ -127,6 +130,7 @@ class PagedAttention(Mixer):
         widest = ops.attention_tile_queries(dtype, self.head_dim, block_size)
         if widest == 64:
             return 64
+        cus = ops.compute_units(ctx.device)
         small = large = 0
         even_blocks = 0.0
         for s in range(ctx.n_seqs):
@@ -136,9 +140,9 @@ class PagedAttention(Mixer):
                 small += -(-n // 64) * self.n_heads
                 large += -(-n // widest) * self.n_heads
                 even_blocks += -(-n // widest) * self.n_heads * (before + n / 2) / (before + n)
-        if small <= 256:
+        if small <= cus:
             return 64
-        return widest if large <= 256 or even_blocks >= 250 else 64
+        return widest if large <= cus or even_blocks >= EVEN_BLOCKS_PER_CU * cus else 64
 
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         table = ctx.block_tables[cache.group]

@@ -584,7 +584,9 @@ def test_how_many_queries_an_item_of_a_prompt_portion_takes(model_folders):
     att = runner.model.blocks[0].mixer                       # 16 heads of 128
     ask = lambda portions, recorded=False, dtype=torch.bfloat16, bs=64: att.tile_queries(
         NS(recorded=recorded, n_seqs=len(portions), q_starts=[sum(n for n, _ in portions[:i]) for i in range(len(portions) + 1)],
-           kv_lens=[before + n for n, before in portions]), dtype, bs)
+           kv_lens=[before + n for n, before in portions], device=torch.device("cuda:0")), dtype, bs)
+    from ferrox_amd import ops
+    assert ops.compute_units("cuda:0") == 256                # the counts below are for this GPU's 256 CUs
     assert ask([(1024, 0)]) == 64                            # 256 items of 64: two groups of waves each
     assert ask([(2048, 0)]) == 128                           # 512 items of 64, 256 of 128: those get the two groups
     assert ask([(2048, 22528)]) == 128

@@ -666,6 +666,34 @@ def test_attention_over_more_pages_than_a_block_copies(hd, bs, window):
         close(out2[L - 1], ref[63], dtype, f"decode attention chunk {chunk}")
 
 
+def test_decode_attention_of_a_short_sequence_beside_a_very_long_one():
+    """One launch, no window, two chunks: a sequence of 2,500 pages, whose chunks span more pages than a block
+    copies into LDS (1024), beside one of 300 keys.  The short sequence's chunks lie far below the range of page
+    ids that its blocks copy (the range is laid out for the launch's longest chunk before the position is known),
+    so every one of its lookups goes to the table in memory; both against the plain attention."""
+    from ferrox_amd import ops
+    nh, nkv, hd, bs, dtype = 4, 2, 64, 16, torch.bfloat16
+    lens = [40005, 300]
+    n_pages = sum(-(-L // bs) for L in lens) + 3
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, lens, 1e6, hd, n_pages)
+    scale = 1.0 / math.sqrt(hd)
+    kp, vp = k_pages.double().cpu(), v_pages.double().cpu()
+    last = [lens[0] - 1, lens[0] + lens[1] - 1]                               # token numbers of the two last positions
+    out = torch.zeros(len(toks), nh * hd, dtype=dtype, device=DEV)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    chunk = 20032                                                             # 1,252 pages a chunk
+    assert chunk // bs > 1024
+    ops.attention_decode(q_rot, out, k_pages, v_pages, table, pos, i32([0, 1]), i32(last), nh, nkv, hd, bs, 0, scale,
+                         max_kv_len=lens[0], chunk=chunk)
+    for s_, L in enumerate(lens):
+        tab = table.cpu()[s_].long()[: -(-L // bs)]
+        ks = kp[tab].permute(0, 2, 1, 3).reshape(-1, nkv, hd)[:L]
+        vs = vp[tab].permute(0, 3, 1, 2).reshape(-1, nkv, hd)[:L]
+        qs = q_rot[last[s_]].double().cpu().reshape(nh, hd)
+        ref = torch.stack([torch.softmax((ks[:, h // (nh // nkv)] @ qs[h]) * scale, 0) @ vs[:, h // (nh // nkv)] for h in range(nh)])
+        close(out[last[s_]].reshape(nh, hd), ref, dtype, f"sequence of {L} keys")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,H,E,k,renorm", [(1, 64, 8, 2, False), (7, 96, 6, 3, True), (33, 200, 60, 4, False),
                                              (5, 128, 130, 8, True), (4, 72, 5, 5, False)])
