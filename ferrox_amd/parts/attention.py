@@ -4,7 +4,10 @@ Per token (ferrox-models/src/decoder.rs:3224-3560): q, k, v = W x + b, the bias
 added before the rotation; q and k rotated by the position encoding; k and v
 written into the pages; the query attends to its sequence's pages (its own
 position included, through the cache just written); the heads' outputs go
-through o_proj (no bias) into the residual stream.
+through o_proj (no bias) into the residual stream.  Optionally every head of q
+and of k goes through a norm of its own between the bias and the rotation
+(`qk_norm`; the reference applies such norms where a model's tensors exist,
+decoder.rs:2099-2104, 3256-3267; this architecture has none).
 """
 from __future__ import annotations
 
@@ -13,8 +16,8 @@ import math
 import torch
 
 from .. import debug, limits, ops
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec, Rotary
-from .linear import Linear, same_dtype
+from .base import MIXERS, NORMS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec, Rotary
+from .linear import Linear, matmul, same_dtype
 
 NO_ROTATION = Rotary(0, 1.0)
 EVEN_BLOCKS_PER_CU = 250 / 256     # items of 128 queries pay from about one evenly loaded block per CU on (measured on 256 CUs)
@@ -59,7 +62,10 @@ class PagedAttention(Mixer):
     graph_safe = True      # its launches depend on device data and on sizes that are fixed per graph
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, bias: bool,
-                 position: PartSpec, window: int | None = None, scale: float | None = None):
+                 position: PartSpec, window: int | None = None, scale: float | None = None,
+                 qk_norm: PartSpec | None = None):
+        """`qk_norm`: kind and arguments of a norm over head_dim; two of them are built, with tensors under
+        `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation."""
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
         if head_dim % limits.HEAD_DIM_STEP or not limits.HEAD_DIM_STEP <= head_dim <= limits.HEAD_DIM_MAX:
@@ -75,9 +81,13 @@ class PagedAttention(Mixer):
         self._position_prefix = position.prefix or ""       # where the encoding's own tensors (if any) are named
         self.qw, self.kvw = n_heads * head_dim, n_kv_heads * head_dim
         self.qkv = self.o_proj = None
+        self.q_norm = self.k_norm = None
+        if qk_norm is not None:
+            self.q_norm, self.k_norm = (NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args))) for _ in range(2))
 
     def children(self):
-        return [(self._position_prefix, self.position)]
+        norms = [("q_norm.", self.q_norm), ("k_norm.", self.k_norm)] if self.q_norm is not None else []
+        return [(self._position_prefix, self.position)] + norms
 
     def param_specs(self):
         H = self.hidden_size
@@ -104,7 +114,7 @@ class PagedAttention(Mixer):
         """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
         more, every block's reading and norming of all rows costs more than the norm kernel)."""
         rms = norm.rms_params()
-        if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16
+        if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16 or self.q_norm is not None
                 or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
         debug.region("qkv")
@@ -115,7 +125,8 @@ class PagedAttention(Mixer):
     def takes_scale_later(self, act_dtype) -> bool:
         """Whether forward takes an ops.ScaleLater as x (the block before then leaves its rows that way)."""
         w = self.qkv.weight
-        return act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0
+        return (self.q_norm is None and act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0
+                and w.data_ptr() % 16 == 0)
 
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
         """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many (a block
@@ -144,13 +155,36 @@ class PagedAttention(Mixer):
             return 64
         return widest if large <= cus or even_blocks >= EVEN_BLOCKS_PER_CU * cus else 64
 
+    def normed_heads(self, x, ctx):
+        """q [T, qw], k [T, kvw] with every head normed, and v [T, kvw]: the q and k products in float32 (the
+        norms read float32 rows), each head a row of a [T * (nh + nkv), head_dim] matrix that the norm kernels
+        gather their rows from."""
+        T, nh, nkv, hd = ctx.n_tokens, self.n_heads, self.n_kv_heads, self.head_dim
+        w, b = self.qkv.weight, self.qkv.bias
+        cut = self.qw + self.kvw
+        qk = matmul(x, w[:cut], bias=None if b is None else b[:cut], epilogue=ops.EPI_STORE_F32)
+        v = matmul(x, w[cut:], bias=None if b is None else b[cut:])
+
+        def head_rows():
+            first = torch.arange(T, dtype=torch.int32, device=qk.device)[:, None] * (nh + nkv)
+            heads = torch.arange(nh + nkv, dtype=torch.int32, device=qk.device)[None, :]
+            rows = first + heads
+            return rows[:, :nh].reshape(-1).contiguous(), rows[:, nh:].reshape(-1).contiguous()
+
+        q_rows, k_rows = ctx.memo(f"head rows {nh} {nkv}", head_rows)
+        heads = qk.view(T * (nh + nkv), hd)
+        q = self.q_norm.forward(heads, ctx, rows=q_rows).view(T, self.qw)
+        k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw)
+        return q, k, v
+
     def forward(self, x, ctx, cache, residual, qkv=None) -> None:
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
         debug.region("qkv")
-        if (qkv is None and rot is not None
-                and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved)):
+        fused = (qkv is None and self.q_norm is None and rot is not None
+                 and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved))
+        if fused:
             # few tokens: rotation and cache write happen in the product's epilogue
             qkv = ops.qkv_rope(x, self.qkv.weight, self.qkv.bias, ctx.positions, ctx.token_seq, table,
                                k_pages if cache.writes else None, v_pages if cache.writes else None,
@@ -158,12 +192,16 @@ class PagedAttention(Mixer):
                                rot.freq_factors)
             q = qkv[:, :self.qw]
         else:
-            if qkv is None:
-                if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
-                    qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
-                else:
-                    qkv = self.qkv(x)
-            q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
+            if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
+                q, k, v = self.normed_heads(x, ctx)
+                qkv = q
+            else:
+                if qkv is None:
+                    if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
+                        qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
+                    else:
+                        qkv = self.qkv(x)
+                q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
             debug.region("rope + cache write")
             if rot is None:
                 self.position.apply(q, k, ctx)

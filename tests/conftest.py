@@ -73,6 +73,9 @@ ODD_F = {
     "rms_norm_eps": 1e-5, "max_position_embeddings": 512, "use_sliding_window": False, "sliding_window": 64,
     "max_window_layers": 2, "tie_word_embeddings": False,
 }
+# every width odd (no vector load or store is aligned), one sparse and one dense layer
+ODD_H = dict(ODD_F, hidden_size=71, moe_intermediate_size=21, shared_expert_intermediate_size=37, intermediate_size=51,
+             vocab_size=97, mlp_only_layers=[1])
 # the larger model's layer sizes with few experts: 7 query heads per kv head, eight experts per token, a shared
 # expert eight times as wide as an expert
 WIDE_G = {
@@ -87,7 +90,7 @@ WIDE_G = {
 # one layer of the smaller model's sizes under its real vocabulary: the head and the sampling at 151,936 columns
 WIDE_DV = dict(WIDE_D, vocab_size=151936)
 TINY = {"DV": (WIDE_DV, 7), "A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5),
-        "G": (WIDE_G, 6)}
+        "G": (WIDE_G, 6), "H": (ODD_H, 8)}
 
 
 @pytest.fixture(scope="session")

@@ -15,7 +15,7 @@ from conftest import ROOT, TINY
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [1, 7, 16, 33, 70, 45], "B": [3, 17, 40, 64, 90, 120], "C": [2, 35, 66, 130, 51],
-           "D": [40, 75], "E": [150, 260], "F": [5, 70, 33, 150], "G": [30, 70]}
+           "D": [40, 75], "E": [150, 260], "F": [5, 70, 33, 150], "G": [30, 70], "H": [5, 70, 33, 150]}
 # float32: |engine - plain| <= absolute + relative * |plain| per logit; the engine differs from a float64
 # computation by float32 rounding only.  bfloat16: weights are the same bfloat16 values on both sides, and the
 # engine's deviation is held to what rounding at the tensors it stores predicts for the model and the tokens at
@@ -504,10 +504,10 @@ def test_preemption_and_seeded_sampling_through_the_entry_point(model_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["D", "E", "F", "G"])
+@pytest.mark.parametrize("name", ["D", "E", "F", "G", "H"])
 def test_production_layer_sizes(model_folders, name, dtype):
-    """one or two layers of the sizes the engine is built for (D, E, G) and of widths that allow no
-    16-byte loads (F), pages of 64: whole prompts (tiled matrix kernels, MFMA prefill attention),
+    """one or two layers of the sizes the engine is built for (D, E, G), of widths that allow no
+    16-byte loads (F) and of odd widths (H: 71, 21, 37, 51, vocabulary 97), pages of 64: whole prompts (tiled matrix kernels, MFMA prefill attention),
     then mixed portions and single tokens (streaming kernels, split decode attention, recorded
     decode steps)"""
     reqs = requests_for(name)

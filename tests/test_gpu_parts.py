@@ -485,3 +485,119 @@ def test_a_rotary_with_a_table_of_frequency_factors(dtype, tol):
     scale = float(want.abs().max())
     assert float((unbanded - want).abs().max()) > 10 * tol * scale, "the factors make no difference in this test"
     assert float((whole - want).abs().max()) < tol * scale and float((cut - want).abs().max()) < tol * scale
+
+
+# ---- blocks from outside the package that hand normed rows on to each other ------------------------------
+from ferrox_amd.parts import BLOCKS, NORMS, Block  # noqa: E402
+
+
+@BLOCKS.register("test_mixer_only")
+class MixerOnly(Block):
+    """h += mixer(norm1(h)), and nothing else.  It chains: it takes norm1(h) from the block before where that block
+    has made it, and says what kind of rows its mixer accepts."""
+    slots = {"norm1": NORMS, "mixer": MIXERS}
+    chains_norms = True
+
+    def __init__(self, parts, prefixes):
+        self.norm1, self.mixer, self._prefixes = parts["norm1"], parts["mixer"], prefixes
+
+    def children(self):
+        return [(self._prefixes["norm1"], self.norm1), (self._prefixes["mixer"], self.mixer)]
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def takes_scale_later(self, act_dtype):
+        return bool(self.mixer.takes_scale_later(act_dtype))
+
+    def forward(self, h, ctx, cache, normed=None, then=None):
+        if normed is not None:
+            self.mixer.forward(normed, ctx, cache, h)
+        elif not self.mixer.forward_from_residual(self.norm1, ctx, cache, h):
+            self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
+        return None
+
+
+@BLOCKS.register("test_ffn_only")
+class FfnOnly(Block):
+    """h += ffn(norm2(h)) around a mixer that does nothing.  It chains: a feed-forward that can norm the rows it
+    has finished for the block that follows is told which norm that is, and what it leaves is handed on."""
+    slots = {"mixer": MIXERS, "norm2": NORMS, "ffn": FEED_FORWARDS}
+    chains_norms = True
+
+    def __init__(self, parts, prefixes):
+        self.mixer, self.norm2, self.ffn, self._prefixes = parts["mixer"], parts["norm2"], parts["ffn"], prefixes
+
+    def children(self):
+        return [(self._prefixes["norm2"], self.norm2), (self._prefixes["ffn"], self.ffn)]
+
+    @property
+    def first_norm(self):
+        return self.norm2
+
+    def forward(self, h, ctx, cache, normed=None, then=None):
+        assert normed is None                       # (takes_scale_later is False and no block before it norms for it)
+        ctx.carry = None
+        more = {"then_norm": then} if then is not None and self.ffn.norms_after else {}
+        if not self.ffn.forward_from_residual(self.norm2, ctx, h, **more):
+            self.ffn.forward(self.norm2.forward(h, ctx), ctx, h, **more)
+        out, ctx.carry = ctx.carry, None
+        return out
+
+
+@MIXERS.register("test_no_mixer_recordable")
+class NoMixerRecordable(NoMixer):
+    graph_safe = True
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "E"])
+def test_two_chaining_blocks_from_outside_equal_the_built_in_block(model_folders, name, dtype):
+    """Every layer of a model cut into two blocks defined here, one with the mixer and one with the feed-forward,
+    which hand normed rows on through the blocks' optional protocol (`chains_norms`, `first_norm`,
+    `takes_scale_later`, `forward(..., normed=, then=)`): the same kernels run in the same order as with the
+    built-in pre-norm block, so the logits are the same bits, for whole prompts and for few tokens from recorded
+    steps, where the feed-forward's last kernel norms for the next layer's mixer."""
+    from conftest import TINY
+    from ferrox_amd.config import Qwen2MoeConfig
+    from ferrox_amd.engine.loading import load_model
+    from ferrox_amd.models.qwen2_moe import build_spec
+    from ferrox_amd.weights import Checkpoint
+    folder = model_folders(name, "bfloat16" if name == "E" else dtype)
+    built_in = load_model(folder, dtype, DEV)
+    spec = build_spec(Qwen2MoeConfig.from_dict(TINY[name][0]), Checkpoint(folder).names())
+    layers = []
+    for ls in spec.layers:
+        layers.append(LayerSpec("test_mixer_only", ls.prefix, {"norm1": ls.parts["norm1"], "mixer": ls.parts["mixer"]}))
+        layers.append(LayerSpec("test_ffn_only", ls.prefix, {"mixer": PartSpec("test_no_mixer_recordable"),
+                                                             "norm2": ls.parts["norm2"], "ffn": ls.parts["ffn"]}))
+    spec.layers, spec.schedule = layers, [ScheduleEntry(i) for i in range(len(layers))]
+    cut = Model(spec)
+    cut.load(Checkpoint(folder), built_in.act_dtype, DEV)
+    reqs = ru.make_requests(TINY[name][0]["vocab_size"], [40, 9, 70], 21)
+    seen = []
+    probe = ops.moe_combine
+
+    def watching(*a, **kw):
+        out = probe(*a, **kw)
+        seen.append(out is not None)
+        return out
+
+    outs = []
+    for model in (built_in, cut):
+        runner = ModelRunner(model, block_size=64 if name == "E" else 16, num_pages=24, max_seqs=3)
+        assert runner.use_graphs
+        ops.moe_combine = watching
+        try:
+            outs.append((ru.run_trace(runner, ru.trace_whole(reqs)), ru.run_trace(runner, ru.trace_tail_decode(reqs, tail=6))))
+        finally:
+            ops.moe_combine = probe
+        assert runner._graphs
+        if dtype == "bfloat16":
+            assert any(seen), "no feed-forward normed its rows for the layer after it: the chain was not exercised"
+        seen.clear()
+    for a, b in zip(outs[0], outs[1]):
+        assert a.keys() == b.keys()
+        for key in a:
+            assert torch.equal(a[key], b[key]), f"{name} {dtype}: position {key} differs between the two ways of cutting a layer into blocks"

@@ -4,8 +4,8 @@ its own, `register_architecture`, then `write_random_model`, `load_model`, `Engi
 line and `trace_run`, against a plain forward pass written here.  Nothing in the package is changed for it.
 
 The stand-in is no published model: dense layers only, adjacent-pair rotation over half of every head, no
-biases, a feed-forward gated by tanh-GELU, two stop ids, and a head tied to an embedding table under another
-name.  What a configuration class must offer, and that `defaulted_keys` reaches the command line, is checked on
+biases, a norm over every head of q and of k before the rotation, a feed-forward gated by tanh-GELU, two stop
+ids, and a head tied to an embedding table under another name.  What a configuration class must offer, and that `defaulted_keys` reaches the command line, is checked on
 the way."""
 import json
 import math
@@ -71,7 +71,8 @@ def build_stand_in(cfg: StandInConfig, tensor_names=None) -> ModelSpec:
             "norm1": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, prefix="ln_a."),
             "mixer": PartSpec("paged_attention", {
                 "hidden_size": cfg.width, "n_heads": cfg.heads, "n_kv_heads": cfg.kv_heads, "head_dim": hd, "bias": False,
-                "position": PartSpec("rope_interleaved", {"head_dim": hd, "theta": cfg.rope_base, "rotary_dim": rot})},
+                "position": PartSpec("rope_interleaved", {"head_dim": hd, "theta": cfg.rope_base, "rotary_dim": rot}),
+                "qk_norm": PartSpec("rmsnorm", {"size": hd, "eps": cfg.eps})},
                 prefix="attn."),
             "norm2": PartSpec("rmsnorm", {"size": cfg.width, "eps": cfg.eps}, prefix="ln_f."),
             "ffn": PartSpec("gated_mlp", {"hidden_size": cfg.width, "intermediate_size": cfg.ff_width,
@@ -114,8 +115,8 @@ def stand_in_forward(cfg: dict, w: dict, tokens) -> torch.Tensor:
     for l in range(cfg["depth"]):
         p = f"blocks.{l}."
         x = plain.rms_norm(h, w[p + "ln_a.weight"], eps)
-        q = rotate((x @ w[p + "attn.q_proj.weight"].T).reshape(T, nh, hd))
-        k = rotate((x @ w[p + "attn.k_proj.weight"].T).reshape(T, nkv, hd))
+        q = rotate(plain.rms_norm((x @ w[p + "attn.q_proj.weight"].T).reshape(T, nh, hd), w[p + "attn.q_norm.weight"], eps))
+        k = rotate(plain.rms_norm((x @ w[p + "attn.k_proj.weight"].T).reshape(T, nkv, hd), w[p + "attn.k_norm.weight"], eps))
         v = (x @ w[p + "attn.v_proj.weight"].T).reshape(T, nkv, hd)
         h = h + plain.causal_attention(q, k, v, nh, nkv, None).reshape(T, nh * hd) @ w[p + "attn.o_proj.weight"].T
         x = plain.rms_norm(h, w[p + "ln_f.weight"], eps)
@@ -172,6 +173,15 @@ def test_an_outside_architecture_through_the_front_door(stand_in, tmp_path, dtyp
     # continuation depends on the whole model (under a tied head and small weights it repeats the last token)
     folder = str(tmp_path / "stand_in")
     write_random_model(dict(RAW), folder, seed=11, dtype=dtype, std=0.05 if dtype == "bfloat16" else 0.2, device="cuda:0")
+    # norm weights are written as ones; give every norm weights of its own, so that a mix-up between them shows
+    from safetensors.torch import load_file, save_file
+    tensors = load_file(os.path.join(folder, "model.safetensors"))
+    g = torch.Generator().manual_seed(3)
+    for name in sorted(tensors):
+        if tensors[name].dim() == 1:
+            tensors[name] = (1.0 + 0.3 * torch.randn(tensors[name].shape, generator=g)).to(tensors[name].dtype)
+    assert sum(".q_norm." in n or ".k_norm." in n for n in tensors) == 2 * RAW["depth"]
+    save_file(tensors, os.path.join(folder, "model.safetensors"))
     written = json.load(open(os.path.join(folder, "config.json")))
     assert written.pop("rope_base") == 10000.0              # (written in full; taken out again, so that reading defaults it)
     json.dump(written, open(os.path.join(folder, "config.json"), "w"))
