@@ -22,7 +22,8 @@ requests) / time, against the published 8 TB/s; the ceilings measured on this
 GPU by the simplest kernels (a streaming read, a copy, a loop of MFMA
 products); and the same batch served through `Engine.generate` (scheduler,
 sampling, ids read back), with the share of the time that the GPU waited for
-the host.
+the host; and 16 such prompts served in steps of at most 512 tokens, prompt
+portions beside decoded tokens, launched kernel by kernel (`served_mixed`).
 (The reference measures pp<N> / tg<N> the same way on synthetic ids with one
 discarded warm-up and the median of three runs, ferrox-cli/src/bench_model.rs:35-60, 239-302.)
 """
@@ -212,6 +213,35 @@ class Bench:
             self.runner.release(rid)
         return dt, distinct, per_part
 
+    def served_mixed(self, batch: int, ctx: int, new_tokens: int, portion: int = 512) -> dict:
+        """`batch` prompts of `ctx` tokens behind `Engine.generate` with steps of at most `portion` tokens: every step
+        but the last few carries the decoded tokens of the requests that are through their prompts beside a
+        prompt portion of the next one, launched kernel by kernel (no step of this kind is recorded).  Beside the
+        rate: the share of the time in which the GPU waited for the host between steps, and what the host spent
+        launching against what the GPU spent running."""
+        from ferrox_amd.engine.api import Engine
+        per_seq = -(-(ctx + new_tokens + 1) // self.block_size)
+        eng = Engine(model=self.model, block_size=self.block_size, num_pages=per_seq * batch + 8, max_seqs=batch,
+                     max_tokens_per_step=portion, prefill_chunk=portion, ctx_size=ctx + new_tokens + 8)
+        eng.time_steps = True
+        prompts = self.prompts(batch, ctx)
+        eng.generate(prompts[:2], max_new_tokens=4, ignore_eos=True)           # (kernels loaded, buffers there)
+        self.torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = eng.generate(prompts, max_new_tokens=new_tokens, ignore_eos=True)
+        wall = time.perf_counter() - t0
+        st = eng.last_stats
+        assert all(len(o) == new_tokens for o in out)
+        mixed = st["steps"] - st["decode_steps"]
+        res = {"value": round(batch * (ctx + new_tokens) / wall, 1), "unit": "tokens/s, prompts and generation",
+               "batch": batch, "prompt_tokens": ctx, "new_tokens": new_tokens, "portion": portion,
+               "seconds": round(wall, 3), "steps": st["steps"], "steps_with_portions": mixed,
+               "ms_per_step": round(1e3 * wall / st["steps"], 3),
+               "host_share": round(1.0 - st["gpu_seconds"] / wall, 4),
+               "host_launch_over_gpu": round(st["launch_seconds"] / st["gpu_seconds"], 3)}
+        del eng
+        return res
+
     def roofline(self, batch: int, kv_len: int, distinct: float, dt: float, ceilings: dict | None = None) -> dict:
         achieved = self.decode_bytes(batch, kv_len, distinct) / dt
         out = {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
@@ -373,7 +403,8 @@ def run_workload(name: str, args) -> int:
 
 # ---- per-kernel table (rocprofv3 around a child process) ----------------------------------------------------------
 KERNEL_TABLES = {"decode_b1": ("decode", 1), "decode_b8": ("decode", 8), "decode_b64": ("decode", 64),
-                 "prefill_2048": ("prefill", 2048), "prefill_512": ("prefill", 512)}
+                 "prefill_2048": ("prefill", 2048), "prefill_512": ("prefill", 512), "prefill_128": ("prefill", 128),
+                 "prefill_4096": ("prefill", 4096)}
 
 
 def profile_run(what: str, args) -> int:
@@ -424,20 +455,31 @@ def profile_run(what: str, args) -> int:
         sink("end")
         debug.region_sink = None
     else:
+        used = []
         for i in range(steps + 1):
             toks = b.prompts(1, n)[0]
             assert b.runner.admit("p") and b.runner.reserve("p", n)
             if i == 1:
                 torch.cuda.synchronize()
                 debug.region_sink = sink
-            b.runner.step([StepEntry("p", toks, [n - 1])])
+            if i == 0:
+                # the untimed run also counts the experts that the prompt's tokens choose: with random weights the
+                # tokens of one sequence look alike to the routers of the later layers, and far fewer experts than
+                # the model has are in use (about 30 of 60 a layer for 2,048 tokens)
+                with debug.trace_routing() as trace:
+                    b.runner.step([StepEntry("p", toks, [n - 1])])
+                    used = [len({e for tok in layer for e in tok}) for layer in trace.read()]
+            else:
+                b.runner.step([StepEntry("p", toks, [n - 1])])
             b.runner.release("p")
+        distinct = sum(used) / max(1, len(used))
         sink("end")
         debug.region_sink = None
     torch.cuda.synchronize()
     ffn = next((blk.ffn for blk in b.model.blocks if hasattr(blk.ffn, "shared_pieces")), None)
     print("PROFILE_RUN " + json.dumps({"labels": labels, "steps": steps, "distinct_experts": distinct,
-                                       "shared_as_pieces": bool(ffn is not None and ffn.shared_pieces and kind == "decode" and n <= 16)}),
+                                       "shared_as_pieces": bool(ffn is not None and ffn.shared_pieces and
+                                                                (n <= 16 if kind == "decode" else n * shape["num_experts_per_tok"] <= 1024))}),
           flush=True)
     return 0
 
@@ -449,7 +491,7 @@ def stage_costs(c, kind: str, n: int, ctx: int, distinct: float, pieces: bool, e
     qw, kvw = c.num_attention_heads * hd, c.num_key_value_heads * hd
     E, k, Im, Is, V = c.num_experts, c.num_experts_per_tok, c.moe_intermediate_size, c.shared_expert_intermediate_size, c.vocab_size
     T = n                                               # tokens in the step
-    used = distinct if kind == "decode" else min(E, E)  # a prompt uses every expert
+    used = distinct if distinct > 0 else E               # experts whose weights the step reads (counted from the routers' choices)
     rows = 1 if kind == "prefill" else n                # rows that go through the head
     act = lambda cols: T * cols * es                    # one activation matrix
     w = lambda elems: elems * es
@@ -539,7 +581,8 @@ def kernel_table(what: str, args) -> int:
              f"  python3 bench.py --kernel-table {what}" + (f" --shape {args.shape}" if args.shape != "a2.7b" else "")
              + (f" --layers {args.layers}" if args.layers else "") + (f" --ctx {args.ctx}" if args.ctx != 2048 else ""),
              "  (it runs itself under `rocprofv3 --kernel-trace`; an empty marker kernel before every stage tells the stages apart;",
-             "   bytes = weights the stage uses once + cache + activations, flops from the sizes; peaks 8 TB/s and 2.5 PFLOP/s)",
+             "   bytes = weights the stage uses once + cache + activations, flops from the sizes; peaks 8 TB/s and 2.5 PFLOP/s;",
+             f"   experts whose weights a step reads: {info['distinct_experts']:.1f} of {c.num_experts} a layer, counted from the routers' choices)",
              f"sum of kernel times {total_ns / info['steps'] / 1e3:.1f} us per step; from the first kernel to the last "
              f"{span_ns / info['steps'] / 1e3:.1f} us per step (the host launches one by one here)",
              "",
@@ -663,6 +706,8 @@ def main() -> int:
     if not args.no_served:
         out["served"] = b.served(args.batch, args.ctx, 64)
         log(f"served through Engine.generate: {out['served']}")
+        out["served_mixed"] = b.served_mixed(16, args.ctx, 32)
+        log(f"served in steps of 512 tokens, prompt portions beside decoded tokens: {out['served_mixed']}")
     print(json.dumps(out), flush=True)
     return 0
 

@@ -1155,6 +1155,7 @@ static int g_few_rows = 3;     // "few_rows": sorted by expert, up to this many 
 static int g_head_rows = 8;    // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
 static int g_tile64_rows = 20; // "tile64_rows": experts with up to this many rows on average take tiles of 64 rows
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
+static int g_wide_grouped = 0; // "wide_grouped": as "wide", for products whose rows are sorted by expert only
 static int g_wide_force = 0;   //         256, 192, 128, 64, 12 or 4 (tiles of 64 rows) picks that tile of the LDS-tiled kernel
 FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "skinny_sets")) { g_skinny_nw = value; return 0; }
@@ -1164,6 +1165,7 @@ FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "tile64_rows")) { g_tile64_rows = value; return 0; }
     if (!strcmp(key, "head_rows")) { g_head_rows = value; return 0; }
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
+    if (!strcmp(key, "wide_grouped")) { g_wide_grouped = value > 1 ? value : 0; return 0; }
     FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, head_rows, wide)", key);
     return 1;
 }
@@ -1397,6 +1399,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         // the widest tile that still gives the CUs (one block each) an even share of the work
         const bool dual = epi == EPI_GATED;
         const long cus = fx_compute_units();
+        const int force = expert_offsets && g_wide_grouped ? g_wide_grouped : g_wide_force;
         auto tiles = [&](int tm, int tn) {
             return (long)ceil_div(N, dual ? tn / 2 : tn) * (M / tm + (expert_offsets ? nonempty : (M % tm != 0)));
         };
@@ -1408,8 +1411,8 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         };
         double s256 = score(256, 256, 1.0), s192 = dual || expert_offsets ? 0.0 : score(256, 192, 0.92), s128 = score(256, 128, 0.85),
                s64 = score(128, 128, 0.7);
-        if (g_wide_force) {
-            s256 = g_wide_force == 256; s192 = g_wide_force == 192 && !dual; s128 = g_wide_force == 128; s64 = 0.5 * (g_wide_force == 64);
+        if (force) {
+            s256 = force == 256; s192 = force == 192 && !dual; s128 = force == 128; s64 = 0.5 * (force == 64);
         }
         // an expert's share of up to 192 rows: the product streams the weights once and multiplies little, so it
         // is bound by how many of them are on their way; a ring of three weight tiles beside two of the rows
@@ -1420,14 +1423,14 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         // 256 do, 273 rows an expert as 2 x 192 instead of 2 x 256: the down product of a 4,096-token step 173
         // against 190 us)
         const long pad192 = ceil_div(per_group, 192) * 192L, pad256 = ceil_div(per_group, 256) * 256L;
-        const bool few_rows = g_wide_force ? g_wide_force == 12
+        const bool few_rows = force ? force == 12
                                            : (expert_offsets ? (per_group <= 176 || pad192 < pad256)
                                                              : (s12 > s256 && s12 > s192 && s12 > s128 && s12 > s64));
         // an expert's share of up to 20 rows on average: a tile of 64 rows leaves LDS for a ring of four weight tiles
         // beside two of the rows (2-5 % less time than tiles of 192 rows with a ring of three, the same bits: decode
         // at 64 sequences 11.2 -> 11.0 ms, a 192-token step 6.8 -> 6.4 ms; from 25 rows on average on, steps of 384
         // tokens, more and more experts need a second tile and it falls behind)
-        if (g_wide_force == 4 || (!g_wide_force && expert_offsets && per_group <= g_tile64_rows))
+        if (force == 4 || (!force && expert_offsets && per_group <= g_tile64_rows))
             launch_wide<4, 256, 4, 2>(g, epi, M / 64 + (expert_offsets ? nonempty : (M % 64 != 0)), s);
         else if (few_rows)
             launch_wide<12, 256, 3, 2>(g, epi, M / 192 + (expert_offsets ? nonempty : (M % 192 != 0)), s);

@@ -106,6 +106,7 @@ class Engine:
         t0 = time.time()
         n_steps = n_tokens = 0
         marks = []            # per step: [event at its first device operation, event after its last launch, all decodes?]
+        launching = 0.0       # (time_steps) seconds the host spent putting steps together and launching them
         if self.time_steps:
             self.runner.before_launch = lambda: marks[-1][0].record()
         # the step whose sampled ids the host has not read yet: its batch, the requests of the rows, the ids on
@@ -150,6 +151,7 @@ class Engine:
                 if self.time_steps:
                     marks.append([torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True),
                                   all(s.n_tokens == 1 for s in batch)])
+                    t_launch = time.perf_counter()
                 logits = self.runner.step(entries, feed=(inflight[2], pairs) if pairs else None)
                 rows = [s.request for s in batch if s.samples]
                 launched = None
@@ -163,6 +165,7 @@ class Engine:
                     launched = (batch, rows, ids, host_ids, copied)
                 if self.time_steps:
                     marks[-1][1].record()
+                    launching += time.perf_counter() - t_launch
                 settle()                      # the ids of the step before this one: they come while this one runs
                 sched.commit_launched(batch)
                 inflight = launched
@@ -185,7 +188,10 @@ class Engine:
             spans = [a.elapsed_time(b) * 1e-3 for a, b, _ in marks]
             gaps = [marks[i][1].elapsed_time(marks[i + 1][0]) * 1e-3 for i in range(len(marks) - 1)]
             dec = [i for i, m in enumerate(marks) if m[2]]
+            # `launch_seconds`: what the host spent inside the steps (packing, one launch after the other, the sampling
+            # call); where it comes near `gpu_seconds` the kernels of a step wait for their launches.
             self.last_stats.update(gpu_seconds=sum(spans), host_gap_seconds=sum(gaps), decode_steps=len(dec),
+                                   launch_seconds=launching,
                                    decode_gpu_seconds=sum(spans[i] for i in dec),
                                    decode_gap_seconds=sum(gaps[i - 1] for i in dec if i > 0))
         return [Completion(r.generated, r.finish_reason or "aborted", len(r.prompt), r.n_preempted) for r in reqs]
