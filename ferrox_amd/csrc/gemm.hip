@@ -666,6 +666,32 @@ __device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
+// The few-row product's weight loads.  A 16 x 16 x 32 product wants lane (li, grp) of a wave to hold row li, k
+// 8 grp .. 8 grp + 7 of a set of 16 weight rows; loaded that way one instruction takes 64 bytes of each of 16
+// rows, half of every 128-byte line, and the other half comes with the next load.  Instead a load takes whole
+// lines of 8 rows: its lanes li < 8 take (row li, the low 32 k of 64), lanes li >= 8 (row li - 8, the high 32 k);
+// the next load takes rows 8 .. 15 the same way, and before the products the halves of each row of 16 lanes
+// change places (`swap_halves`, one DPP move a register).  Loads of whole lines can carry the non-temporal hint
+// (weights are read once a step and need no place in the caches), which memory answers about a tenth faster;
+// on half lines the hint costs time.  Measured at 8 tokens of the A2.7B sizes: the experts' gate/up product
+// 69.1 -> 64.4 us, their down product 36.6 -> 32.7 us, the head 132 -> 101 us (4.7 -> 6.2 TB/s).
+typedef unsigned int fx_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_lines16(const void* p) {
+    const fx_u32x4 v = __builtin_nontemporal_load((const fx_u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+// keep: this lane's value where its bank (four lanes) is not in BANKS, else other's value from the lane eight
+// further round its row of 16 lanes
+template <int BANKS>
+__device__ __forceinline__ uint4 swap_halves(uint4 keep, uint4 other) {
+    uint4 r;
+    r.x = __builtin_amdgcn_update_dpp(keep.x, other.x, 0x128, 0xF, BANKS, false);
+    r.y = __builtin_amdgcn_update_dpp(keep.y, other.y, 0x128, 0xF, BANKS, false);
+    r.z = __builtin_amdgcn_update_dpp(keep.z, other.z, 0x128, 0xF, BANKS, false);
+    r.w = __builtin_amdgcn_update_dpp(keep.w, other.w, 0x128, 0xF, BANKS, false);
+    return r;
+}
+
 // NW: sets of 16 weight rows per wave; in dual mode set a is the gate (a even) or up (a odd) rows of
 // column group a / 2.
 template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false, bool ROPE = false>
@@ -710,18 +736,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         rope_c0 = rope_rotated ? 16 * rope_j : (is_v ? 32 * rope_j : g.rope_rot + 32 * (rope_j - n_rot));
         rope_c1 = rope_rotated ? rope_c0 + (g.rope_rot >> 1) : rope_c0 + 16;
     }
-    const bf16* wrow[NW];
+    const bf16* wrow[NW];     // this lane's place in the set's first load, and how far behind it the second is
+    int wrow_b[NW];
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
         const int n = ROPE ? rope_head * g.rope_hd + (a ? rope_c1 : rope_c0) + li
                            : (DUAL ? n0 + (a >> 1) * 16 + li : n0 + a * 16 + li);
         const bool up = DUAL && (a & 1);
-        // rows past the end repeat the last one: their columns are never stored
-        const int nc = min(n, g.N - 1);
-        if (g.kb_stride)
-            wrow[a] = Wbase + ((size_t)nc + (up ? g.up_offset / g.K : 0)) * 64;
-        else
-            wrow[a] = Wbase + (size_t)nc * g.K + (up ? g.up_offset : 0);
+        // whole lines per load: the lanes of a set's first load take rows li % 8, those of its second rows
+        // 8 + li % 8, both k 32 (li / 8) .. of every 64; rows past the end repeat the last one, never stored
+        const int nl = n - li + (li & 7);
+        const int na = min(nl, g.N - 1), nb = min(nl + 8, g.N - 1);
+        const size_t rs = g.kb_stride ? 64 : (size_t)g.K;
+        const size_t first = g.kb_stride ? (size_t)(up ? g.up_offset / g.K : 0) * 64 : (size_t)(up ? g.up_offset : 0);
+        wrow[a] = Wbase + first + (size_t)na * rs + 32 * (li >> 3);
+        wrow_b[a] = (int)((nb - na) * rs);
     }
     const size_t slab = g.kb_stride ? (size_t)g.kb_stride : 64;     // element (row, k) is at row + (k / 64) * slab + k % 64
     const bf16* xrow[MT];       // NORM: float rows, kept under the same name
@@ -750,12 +779,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
         constexpr bool FULL = decltype(full)::value;
         const int kb = sp * 128 + grp * 8;     // load u of this lane: k = kb + 32u .. +7
 #pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int kl = kb + 64 * h;                       // this lane's k without its half: 32 (li / 8) is in wrow
+            const bool kin = FULL || kl + 32 * (li >> 3) < g.K;
+            const size_t woff = (size_t)(kl >> 6) * slab + (kl & 63);
+#pragma unroll
+            for (int a = 0; a < NW; ++a) {
+                w[a][2 * h] = kin ? load_lines16(wrow[a] + woff) : make_uint4(0, 0, 0, 0);
+                w[a][2 * h + 1] = kin ? load_lines16(wrow[a] + woff + wrow_b[a]) : make_uint4(0, 0, 0, 0);
+            }
+        }
+#pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int k = kb + 32 * u;
             const bool kin = FULL || k < g.K;
-            const size_t woff = (size_t)(k >> 6) * slab + (k & 63);
-#pragma unroll
-            for (int a = 0; a < NW; ++a) w[a][u] = kin ? *(const uint4*)(wrow[a] + woff) : make_uint4(0, 0, 0, 0);
             if constexpr (NORM) {
                 float gv[8];
                 if (g.norm_dtype == FX_F32) {
@@ -784,13 +821,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
     };
     auto multiply_into = [&](f32x4_t (&to)[MT][NW], const uint4 (&w)[NW][4], const uint4 (&x)[MT][4]) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int u = 0; u < 4; ++u)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x[mt][u]);
+            for (int a = 0; a < NW; ++a) {
+                // low k: own first load below lane 8 of a row of 16, the other half's second load above;
+                // high k: the other half's first load below, own second load above
+                const uint4 wu = (u & 1) ? swap_halves<0x3>(w[a][u], w[a][u - 1]) : swap_halves<0xC>(w[a][u], w[a][u + 1]);
 #pragma unroll
-                for (int a = 0; a < NW; ++a)
-                    to[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w[a][u]), xb, to[mt][a], 0, 0, 0);
+                for (int mt = 0; mt < MT; ++mt)
+                    to[mt][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wu), __builtin_bit_cast(bf16x8_t, x[mt][u]),
+                                                                        to[mt][a], 0, 0, 0);
             }
     };
     // piece sp belongs to part sp / per, the (sp / per - wave * VW)-th of this wave (the same for all its lanes)
@@ -1161,7 +1201,7 @@ static int g_skinny_nw = 0;    // "skinny_sets": 1 or 2 sets of weight rows per 
 static int g_skinny_mt = 0;    // "skinny_row_tiles": 1, 2 or 4 tiles of 16 rows per block of that product (0: by the sizes)
 static int g_skinny_waves = 0; // "skinny_waves": 1, 2, 4 or 8 waves that split K in a block of that product (0: by the sizes)
 static int g_few_rows = 3;     // "few_rows": sorted by expert, up to this many rows an expert go to the product for few rows (at most 64)
-static int g_head_rows = 8;    // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
+static int g_head_rows = 16;   // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
 static int g_tile64_rows = 20; // "tile64_rows": experts with up to this many rows on average take tiles of 64 rows
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
 static int g_stream_w = -1;    // "stream_w": 1 / 0 forces the non-temporal hint on the tiled kernel's weight loads on / off; -1: by the shape
@@ -1358,9 +1398,10 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     const long per_group = expert_offsets ? (M + E - 1) / E : M;
     const bool wide_ok = g.vec_ok && K % 64 == 0 && !g_no_wide;
     FX_REQUIRE(!pair_ids || g.vec_ok, "gemm: unsorted pairs need K a multiple of 8 and 16-byte aligned rows");
-    // 9..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights at the same
+    // 17..64 plain rows against very many weight rows (the head): tiles of 128 rows stream the weights at the same
     // speed whatever the rows (151,936 weight rows: 131-136 us from 1 to 33 rows), the kernel for few rows slows
-    // down with them (108 us at 1 row, 134 at 8, 150 at 16, 182 at 32)
+    // down with them (98 us at 1 row, 101 at 8; decode steps of 12 and 16 sequences are 20 us shorter with it, those
+    // of 24 and 32 the same either way)
     const bool many_columns = g.vec_ok && !expert_offsets && !pair_ids && !norm_w && !row_ss && !g.kb_stride && M > g_head_rows && K % 64 == 0 &&
                               !g_no_wide && ceil_div(N, 128) >= 512;
     // Rows sorted by expert: the product for few rows only up to three rows an expert on average.  Its waves fetch
