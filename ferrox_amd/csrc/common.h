@@ -193,6 +193,31 @@ __device__ __forceinline__ bool last_block_arrives(unsigned* counter, unsigned t
     return fx_last_flag != 0;
 }
 
+// Streams that are read once (weights, the keys and values of a decode step) in whole 128-byte lines.  An MFMA
+// operand wants lane (li, g) of a wave to hold 16 bytes of row li, so a plain 16-byte load per lane takes 64 bytes
+// of each of 16 rows: half of every line, the other half with the next load.  Instead one load takes whole lines
+// of eight rows (lanes li < 8 the low half of row li, lanes li >= 8 the high half of row li - 8), the next load
+// rows 8 .. 15 the same way, and before the products the halves of each row of 16 lanes change places
+// (`swap_halves`, one DPP move a register).  Loads of whole lines can carry the non-temporal hint (the data needs
+// no place in the caches), which memory answers a tenth to a fifth faster; on half lines the hint costs time.
+typedef unsigned int fx_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_lines16(const void* p) {
+    const fx_u32x4 v = __builtin_nontemporal_load((const fx_u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+// keep: this lane's value where its bank (four lanes) is not in BANKS, else other's value from the lane eight
+// further round its row of 16 lanes.  With (first, second) the two loads described above:
+// low half of row li = swap_halves<0xC>(first, second), high half = swap_halves<0x3>(second, first).
+template <int BANKS>
+__device__ __forceinline__ uint4 swap_halves(uint4 keep, uint4 other) {
+    uint4 r;
+    r.x = __builtin_amdgcn_update_dpp(keep.x, other.x, 0x128, 0xF, BANKS, false);      // 0x128: row_ror:8
+    r.y = __builtin_amdgcn_update_dpp(keep.y, other.y, 0x128, 0xF, BANKS, false);
+    r.z = __builtin_amdgcn_update_dpp(keep.z, other.z, 0x128, 0xF, BANKS, false);
+    r.w = __builtin_amdgcn_update_dpp(keep.w, other.w, 0x128, 0xF, BANKS, false);
+    return r;
+}
+
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 
 // Compute units of the current device, asked for once per device.  Dispatch decisions that weigh a launch's

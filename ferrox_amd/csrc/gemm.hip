@@ -666,32 +666,9 @@ __device__ __forceinline__ void load8f(const float* p, bool ok, float* v) {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
-// The few-row product's weight loads.  A 16 x 16 x 32 product wants lane (li, grp) of a wave to hold row li, k
-// 8 grp .. 8 grp + 7 of a set of 16 weight rows; loaded that way one instruction takes 64 bytes of each of 16
-// rows, half of every 128-byte line, and the other half comes with the next load.  Instead a load takes whole
-// lines of 8 rows: its lanes li < 8 take (row li, the low 32 k of 64), lanes li >= 8 (row li - 8, the high 32 k);
-// the next load takes rows 8 .. 15 the same way, and before the products the halves of each row of 16 lanes
-// change places (`swap_halves`, one DPP move a register).  Loads of whole lines can carry the non-temporal hint
-// (weights are read once a step and need no place in the caches), which memory answers about a tenth faster;
-// on half lines the hint costs time.  Measured at 8 tokens of the A2.7B sizes: the experts' gate/up product
-// 69.1 -> 64.4 us, their down product 36.6 -> 32.7 us, the head 132 -> 101 us (4.7 -> 6.2 TB/s).
-typedef unsigned int fx_u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 load_lines16(const void* p) {
-    const fx_u32x4 v = __builtin_nontemporal_load((const fx_u32x4*)p);
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
-// keep: this lane's value where its bank (four lanes) is not in BANKS, else other's value from the lane eight
-// further round its row of 16 lanes
-template <int BANKS>
-__device__ __forceinline__ uint4 swap_halves(uint4 keep, uint4 other) {
-    uint4 r;
-    r.x = __builtin_amdgcn_update_dpp(keep.x, other.x, 0x128, 0xF, BANKS, false);
-    r.y = __builtin_amdgcn_update_dpp(keep.y, other.y, 0x128, 0xF, BANKS, false);
-    r.z = __builtin_amdgcn_update_dpp(keep.z, other.z, 0x128, 0xF, BANKS, false);
-    r.w = __builtin_amdgcn_update_dpp(keep.w, other.w, 0x128, 0xF, BANKS, false);
-    return r;
-}
-
+// The weights come in whole lines with the non-temporal hint (`load_lines16`, `swap_halves`).  Measured at 8
+// tokens of the A2.7B sizes against 16-byte loads of half lines: the experts' gate/up product 69.1 -> 64.4 us, their
+// down product 36.6 -> 32.7 us, the head 132 -> 101 us (4.7 -> 6.2 TB/s).
 // NW: sets of 16 weight rows per wave; in dual mode set a is the gate (a even) or up (a odd) rows of
 // column group a / 2.
 template <int MT, int WAVES, int NW, bool DUAL, int EPI, bool NORM = false, bool ROPE = false>
