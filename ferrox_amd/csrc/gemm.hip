@@ -177,15 +177,26 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
 //   ACT_RELU       max(x, 0)
 enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_GELU = 2, ACT_RELU = 3, ACT_COUNT = 4 };
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
-__device__ __forceinline__ float gated_f(int act, float gate, float up) {
+template <int ACT>
+__device__ __forceinline__ float gated_c(float gate, float up) {
     float a;
-    switch (act) {
-        case ACT_GELU_TANH: a = 0.5f * gate * (1.0f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate))); break;
-        case ACT_GELU: a = 0.5f * gate * (1.0f + erff(gate * 0.7071067811865476f)); break;
-        case ACT_RELU: a = fmaxf(gate, 0.0f); break;
-        default: a = silu_f(gate); break;
-    }
+    if constexpr (ACT == ACT_GELU_TANH) a = 0.5f * gate * (1.0f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate)));
+    else if constexpr (ACT == ACT_GELU) a = 0.5f * gate * (1.0f + erff(gate * 0.7071067811865476f));
+    else if constexpr (ACT == ACT_RELU) a = fmaxf(gate, 0.0f);
+    else a = silu_f(gate);
     return a * up;
+}
+// f(the activation as a compile-time constant): an epilogue calls this once around its loops, so that the choice is
+// one jump per block and not work inside the loops (left inside, the compiler works out every activation for every
+// element and picks one: the tiled products of a prompt were 4-10 % slower for it)
+template <typename F>
+__device__ __forceinline__ void with_activation(int act, F&& f) {
+    switch (act) {
+        case ACT_GELU_TANH: f(std::integral_constant<int, ACT_GELU_TANH>{}); break;
+        case ACT_GELU: f(std::integral_constant<int, ACT_GELU>{}); break;
+        case ACT_RELU: f(std::integral_constant<int, ACT_RELU>{}); break;
+        default: f(std::integral_constant<int, ACT_SILU>{}); break;
+    }
 }
 
 // ===========================================================================
@@ -325,6 +336,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) bias_v[j] = 0.f;
     if (!DUAL && g.bias) load_strided_as_float<NT, 16>(g.bias, g.bias_dtype, n0 + wn * WN + (lane & 15), g.N, bias_v);
+    if constexpr (DUAL) {
+        with_activation(g.act, [&](auto ac) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int ml = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
+                    if (ml >= r_end) continue;
+                    const int m = g.c_rows ? g.c_rows[ml] : ml;
+#pragma unroll
+                    for (int j = 0; j < NT; j += 2) {
+                        const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
+                        if (n < g.N)
+                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r], acc[i][j + 1][r]));
+                    }
+                }
+        });
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -332,14 +362,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
             const int ml = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
             if (ml >= r_end) continue;
             const int m = g.c_rows ? g.c_rows[ml] : ml;
-            if (DUAL) {
-#pragma unroll
-                for (int j = 0; j < NT; j += 2) {
-                    const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
-                    if (n < g.N)
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, acc[i][j][r], acc[i][j + 1][r]));
-                }
-            } else {
+            {
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
                     const int n = n0 + wn * WN + j * 16 + (lane & 15);
@@ -390,10 +413,10 @@ __device__ __forceinline__ void wait_loads_but() {
 }
 
 // The K loop of one wave for NA active row blocks (blocks wm, wm+2, ... of the tile).
-template <int NA, int MT, int NT, int TM, int TN, int NSA, int NSB>
+template <int NA, int MT, int NT, int TM, int TN, int NSA, int NSB, bool STREAM>
 __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* const (&a_src)[TM / 64],
                                             const bf16* const (&b_src)[TN / 64], bf16* stages, int K, int wave,
-                                            int a_off, int b_off, int sw, int kq, long kb_stride, bool stream_w) {
+                                            int a_off, int b_off, int sw, int kq, long kb_stride) {
     static_assert(NSA >= 2 && NSB >= NSA, "the weights' ring is at least as deep as the rows'");
     const int koff0 = (kq ^ sw) * 8, koff1 = ((4 + kq) ^ sw) * 8;
     constexpr int NLA = TM / 64, NLB = TN / 64;     // wave-loads per wave and step
@@ -414,12 +437,9 @@ __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* 
         for (int i = 0; i < NLB; ++i) {
             // weights that nothing reads twice come with the non-temporal hint (cache policy operand 2): each
             // load takes whole 128-byte lines that need no place in the caches, and memory delivers them up to a
-            // tenth faster (a 2 GiB read: 7.16 against 6.47 TB/s).  Where a load instruction takes half lines,
-            // as the skinny kernel's do, the hint costs time instead, so that kernel loads plainly.
-            if (stream_w)
-                __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 2);
-            else
-                __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, 0);
+            // tenth faster.  A compile-time choice: as a flag tested here the tiled products of a prompt, which
+            // do not stream, were 3-4 % slower.
+            __builtin_amdgcn_global_load_lds((fx_global_ptr)(b_src[i] + w0), (fx_lds_ptr)(st + (wave + 8 * i) * 512), 16, 0, STREAM ? 2 : 0);
         }
     };
     // Each step issues the rows of step kt + NSA - 1, then the weights of step kt + NSB - 1.  Weights come from
@@ -465,7 +485,7 @@ __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* 
     wait_loads_but<0>();                       // the loads past the end, before the block leaves
 }
 
-template <int TMB, int TN, int NS, bool DUAL, int EPI, int NSA = NS>
+template <int TMB, int TN, int NS, bool DUAL, int EPI, int NSA = NS, bool STREAM = false>
 __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     constexpr int TM = TMB * 16;
     constexpr int MT = TMB / 2;            // row blocks per wave
@@ -540,7 +560,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
     const int a_off = (wm * 16 + (lane & 15)) * 64, b_off = (wn * WN + (lane & 15)) * 64;
     const int na = (nblk - wm + 1) >> 1;         // this wave's active row blocks
 #define FX_LOOP(NA) \
-    wide_k_loop<NA, MT, NT, TM, TN, NSA, NS>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride, g.stream_w != 0)
+    wide_k_loop<NA, MT, NT, TM, TN, NSA, NS, STREAM>(acc, a_src, b_src, stages, g.K, wave, a_off, b_off, sw, kq, g.kb_stride)
     if constexpr (MT >= 4) {
         if (na > 3 * MT / 4) FX_LOOP(MT);
         else if (na > MT / 2) FX_LOOP(3 * MT / 4);
@@ -570,6 +590,25 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
             m_of[i][r] = g.c_rows ? g.c_rows[safe] : safe;
             scale_of[i][r] = (EPI == EPI_RESID && g.row_scale) ? g.row_scale[safe] : 1.f;
         }
+    if constexpr (DUAL) {
+        with_activation(g.act, [&](auto ac) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
+                    if (ml >= r_end || ml >= r0 + TM) continue;
+                    const int m = m_of[i][r];
+#pragma unroll
+                    for (int j = 0; j < NT; j += 2) {
+                        const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
+                        if (n < g.N)
+                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r], acc[i][j + 1][r]));
+                    }
+                }
+        });
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         float old[4][NT];
@@ -587,14 +626,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
             const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
             if (ml >= r_end || ml >= r0 + TM) continue;
             const int m = m_of[i][r];
-            if (DUAL) {
-#pragma unroll
-                for (int j = 0; j < NT; j += 2) {
-                    const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
-                    if (n < g.N)
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, acc[i][j][r], acc[i][j + 1][r]));
-                }
-            } else {
+            {
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
                     const int n = n0 + wn * WN + j * 16 + (lane & 15);
@@ -623,10 +655,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
 // MFMA operands, no LDS staging.  A block owns NW sets of 16 rows of W and up
 // to 16*MT logical rows; its WAVES waves split K between them in pieces of 128
 // (with few accumulators, the next piece's loads are issued before this piece's
-// products) and their partial sums are added in wave order through LDS.  In each
-// of the four loads of a piece the lanes (i = lane%16, g = lane/16) of a row
-// read 64 contiguous bytes of W row n0+i; the activations use the same
-// k -> lane assignment, which is all the MFMA needs to be right.
+// products) and their partial sums are added in wave order through LDS.  A
+// product wants lane (i = lane%16, g = lane/16) to hold 16 bytes (k 8g..8g+7 of
+// every 32) of W row n0+i; they arrive in whole 128-byte lines, two loads and an
+// exchange between lanes per 64 k (see `load_lines16`).  The activations use the
+// same k -> lane assignment, which is all the MFMA needs to be right.
 // W is the A operand: the accumulator of lane (m = lane%16, g) holds
 // C[m][n0 + 4g + r], r = 0..3.
 // ---------------------------------------------------------------------------
@@ -1041,7 +1074,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             float o = v[r] * rstd;
             asm volatile("" : "+v"(o));          // the product is rounded before the bias is added (no fused multiply-add)
             if (DUAL) {
-                from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_f(g.act, o, v2[r]));
+                with_activation(g.act, [&](auto ac) { from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(o, v2[r])); });
                 continue;
             }
             if (g.bias) o += bias_v[r];
@@ -1137,7 +1170,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             float v = acc[i][j];
             float* out = (float*)g.C + (size_t)m * g.ldc + n;
             if (DUAL) {
-                *out = gated_f(g.act, v, acc2[i][j]);
+                with_activation(g.act, [&](auto ac) { *out = gated_c<decltype(ac)::value>(v, acc2[i][j]); });
             } else {
                 if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
                 if (EPI == EPI_RESID) {
@@ -1198,19 +1231,30 @@ FX_API int fx_debug_set(const char* key, int value) {
     return 1;
 }
 
+template <int TMB, int TN, int NS, int NSA, bool STREAM>
+static void launch_wide_as(const GemmArgs& g, int epi, dim3 grid, hipStream_t s) {
+    switch (epi) {
+        case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE, NSA, STREAM><<<grid, 512, 0, s>>>(g); break;
+        case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32, NSA, STREAM><<<grid, 512, 0, s>>>(g); break;
+        case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID, NSA, STREAM><<<grid, 512, 0, s>>>(g); break;
+        default:
+            if constexpr (TN % 128 == 0) gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_GATED, NSA, STREAM><<<grid, 512, 0, s>>>(g);
+            break;
+    }
+}
 template <int TMB, int TN, int NS, int NSA = NS>
 static void launch_wide(GemmArgs g, int epi, int m_tiles, hipStream_t s) {
     g.n_col_tiles = ceil_div(g.N, epi == EPI_GATED ? TN / 2 : TN);
     g.n_row_tiles = m_tiles;
     dim3 grid(g.expert_offsets ? 8 * ceil_div(m_tiles, 8) * g.n_col_tiles : 8 * ceil_div((long)g.n_col_tiles * m_tiles, 8));
-    switch (epi) {
-        case EPI_STORE: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE, NSA><<<grid, 512, 0, s>>>(g); break;
-        case EPI_STORE_F32: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_STORE_F32, NSA><<<grid, 512, 0, s>>>(g); break;
-        case EPI_RESID: gemm_bf16_wide_kernel<TMB, TN, NS, false, EPI_RESID, NSA><<<grid, 512, 0, s>>>(g); break;
-        default:
-            if constexpr (TN % 128 == 0) gemm_bf16_wide_kernel<TMB, TN, NS, true, EPI_GATED, NSA><<<grid, 512, 0, s>>>(g);
-            break;
+    // the streaming variant exists for the tiles that few rows take (up to 192 of them)
+    if constexpr (TMB <= 12) {
+        if (g.stream_w) {
+            launch_wide_as<TMB, TN, NS, NSA, true>(g, epi, grid, s);
+            return;
+        }
     }
+    launch_wide_as<TMB, TN, NS, NSA, false>(g, epi, grid, s);
 }
 
 template <int MT, int WAVES, int NW>

@@ -2,7 +2,9 @@
 // kernels, as the ceilings that the engine's kernels are priced against beside the published peaks.
 // Nothing on the product path calls them (bench.py does).
 //
-//  fx_probe_read : every byte of a buffer once, 16 bytes per lane and load, summed so that the loads stay
+//  fx_probe_read : every byte of a buffer once, 16 bytes per lane and load, summed so that the loads stay;
+//                  `stream` != 0: the loads carry the non-temporal hint, as the engine's loads of weights, keys
+//                  and values do
 //  fx_probe_copy : buffer to buffer, 16 bytes per lane
 //  fx_probe_mfma : a loop of independent bf16 MFMA products on registers, no memory traffic
 //  fx_probe_mark : an empty kernel whose grid size is a label: in a profiler's kernel trace it says which part
@@ -14,12 +16,18 @@ FX_DEFINE_LAST_ERROR()
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 probe_bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float probe_f32x4;
 
+template <bool STREAM>
+__device__ __forceinline__ uint4 probe_load(const uint4* p) {
+    if constexpr (STREAM) return load_lines16(p);
+    else return *p;
+}
+template <bool STREAM>
 __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ src, size_t n16, unsigned* __restrict__ out) {
     const size_t groups = n16 / 1024;                 // whole groups of 1024 x 16 bytes: four loads in flight per lane
     unsigned acc = 0;
     for (size_t g = blockIdx.x; g < groups; g += gridDim.x) {
         const uint4* p = src + g * 1024 + threadIdx.x;
-        const uint4 a = p[0], b = p[256], c = p[512], d = p[768];
+        const uint4 a = probe_load<STREAM>(p), b = probe_load<STREAM>(p + 256), c = probe_load<STREAM>(p + 512), d = probe_load<STREAM>(p + 768);
         acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
     }
     if (blockIdx.x == 0)                              // what is left of the buffer
@@ -61,11 +69,12 @@ FX_API int fx_probe_mark(void* stream, int label) {
     return 0;
 }
 
-FX_API int fx_probe_read(void* stream, const void* src, long n_bytes, void* out) {
+FX_API int fx_probe_read(void* stream, const void* src, long n_bytes, void* out, int non_temporal) {
     FX_REQUIRE(n_bytes > 0 && n_bytes % 16 == 0 && ((uintptr_t)src % 16) == 0, "probe_read: a 16-byte aligned buffer of whole 16 bytes");
     const size_t n16 = (size_t)n_bytes / 16;
     const unsigned blocks = (unsigned)((n16 + 1023) / 1024 < 256 * 16 ? (n16 + 1023) / 1024 : 256 * 16);
-    probe_read_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)src, n16, (unsigned*)out);
+    if (non_temporal) probe_read_kernel<true><<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)src, n16, (unsigned*)out);
+    else probe_read_kernel<false><<<blocks, 256, 0, (hipStream_t)stream>>>((const uint4*)src, n16, (unsigned*)out);
     FX_CHECK_LAUNCH("probe_read");
     return 0;
 }
