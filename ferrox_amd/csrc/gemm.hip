@@ -1214,6 +1214,7 @@ static int g_few_rows = 3;     // "few_rows": sorted by expert, up to this many 
 static int g_head_rows = 16;   // "head_rows": plain rows against very many weight rows go to the tiled kernel from more than this many on
 static int g_tile64_rows = 20; // "tile64_rows": experts with up to this many rows on average take tiles of 64 rows
 static int g_no_wide = 0;      // "wide": 0 sends many-row products to the register-staged tiled kernel, 1 (default) by the sizes,
+static int g_plain_rows = 0;   // "plain_rows": plain rows up to this many go to the product for few rows whatever the weight rows (0: by the sizes)
 static int g_stream_w = -1;    // "stream_w": 1 / 0 forces the non-temporal hint on the tiled kernel's weight loads on / off; -1: by the shape
 static int g_wide_grouped = 0; // "wide_grouped": as "wide", for products whose rows are sorted by expert only
 static int g_wide_force = 0;   //         256, 192, 128, 64, 12 or 4 (tiles of 64 rows) picks that tile of the LDS-tiled kernel
@@ -1227,7 +1228,8 @@ FX_API int fx_debug_set(const char* key, int value) {
     if (!strcmp(key, "wide")) { g_no_wide = !value; g_wide_force = value > 1 ? value : 0; return 0; }
     if (!strcmp(key, "wide_grouped")) { g_wide_grouped = value > 1 ? value : 0; return 0; }
     if (!strcmp(key, "stream_w")) { g_stream_w = value; return 0; }
-    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, head_rows, wide)", key);
+    if (!strcmp(key, "plain_rows")) { g_plain_rows = value; return 0; }
+    FX_REQUIRE(false, "gemm: no debug switch '%s' (skinny_sets, skinny_row_tiles, skinny_waves, few_rows, head_rows, tile64_rows, wide, wide_grouped, stream_w, plain_rows)", key);
     return 1;
 }
 
@@ -1431,9 +1433,17 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     // holds an expert's share, streams the weights at the same speed whatever the rows (400 us at 5.9 TB/s); decode
     // steps of 48 and 64 sequences 10.3 -> 10.0 and 12.0 -> 11.4 ms, of 17 to 64 of the larger model's sizes 8-24 %
     // less; with three rows an expert the product for few rows is still 1-2 % ahead of the tiles of 64 rows.
-    const long few_limit = expert_offsets && wide_ok ? g_few_rows : 64;
+    // 65 to 256 plain rows against so few weight rows that the tiled kernel, whose smallest tiles are 128 x 128, would
+    // run on 32 CUs or fewer (the attention's output product): its chain of K steps takes 20-25 us whatever the rows,
+    // the product for few rows, 32 or 64 rows a block, streams the weights through every CU (2,048 x 2,048 weights:
+    // 11 us up to 128 rows and 18 us up to 256 against 20-24 us; 3,584 x 3,584: 26-30 us up to 128 rows against 31-39;
+    // with 48 tiles, the q/k/v product, the tiled kernel is ahead)
+    const bool few_tiles = !expert_offsets && !pair_ids && M > 64 && M <= 256 && (long)ceil_div(N, 128) * ceil_div(M, 128) <= 32 && !g_wide_force;
+    const long plain_limit = g_plain_rows > 0 ? g_plain_rows : (few_tiles ? 256 : 64);
+    const long few_limit = expert_offsets ? (wide_ok ? g_few_rows : 64) : plain_limit;
     if (g.vec_ok && (per_group <= few_limit || pair_ids) && !many_columns) {
         int mt = pair_ids ? 1 : (per_group <= 16 ? 1 : (per_group <= 32 ? 2 : 4));
+        if (!expert_offsets && !pair_ids && M > 64 && (long)ceil_div(N, 32) * ceil_div(M, 64) < 256) mt = 2;     // more blocks where they are few
         const bool dual = epi == EPI_GATED;
         // 33 to 64 plain rows against few weight rows (the attention's output product: 2,048): four row tiles a
         // block leave 128 blocks; a block per row tile, with two sets of weight rows, gives 256 and every block a

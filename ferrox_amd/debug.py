@@ -22,7 +22,7 @@ import ctypes
 import torch
 
 KERNEL_SWITCH_DEFAULTS = {("gemm", "skinny_sets"): 0, ("gemm", "skinny_row_tiles"): 0, ("gemm", "skinny_waves"): 0, ("gemm", "few_rows"): 3, ("gemm", "head_rows"): 16, ("gemm", "tile64_rows"): 20,
-                          ("gemm", "wide"): 1, ("gemm", "wide_grouped"): 0, ("gemm", "stream_w"): -1, ("attention", "direct_stages"): 2, ("attention", "direct_groups"): 0}
+                          ("gemm", "wide"): 1, ("gemm", "wide_grouped"): 0, ("gemm", "stream_w"): -1, ("gemm", "plain_rows"): 0, ("attention", "direct_stages"): 2, ("attention", "direct_groups"): 0}
 
 
 class RoutingTrace:

@@ -29,7 +29,8 @@ def close(got, want, dtype, what, k=1):
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 100, 96), (16, 256, 128), (17, 257, 200), (33, 72, 40),
                                     (64, 64, 64), (130, 300, 520), (257, 129, 1032), (3, 50, 100),
                                     (130, 300, 512), (257, 129, 1024), (300, 520, 64), (513, 72, 128), (65, 16, 192),
-                                    (40, 65600, 64), (64, 65536, 128)])
+                                    (40, 65600, 64), (64, 65536, 128), (128, 2048, 2048), (256, 3584, 512), (200, 96, 264),
+                                    (256, 4200, 64)])
 def test_gemm_plain_and_epilogues(dtype, M, N, K):
     from ferrox_amd import ops
     a, w = rnd(M, K, dtype=dtype), rnd(N, K, dtype=dtype, seed=1)
