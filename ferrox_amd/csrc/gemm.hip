@@ -120,11 +120,14 @@ __device__ __forceinline__ unsigned long long same_expert_lanes(int e, int bits)
     return e >= 0 ? m : 0ull;
 }
 
-// Up to 64 unsorted pairs: the experts that occur, in ascending order, get one tile per 16 of their
-// pairs, and a tile's rows are those pairs in their order.  Every wave works this out by itself
-// from the ids (a lane per pair).  After those tiles come the experts that every row takes
-// (n_always of them, a shared expert cut into pieces), one tile each.  Returns false for a tile
-// past the last one; else the expert, and for tile row lane % 16 the rows of A and C (or -1).
+// Up to 64 unsorted pairs: the experts that occur, in the order of their first pairs, get one tile per 16 of
+// their pairs, and a tile's rows are those pairs in their order.  Every wave works this out by itself from the
+// ids (a lane per pair) with ballots and counts alone: a lane that holds an expert's first pair counts the tiles
+// of the first pairs in the lanes below it (an expert has one to four tiles, so four ballots), and what the tile's
+// owner knows is read from its lane directly.  (A loop over the experts that occur, two exchanges between lanes
+// each, cost a wave 1-2 us before its first load.)  After those tiles come the experts that every row takes
+// (n_always of them, a shared expert cut into pieces), one tile each.  Returns false for a tile past the last one;
+// else the expert, and for tile row lane % 16 the rows of A and C (or -1).
 __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& expert, int& a_row, int& c_row) {
     const int lane = threadIdx.x & 63, li = lane & 15;
     int e = lane < g.M ? g.pair_ids[lane] : -1;
@@ -134,12 +137,13 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
     const unsigned long long same = same_expert_lanes(e, bits);
     const bool first = e >= 0 && lane == __ffsll((long long)same) - 1;
     const int my_tiles = (__popcll(same) + 15) >> 4;
-    int before = 0, total = 0;      // tiles of the experts that occur and are smaller than this lane's; of all
-    for (unsigned long long m = __ballot(first); m; m &= m - 1) {
-        const int src = __ffsll((long long)m) - 1;
-        const int oe = __shfl(e, src, 64), ot = __shfl(my_tiles, src, 64);
-        if (oe < e) before += ot;
-        total += ot;
+    const unsigned long long below = (1ull << lane) - 1;
+    int before = 0, total = 0;      // tiles of the experts whose first pair comes earlier than this lane's; of all
+#pragma unroll
+    for (int t = 1; t <= 4; ++t) {
+        const unsigned long long f = __ballot(first && my_tiles >= t);
+        before += __popcll(f & below);
+        total += __popcll(f);
     }
     a_row = c_row = -1;
     if (tile >= total) {
@@ -153,18 +157,20 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
         return true;
     }
     const unsigned long long sel = __ballot(first && tile >= before && tile < before + my_tiles);
-    const int src = __ffsll((long long)sel) - 1;
-    expert = __shfl(e, src, 64);
-    const int skip = (tile - __shfl(before, src, 64)) * 16;      // pairs of this expert in its earlier tiles
-    unsigned long long rows = ((unsigned long long)(unsigned)__shfl((int)(same >> 32), src, 64) << 32) |
-                              (unsigned)__shfl((int)(unsigned)same, src, 64);
+    const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)sel) - 1);
+    expert = __builtin_amdgcn_readlane(e, src);
+    const int skip = (tile - __builtin_amdgcn_readlane(before, src)) * 16;      // pairs of this expert in its earlier tiles
+    unsigned long long rows = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(same >> 32), src) << 32) |
+                              (unsigned)__builtin_amdgcn_readlane((int)(unsigned)same, src);
+    int mine = -1;                  // pair number skip + li of this expert, if it has so many
     for (int j = 0; j < skip + 16 && rows; ++j) {
         const int p = __ffsll((long long)rows) - 1;
         rows &= rows - 1;
-        if (j == skip + li) {
-            c_row = p;
-            a_row = p / g.pair_div;
-        }
+        if (j == skip + li) mine = p;
+    }
+    if (mine >= 0) {
+        c_row = mine;
+        a_row = mine / g.pair_div;
     }
     return true;
 }
