@@ -68,6 +68,19 @@ struct GemmArgs {
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
 
+// v of this lane and of all lanes below it, added up: inside each row of 16 lanes by four shifted adds, then
+// row 0's total onto row 1 and row 2's onto row 3, then the lower half's total onto the upper half (DPP moves of
+// gfx9, no LDS; a lane with no source lane adds 0)
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);      // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);      // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);      // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);      // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);      // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);      // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // block -> (first logical row, end of rows, expert).  Plain: tiles of TM rows.
 // Grouped: expert e has ceil(rows_e / TM) tiles, in the order of the experts; a tile past the
 // last one gets r0 = -1.  Every wave finds its tile by itself, 64 experts at a time: each lane
@@ -91,22 +104,17 @@ __device__ __forceinline__ void locate_rows(const GemmArgs& g, int tile, int& r0
         const int e = base + lane;
         const int b = e < g.E ? g.expert_offsets[e] : 0, en = e < g.E ? g.expert_offsets[e + 1] : 0;
         const int nt = (en - b + TM - 1) / TM;
-        int incl = nt;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int u = __shfl_up(incl, o, 64);
-            if (lane >= o) incl += u;
-        }
+        const int incl = wave_inclusive_sum(nt);
         const int first = before + incl - nt;
         const unsigned long long hit = __ballot(tile >= first && tile < first + nt);
-        if (hit) {
-            const int src = __ffsll((long long)hit) - 1;
-            r0 = __shfl(b + (tile - first) * TM, src, 64);
-            r_end = __shfl(en, src, 64);
+        if (hit) {      // (the same in every lane: what the owner knows is read from its lane, no exchange)
+            const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)hit) - 1);
+            r0 = __builtin_amdgcn_readlane(b + (tile - first) * TM, src);
+            r_end = __builtin_amdgcn_readlane(en, src);
             expert = base + src;
             return;
         }
-        before += __shfl(incl, 63, 64);
+        before += __builtin_amdgcn_readlane(incl, 63);
     }
 }
 
