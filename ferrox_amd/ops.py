@@ -451,6 +451,9 @@ def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, 
           int(window or 0), float(scale), int(tile_q))
 
 
+SPLIT_PARTIAL_ROUNDS = True      # decode attention: more chunks where the blocks' last round over the CUs would be far from full
+
+
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
                      waves=0) -> None:
@@ -459,13 +462,23 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
     batch); bfloat16, whose blocks of eight waves share a chunk, cuts every sequence's own range of keys (from its
     window's first key to its position) into that many equal chunks of whole tiles of 64, and by default takes the
     fewest chunks that still put about two thousand waves on the GPU: one chunk, and no merge launch, from 256
-    (sequence, kv head) pairs on."""
+    (sequence, kv head) pairs on, unless the blocks' last round over the CUs would be far from full."""
     n = item_seq.numel()
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
             pairs = n * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
             want = max(1, 2048 // max(1, pairs * 8))
+            # More (sequence, kv head) pairs than CUs: a CU holds one block of eight waves, so the blocks run in
+            # rounds, and a last round that is far from full (272 blocks on 256 CUs: 17 sequences of 16 kv heads)
+            # costs as much as a full one.  Eight chunks a sequence, which the launch then gives to blocks of one or
+            # two waves, fill the CUs evenly: 17 sequences at 2,060 keys 80 -> 58 us, 24 sequences 87 -> 79 us, 17 at
+            # 8,200 keys 285 -> 192 us; where the last round is at least 85 % full one chunk stays ahead.
+            cus = compute_units(q.device)
+            if SPLIT_PARTIAL_ROUNDS and pairs > cus and max_kv_len >= 1024:
+                rounds = -(-pairs // cus)
+                if (rounds * cus - pairs) / (rounds * cus) >= 0.15:
+                    want = 8
             chunk = max(64, -(-(-(-max_kv_len // want)) // 64) * 64)
     splits = max(1, -(-max_kv_len // chunk))
     part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)

@@ -695,6 +695,38 @@ def test_decode_attention_of_a_short_sequence_beside_a_very_long_one():
         close(out[last[s_]].reshape(nh, hd), ref, dtype, f"sequence of {L} keys")
 
 
+def test_decode_attention_of_more_sequences_than_fill_the_cus_once():
+    """20 sequences of 16 kv heads are 320 blocks for 256 CUs: the chunks are then chosen by how full the blocks' last
+    round would be (eight a sequence here, one with 16 sequences), and sequences of every length, down to one key and
+    up to the bound, must come out as plain attention gives them, with the chunks chosen and with one."""
+    from ferrox_amd import ops
+    nh, nkv, hd, bs, dtype = 16, 16, 64, 64, torch.bfloat16
+    lens = [1100, 1, 64, 65, 1087, 1088, 1089, 700, 513, 128] * 2
+    n_pages = sum(-(-L // bs) for L in lens) + 3
+    q, k, v, q_rot, k_pages, v_pages, table, pos, seq, toks = paged_setup(dtype, nh, nkv, hd, bs, lens, 1e6, hd, n_pages)
+    scale = 1.0 / math.sqrt(hd)
+    kp, vp = k_pages.double().cpu(), v_pages.double().cpu()
+    ends, last = 0, []
+    for L in lens:
+        ends += L
+        last.append(ends - 1)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    outs = []
+    for chunk in (None, 1152):
+        out = torch.zeros(len(toks), nh * hd, dtype=dtype, device=DEV)
+        ops.attention_decode(q_rot, out, k_pages, v_pages, table, pos, i32(list(range(len(lens)))), i32(last), nh, nkv, hd, bs, 0,
+                             scale, max_kv_len=1152, chunk=chunk)
+        outs.append(out)
+    for s_, L in enumerate(lens):
+        tab = table.cpu()[s_].long()[: -(-L // bs)]
+        ks = kp[tab].permute(0, 2, 1, 3).reshape(-1, nkv, hd)[:L]
+        vs = vp[tab].permute(0, 3, 1, 2).reshape(-1, nkv, hd)[:L]
+        qs = q_rot[last[s_]].double().cpu().reshape(nh, hd)
+        ref = torch.stack([torch.softmax((ks[:, h] @ qs[h]) * scale, 0) @ vs[:, h] for h in range(nh)])
+        for out, what in zip(outs, ("chunks as chosen", "one chunk")):
+            close(out[last[s_]].reshape(nh, hd), ref, dtype, f"sequence {s_} of {L} keys, {what}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,H,E,k,renorm", [(1, 64, 8, 2, False), (7, 96, 6, 3, True), (33, 200, 60, 4, False),
                                              (5, 128, 130, 8, True), (4, 72, 5, 5, False)])
