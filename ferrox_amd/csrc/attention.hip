@@ -622,11 +622,16 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
 template <int HD, int MAX_THREADS>
 __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(AttnArgs a) {
     extern __shared__ float wave_out[];      // [waves][rows][HD + 2]: o, then m and l
-    const int item = blockIdx.x, split = blockIdx.z;
+    // The grid is (heads, items, splits): blocks go to the eight XCDs in turn, so with the heads fastest every
+    // item's blocks are spread over all of them, and with the splits slowest a sequence's last, shorter chunks start
+    // last.  (With the items fastest and their number a multiple of eight, as a recorded step's is, an item's blocks
+    // all land on one XCD, and 17 live sequences beside 7 stand-ins give one XCD three sequences and the others
+    // two: 73 against 57 us.)
+    const int item = blockIdx.y, split = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
     const int li = lane & 15, g = lane >> 4;
     const int group = a.nh / a.nkv, gblocks = (group + 15) / 16;
-    const int kvh = blockIdx.y / gblocks, hb = blockIdx.y % gblocks;
+    const int kvh = blockIdx.x / gblocks, hb = blockIdx.x % gblocks;
     const int tok = a.item_tok[item];
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
@@ -1194,14 +1199,15 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
         attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
     } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
         const int group = nh / nkv;
-        dim3 gridm(n_items, nkv * ((group + 15) / 16), splits);
+        dim3 gridm(nkv * ((group + 15) / 16), n_items, splits);
         // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS
         const int rows = group < 16 ? group : 16;
         const int hdc = hd <= 32 ? 32 : (hd <= 64 ? 64 : (hd <= 128 ? 128 : 256));
         const int nw_max = hd <= 128 ? 8 : 4;      // the widest heads need the registers of half a block
         int nw = nw_max;
         FX_REQUIRE(waves >= 0 && waves <= nw_max, "attn_decode: %d waves per block, this head size takes up to %d", waves, nw_max);
-        const long n_blocks = (long)n_items * gridm.y * splits;
+        const long n_blocks = (long)n_items * gridm.x * splits;
+        FX_REQUIRE(n_items <= 65535 && splits <= 65535, "attn_decode: %d single queries in %d chunks each are more than a launch takes", n_items, splits);
         // fewer waves per block when there are blocks enough: a chunk's tiles then divide more evenly
         while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk || n_blocks * (nw / 2) >= 2048))
             nw >>= 1;
