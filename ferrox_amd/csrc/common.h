@@ -126,14 +126,46 @@ __device__ __forceinline__ void rotate_pair(float a, float b, float cs, float sn
 }
 
 // ---- wave (64 lanes) and block reductions in a fixed order ------------------
+// Sum and maximum over the 64 lanes of a wave, in every lane: a butterfly over the lanes 32, 16, 8, 4, 2 and 1
+// away, in that order (the order fixes the sum's bits).  The exchanges stay in the vector unit: the halves of the
+// wave and the rows of 16 lanes pairwise by the lane-swapping moves of gfx950, then rotations inside a row by DPP
+// (after the step over 8 lanes the lanes i and i ^ 8 hold the same value, so the lane four further round the row
+// holds what lane i ^ 4 holds, and so on down): the same values in the same order as exchanges through the LDS
+// crossbar (__shfl_xor) give, without waiting for it six times.
+__device__ __forceinline__ float wave_partner_32(float v, float& other) {
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    other = __uint_as_float(a[1]);
+    return __uint_as_float(a[0]);
+}
+__device__ __forceinline__ float wave_partner_16(float v, float& other) {
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    other = __uint_as_float(a[1]);
+    return __uint_as_float(a[0]);
+}
+template <int CTRL>
+__device__ __forceinline__ float row_rotated(float v) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    float o;
+    v = wave_partner_32(v, o) + o;
+    v = wave_partner_16(v, o) + o;
+    v += row_rotated<0x128>(v);      // row_ror:8
+    v += row_rotated<0x124>(v);      // row_ror:4
+    v += row_rotated<0x122>(v);      // row_ror:2
+    v += row_rotated<0x121>(v);      // row_ror:1
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    float o;
+    v = fmaxf(wave_partner_32(v, o), o);
+    v = fmaxf(wave_partner_16(v, o), o);
+    v = fmaxf(v, row_rotated<0x128>(v));
+    v = fmaxf(v, row_rotated<0x124>(v));
+    v = fmaxf(v, row_rotated<0x122>(v));
+    v = fmaxf(v, row_rotated<0x121>(v));
     return v;
 }
 
@@ -216,6 +248,19 @@ __device__ __forceinline__ uint4 swap_halves(uint4 keep, uint4 other) {
     r.z = __builtin_amdgcn_update_dpp(keep.z, other.z, 0x128, 0xF, BANKS, false);
     r.w = __builtin_amdgcn_update_dpp(keep.w, other.w, 0x128, 0xF, BANKS, false);
     return r;
+}
+
+// v of this lane and of all lanes below it, added up: inside each row of 16 lanes by four shifted adds, then
+// row 0's total onto row 1 and row 2's onto row 3, then the lower half's total onto the upper half (DPP moves of
+// gfx9, no LDS; a lane with no source lane adds 0)
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);      // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);      // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);      // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);      // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);      // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);      // row_bcast:31 into rows 2 and 3
+    return v;
 }
 
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -68,19 +68,6 @@ struct GemmArgs {
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
 
-// v of this lane and of all lanes below it, added up: inside each row of 16 lanes by four shifted adds, then
-// row 0's total onto row 1 and row 2's onto row 3, then the lower half's total onto the upper half (DPP moves of
-// gfx9, no LDS; a lane with no source lane adds 0)
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);      // row_shr:1
-    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);      // row_shr:2
-    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);      // row_shr:4
-    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);      // row_shr:8
-    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);      // row_bcast:15 into rows 1 and 3
-    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);      // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
 // block -> (first logical row, end of rows, expert).  Plain: tiles of TM rows.
 // Grouped: expert e has ceil(rows_e / TM) tiles, in the order of the experts; a tile past the
 // last one gets r0 = -1.  Every wave finds its tile by itself, 64 experts at a time: each lane

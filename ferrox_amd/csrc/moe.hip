@@ -27,6 +27,45 @@ enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
 //   GATE_SIGMOID scores each expert with 1/(1+exp(-logit)) instead
 //   (ferrox-moe/src/lib.rs:100-121).
 //   gate_out[t] = sigmoid(logits[t, E])  (decoder.rs:2670-2672).
+// The best (score, expert) of the wave in every lane: higher score first, then the lower expert.  Six exchanges
+// that stay in the vector unit (pairs inside a quad, quads, halves of a row of 16 lanes by DPP moves; rows and halves
+// of the wave by the lane-swapping moves of gfx950): the order is total, so the result is the one that exchanges
+// through the LDS crossbar gave, and a selection of k experts no longer waits 12 k times for that crossbar.
+__device__ __forceinline__ void better_of(float& best, int& bi, float ob, int oi) {
+    if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+    }
+}
+template <int CTRL>
+__device__ __forceinline__ void argmax_dpp_step(float& best, int& bi) {
+    const float ob = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(best), CTRL, 0xF, 0xF, true));
+    const int oi = __builtin_amdgcn_update_dpp(0, bi, CTRL, 0xF, 0xF, true);
+    better_of(best, bi, ob, oi);
+}
+__device__ __forceinline__ void wave_argmax(float& best, int& bi) {
+    argmax_dpp_step<0xB1>(best, bi);      // quad_perm [1,0,3,2]
+    argmax_dpp_step<0x4E>(best, bi);      // quad_perm [2,3,0,1]
+    argmax_dpp_step<0x141>(best, bi);     // row_half_mirror: the quads of eight lanes
+    argmax_dpp_step<0x140>(best, bi);     // row_mirror: the halves of a row
+    {
+        const unsigned ub = __float_as_uint(best), ui = (unsigned)bi;
+        const auto a = __builtin_amdgcn_permlane16_swap(ub, ub, false, false);
+        const auto b = __builtin_amdgcn_permlane16_swap(ui, ui, false, false);
+        best = __uint_as_float(a[0]);
+        bi = (int)b[0];
+        better_of(best, bi, __uint_as_float(a[1]), (int)b[1]);
+    }
+    {
+        const unsigned ub = __float_as_uint(best), ui = (unsigned)bi;
+        const auto a = __builtin_amdgcn_permlane32_swap(ub, ub, false, false);
+        const auto b = __builtin_amdgcn_permlane32_swap(ui, ui, false, false);
+        best = __uint_as_float(a[0]);
+        bi = (int)b[0];
+        better_of(best, bi, __uint_as_float(a[1]), (int)b[1]);
+    }
+}
+
 // selection for one token by one wave; `score` is E floats of LDS owned by the wave
 // (`es`: distance between the logits of neighbouring experts, 1 for a row of a [T, E] matrix)
 __device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm,
@@ -55,15 +94,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         for (int j = 0; j < k; ++j) {
             float best = sc;
             int bi = mine ? lane : 0x7fffffff;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float ob = __shfl_xor(best, o, 64);
-                const int oi = __shfl_xor(bi, o, 64);
-                if (ob > best || (ob == best && oi < bi)) {
-                    best = ob;
-                    bi = oi;
-                }
-            }
+            wave_argmax(best, bi);
             if (lane == j) {
                 my_w = best;
                 my_id = bi;
@@ -108,15 +139,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
                 bi = e;
             }
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ob = __shfl_xor(best, o, 64);
-            const int oi = __shfl_xor(bi, o, 64);
-            if (ob > best || (ob == best && oi < bi)) {
-                best = ob;
-                bi = oi;
-            }
-        }
+        wave_argmax(best, bi);
         if (lane == j) my_w = best;
         if (lane == 0) {
             store_shared(ids + t * k + j, bi);
@@ -210,14 +233,9 @@ __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E,
         for (int base = 0; base < R; base += 64) {
             const int r = base + lane;
             const int c = r < R ? cnt[r * E + e] : 0;
-            int v = c;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const int u = __shfl_up(v, o, 64);
-                if (lane >= o) v += u;
-            }
+            const int v = wave_inclusive_sum(c);
             if (r < R) cnt[r * E + e] = carry + v - c;
-            carry += __shfl(v, 63, 64);
+            carry += __builtin_amdgcn_readlane(v, 63);
         }
         if (lane == 0) offs[e + 1] = carry;
     }
@@ -227,14 +245,9 @@ __device__ __forceinline__ void align_block(const int* ids, int n, int k, int E,
         if (lane == 0) offs[0] = 0;
         for (int base = 0; base < E; base += 64) {
             const int e = base + lane;
-            int v = e < E ? offs[e + 1] : 0;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const int u = __shfl_up(v, o, 64);
-                if (lane >= o) v += u;
-            }
+            const int v = wave_inclusive_sum(e < E ? offs[e + 1] : 0);
             if (e < E) offs[e + 1] = carry + v;
-            carry += __shfl(v, 63, 64);
+            carry += __builtin_amdgcn_readlane(v, 63);
         }
     }
     __syncthreads();
@@ -366,14 +379,9 @@ __global__ __launch_bounds__(SORT_WAVES * 64) void moe_place_kernel(const int* _
         if (lane == 0) offs[0] = 0;
         for (int base = 0; base < E; base += 64) {
             const int e = base + lane;
-            int v = e < E ? offs[e + 1] : 0;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const int u = __shfl_up(v, o, 64);
-                if (lane >= o) v += u;
-            }
+            const int v = wave_inclusive_sum(e < E ? offs[e + 1] : 0);
             if (e < E) offs[e + 1] = carry + v;
-            carry += __shfl(v, 63, 64);
+            carry += __builtin_amdgcn_readlane(v, 63);
         }
     }
     __syncthreads();
