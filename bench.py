@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]          the one JSON line
     python bench.py --workload config3|config4|config5           serving runs through Engine.generate
-    python bench.py --kernel-table decode_b8|decode_b1|decode_b64|prefill_2048|prefill_512 [--out FILE]
+    python bench.py --kernel-table decode_b1|decode_b8|decode_b16|..|decode_b64|prefill_128|prefill_512|prefill_2048|prefill_4096 [--out FILE]
                                                                  per-kernel times under rocprofv3 (a child process)
 
 Model: the layer sizes of Qwen1.5-MoE-A2.7B with seeded random bf16 weights
