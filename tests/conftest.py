@@ -88,9 +88,19 @@ WIDE_G = {
     "max_window_layers": 1, "tie_word_embeddings": False,
 }
 # one layer of the smaller model's sizes under its real vocabulary: the head and the sampling at 151,936 columns
+# sixteen kv heads of 64 on a narrow model: enough (sequence, kv head) pairs for the decode attention of some twenty
+# sequences to be more blocks than the GPU has CUs, while the plain model stays fast at a few hundred positions
+MANY_K = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "hidden_act": "silu",
+    "num_hidden_layers": 1, "hidden_size": 128, "num_attention_heads": 16, "num_key_value_heads": 16, "head_dim": 64,
+    "num_experts": 12, "num_experts_per_tok": 3, "norm_topk_prob": False, "moe_intermediate_size": 48,
+    "shared_expert_intermediate_size": 96, "intermediate_size": 128, "decoder_sparse_step": 1, "mlp_only_layers": [],
+    "vocab_size": 300, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "max_position_embeddings": 2048,
+    "use_sliding_window": False, "sliding_window": 4096, "max_window_layers": 0, "tie_word_embeddings": False,
+}
 WIDE_DV = dict(WIDE_D, vocab_size=151936)
 TINY = {"DV": (WIDE_DV, 7), "A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (WIDE_D, 3), "E": (WIDE_E, 4), "F": (ODD_F, 5),
-        "G": (WIDE_G, 6), "H": (ODD_H, 8)}
+        "G": (WIDE_G, 6), "H": (ODD_H, 8), "K": (MANY_K, 9)}
 
 
 @pytest.fixture(scope="session")

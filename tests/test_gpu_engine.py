@@ -663,6 +663,38 @@ def test_recorded_decode_steps_of_many_requests(model_folders, name, n_live, dty
     check(got, folder, reqs, dtype, f"{name} {dtype} {n_live} requests decoded from graphs", routing)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_of_many_deep_sequences(model_folders, dtype):
+    """19 sequences of 16 kv heads, more than 512 positions deep, decoded together from a step recorded for 24: the
+    decode attention then has more (sequence, kv head) blocks than the GPU has CUs and cuts every sequence's keys
+    into eight chunks beside the stand-in rows' single key, the experts take the sorted layout; later steps have 17
+    live sequences in the same recording.  Every position against the plain model."""
+    cfg, seed = TINY["K"]
+    n_live, tail = 19, 6
+    rng = __import__("random").Random(19)
+    lengths = [rng.randint(514, 530) for _ in range(n_live)]
+    reqs = ru.make_requests(cfg["vocab_size"], [L + tail for L in lengths], 77)
+    ids = list(reqs)
+    steps = []
+    for i in range(0, n_live, 4):       # prompts whole, four a step, logits at every place
+        steps.append({"entries": [{"id": r, "tokens": reqs[r][:lengths[ids.index(r)]], "want": list(range(lengths[ids.index(r)]))}
+                                  for r in ids[i:i + 4]], "end": []})
+    for d in range(tail):
+        live = ids if d < tail // 2 else ids[:17]
+        steps.append({"entries": [{"id": r, "tokens": [reqs[r][lengths[ids.index(r)] + d]], "want": [0]} for r in live], "end": []})
+    steps[-1]["end"] = list(ids)
+    fed = {r: sum(len(e["tokens"]) for s_ in steps for e in s_["entries"] if e["id"] == r) for r in ids}
+    reqs = {r: reqs[r][:fed[r]] for r in ids}
+    bs = 64
+    pages = sum(-(-(L + tail) // bs) for L in lengths)
+    folder, runner = runner_for(model_folders, "K", dtype, block_size=bs, num_pages=pages, max_seqs=n_live)
+    routing = {} if dtype == "bfloat16" else None
+    got = ru.run_trace(runner, steps, routing)
+    assert {key[:2] for key in runner._graphs} == {(24, 1024)}, f"recorded {sorted(runner._graphs)}"
+    assert runner.manager.n_free_pages() == pages
+    check(got, folder, reqs, dtype, f"K {dtype} {n_live} deep sequences decoded from graphs", routing, cfg["hidden_size"])
+
+
 def test_recorded_decode_steps_at_production_width(model_folders):
     """the same at the layer sizes the engine is built for (bfloat16, pages of 64): 20 requests, so that the
     expert products take the sorted layout and the shared expert its own matrices on the second stream,
