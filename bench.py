@@ -407,7 +407,7 @@ def run_workload(name: str, args) -> int:
 
 # ---- per-kernel table (rocprofv3 around a child process) ----------------------------------------------------------
 KERNEL_TABLES = {"decode_b1": ("decode", 1), "decode_b8": ("decode", 8), "decode_b16": ("decode", 16), "decode_b17": ("decode", 17), "decode_b24": ("decode", 24),
-                 "decode_b32": ("decode", 32), "decode_b64": ("decode", 64),
+                 "decode_b32": ("decode", 32), "decode_b64": ("decode", 64), "decode_b96": ("decode", 96), "decode_b128": ("decode", 128),
                  "prefill_2048": ("prefill", 2048), "prefill_512": ("prefill", 512), "prefill_128": ("prefill", 128),
                  "prefill_4096": ("prefill", 4096)}
 
