@@ -1208,9 +1208,15 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
         FX_REQUIRE(waves >= 0 && waves <= nw_max, "attn_decode: %d waves per block, this head size takes up to %d", waves, nw_max);
         const long n_blocks = (long)n_items * gridm.x * splits;
         FX_REQUIRE(n_items <= 65535 && splits <= 65535, "attn_decode: %d single queries in %d chunks each are more than a launch takes", n_items, splits);
-        // fewer waves per block when there are blocks enough: a chunk's tiles then divide more evenly
-        while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk || n_blocks * (nw / 2) >= 2048))
-            nw >>= 1;
+        // fewer waves per block when there are blocks enough: a chunk's tiles then divide more evenly.  Whole
+        // sequences (one chunk) keep four waves a block, or get one each once the blocks number half the GPU's wave
+        // slots; two waves a block are behind both (decode steps of 72, 96 and 128 sequences of 16 kv heads: 12.3,
+        // 14.3 and 16.1 ms with two waves a block, 11.9, 13.5 and 15.9 with four, 11.7, 13.3 and 15.6 with one).
+        const long slots = 8L * fx_compute_units();
+        const int nw_min = splits > 1 ? 1 : 4;
+        while (nw > 1 && ((size_t)nw * rows * (hdc + 2) * 4 > 48 * 1024 || nw * 64 >= 2 * chunk)) nw >>= 1;
+        while (nw > nw_min && n_blocks * (nw / 2) >= slots) nw >>= 1;
+        if (splits == 1 && 2 * n_blocks >= slots) nw = 1;
         if (waves > 0 && (size_t)waves * rows * (hdc + 2) * 4 <= 48 * 1024) nw = waves;      // the caller's choice
         const size_t shm = (size_t)nw * rows * (hdc + 2) * 4;
         if (hd <= 32) attn_mfma_decode_block_kernel<32, 512><<<gridm, nw * 64, shm, s>>>(a);

@@ -472,20 +472,20 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
             pairs = n * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
             want = max(1, 2048 // max(1, pairs * 8))
             # More (sequence, kv head) pairs than CUs: a CU holds eight waves of this kernel, which the launch groups
-            # into blocks of eight, four, two or one by the number of blocks, so the waves run in rounds, and a last
-            # round that is far from full (272 blocks of eight waves on 256 CUs: 17 sequences of 16 kv heads) costs
-            # nearly as much as a full one.  More chunks a sequence, which the launch then gives to blocks of one or two
-            # waves, fill the CUs evenly: 17 sequences at 2,060 keys 80 -> 58 us, 24 sequences 87 -> 79 us, 72 sequences
-            # 231 -> 209 us, 96 sequences 297 -> 266 us, 17 at 8,200 keys 285 -> 192 us; where the last round is full
-            # (32, 64, 128 sequences) one chunk is 2-4 % ahead, and where it is 85-90 % full the two are level.
+            # into blocks of eight or four (one chunk a sequence), so the waves run in rounds, and a last round that
+            # is far from full (272 blocks of eight waves on 256 CUs: 17 sequences of 16 kv heads) costs nearly as much
+            # as a full one.  Eight chunks a sequence, which the launch then gives to blocks of one wave, fill the CUs
+            # evenly: 17 sequences at 2,060 keys 80 -> 58 us, 24 sequences 81 -> 77 us, 36 sequences 125 -> 108 us, 17 at
+            # 8,200 keys 285 -> 192 us; where the last round is full (32, 64 sequences) one chunk is 2-4 % ahead, and
+            # from 1,024 pairs on one chunk in blocks of four waves is level with every other choice.
             cus = compute_units(q.device)
-            if SPLIT_PARTIAL_ROUNDS and pairs > cus and max_kv_len >= 1024:
-                waves = 8                       # per block, as fx_attn_decode picks them for one chunk a sequence
-                while waves > 1 and pairs * (waves // 2) >= 8 * cus:
-                    waves //= 2
-                rounds = pairs * waves / (8 * cus)
+            if SPLIT_PARTIAL_ROUNDS and cus < pairs <= 4 * cus and max_kv_len >= 1024:
+                per_block = 8                   # waves, as fx_attn_decode picks them for one chunk a sequence
+                while per_block > 4 and pairs * (per_block // 2) >= 8 * cus:
+                    per_block //= 2
+                rounds = pairs * per_block / (8 * cus)
                 if (math.ceil(rounds) - rounds) / math.ceil(rounds) >= 0.10:
-                    want = 8 if pairs <= 4 * cus else 4
+                    want = 8
             chunk = max(64, -(-(-(-max_kv_len // want)) // 64) * 64)
     splits = max(1, -(-max_kv_len // chunk))
     part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
