@@ -456,37 +456,42 @@ def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, 
 SPLIT_PARTIAL_ROUNDS = True      # decode attention: more chunks where the blocks' last round over the CUs would be far from full
 
 
+def decode_attention_chunk(n_items: int, n_heads: int, n_kv_heads: int, max_kv_len: int, cus: int) -> int:
+    """Keys per chunk of the bfloat16 decode attention, where the caller names none: the fewest chunks that still put
+    about eight waves on every CU (one chunk, and no merge launch, from as many (sequence, kv head) pairs as CUs
+    on), unless the waves' last round over the CUs would be far from full."""
+    pairs = n_items * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
+    want = max(1, 8 * cus // max(1, pairs * 8))
+    # More (sequence, kv head) pairs than CUs: a CU holds eight waves of this kernel, which the launch groups
+    # into blocks of eight or four (one chunk a sequence), so the waves run in rounds, and a last round that
+    # is far from full (272 blocks of eight waves on 256 CUs: 17 sequences of 16 kv heads) costs nearly as much
+    # as a full one.  Eight chunks a sequence, which the launch then gives to blocks of one wave, fill the CUs
+    # evenly: 17 sequences at 2,060 keys 80 -> 58 us, 24 sequences 81 -> 77 us, 36 sequences 125 -> 108 us, 17 at
+    # 8,200 keys 285 -> 192 us; where the last round is full (32, 64 sequences) one chunk is 2-4 % ahead, and
+    # from four pairs a CU on one chunk is level with every other choice.
+    if SPLIT_PARTIAL_ROUNDS and cus < pairs <= 4 * cus and max_kv_len >= 1024:
+        per_block = 8                   # waves, as fx_attn_decode picks them for one chunk a sequence
+        while per_block > 4 and pairs * (per_block // 2) >= 8 * cus:
+            per_block //= 2
+        rounds = pairs * per_block / (8 * cus)
+        if (math.ceil(rounds) - rounds) / math.ceil(rounds) >= 0.10:
+            want = 8
+    return max(64, -(-(-(-max_kv_len // want)) // 64) * 64)
+
+
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
                      waves=0) -> None:
     """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
     order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
-    batch); bfloat16, whose blocks of eight waves share a chunk, cuts every sequence's own range of keys (from its
-    window's first key to its position) into that many equal chunks of whole tiles of 64, and by default takes the
-    fewest chunks that still put about two thousand waves on the GPU: one chunk, and no merge launch, from 256
-    (sequence, kv head) pairs on, unless the blocks' last round over the CUs would be far from full."""
+    batch); bfloat16, whose blocks of up to eight waves share a chunk, cuts every sequence's own range of keys (from
+    its window's first key to its position) into that many equal chunks of whole tiles of 64, `chunk` by default as
+    `decode_attention_chunk` picks it.  `waves`: waves per block, 0 for the launch's own choice."""
     n = item_seq.numel()
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
-            pairs = n * n_kv_heads * (-(-(n_heads // n_kv_heads) // 16))
-            want = max(1, 2048 // max(1, pairs * 8))
-            # More (sequence, kv head) pairs than CUs: a CU holds eight waves of this kernel, which the launch groups
-            # into blocks of eight or four (one chunk a sequence), so the waves run in rounds, and a last round that
-            # is far from full (272 blocks of eight waves on 256 CUs: 17 sequences of 16 kv heads) costs nearly as much
-            # as a full one.  Eight chunks a sequence, which the launch then gives to blocks of one wave, fill the CUs
-            # evenly: 17 sequences at 2,060 keys 80 -> 58 us, 24 sequences 81 -> 77 us, 36 sequences 125 -> 108 us, 17 at
-            # 8,200 keys 285 -> 192 us; where the last round is full (32, 64 sequences) one chunk is 2-4 % ahead, and
-            # from 1,024 pairs on one chunk in blocks of four waves is level with every other choice.
-            cus = compute_units(q.device)
-            if SPLIT_PARTIAL_ROUNDS and cus < pairs <= 4 * cus and max_kv_len >= 1024:
-                per_block = 8                   # waves, as fx_attn_decode picks them for one chunk a sequence
-                while per_block > 4 and pairs * (per_block // 2) >= 8 * cus:
-                    per_block //= 2
-                rounds = pairs * per_block / (8 * cus)
-                if (math.ceil(rounds) - rounds) / math.ceil(rounds) >= 0.10:
-                    want = 8
-            chunk = max(64, -(-(-(-max_kv_len // want)) // 64) * 64)
+            chunk = decode_attention_chunk(n, n_heads, n_kv_heads, max_kv_len, compute_units(q.device))
     splits = max(1, -(-max_kv_len // chunk))
     part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n, n_heads, splits, 2), dtype=torch.float32, device=q.device)
