@@ -1462,14 +1462,13 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
         if (!dual && (norm_w || (M <= 2 && (long)ceil_div(N, 16) * m_tiles >= 4096))) nw = 1;
         if (spread_rows) nw = 2;
         if ((g_skinny_nw == 1 && !dual) || (g_skinny_nw == 2 && !norm_w)) nw = g_skinny_nw;
-        // Waves per block: four, a part of K each.  Unsorted pairs: one wave that runs through all four parts when
-        // the blocks number no more than the waves that the GPU holds at a time (twelve a CU: 3,072), else two (a wave then spends
-        // less of its time finding its rows and more of it streaming; measured at the sizes of the engine, one
-        // token's gate/up product 20.5 against 23.3 us, its down product 11.2 against 12.0, sixteen tokens' 96 and
-        // 53 against 104 and 62 us, eight tokens' within 3 %).  The sums are the same bits either way.
+        // Waves per block: four, a part of K each, for unsorted pairs too.  (Those ran with one wave that went
+        // through all four parts, or two, while a wave found its tile with a loop over the experts and each such
+        // search cost 1-2 us; since the search is a few ballots, four waves are ahead again: decode steps of 1, 4, 8
+        // and 16 sequences 1.87, 2.80, 3.70 and 5.17 ms with one or two waves, 1.84, 2.72, 3.64 and 5.06 ms with four.)
+        // The sums are the same bits with one, two and four waves.
         int waves = 4;
-        if (pair_ids) waves = (long)ceil_div(N, dual ? 8 * nw : 16 * nw) * m_tiles <= 12L * fx_compute_units() ? 1 : 2;
-        else if (expert_offsets && mt == 1) waves = 2;      // sorted, up to 16 rows per expert: 152 against 159 us at 64 tokens
+        if (expert_offsets && mt == 1) waves = 2;      // sorted, up to 16 rows per expert: 152 against 159 us at 64 tokens
         if (g_skinny_waves == 8 || g_skinny_waves == 4 || g_skinny_waves == 2 || g_skinny_waves == 1) waves = g_skinny_waves;
         launch_skinny(g, epi, mt, nw, waves, m_tiles, s);
         FX_CHECK_LAUNCH("gemm_bf16_skinny");
