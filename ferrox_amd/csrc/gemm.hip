@@ -470,9 +470,9 @@ __device__ __forceinline__ void wide_k_loop(f32x4_t (&acc)[MT][NT], const bf16* 
             fr[u] = *(const bf16x8_t*)(base_a + a_off + (u % NA) * 32 * 64 + ((u / NA) ? koff1 : koff0));
         static_for(std::make_integer_sequence<int, U>{}, [&](auto uc) {
             constexpr int u = decltype(uc)::value;
-            if (u + D < U)
+            if constexpr (u + D < U)
                 fr[u + D] = *(const bf16x8_t*)(base_a + a_off + ((u + D) % NA) * 32 * 64 + (((u + D) / NA) ? koff1 : koff0));
-            if (u == 0) {
+            if constexpr (u == 0) {
 #pragma unroll
                 for (int j = 0; j < NT; ++j) bfr[1][j] = *(const bf16x8_t*)(base_b + b_off + j * 16 * 64 + koff1);
             }
