@@ -213,8 +213,13 @@ class ModelRunner:
             # that shrinks by one request at a time then records a step once in eight times, not every time
             n_rec = n_seqs if n_seqs <= 8 else -(-n_seqs // 8) * 8
             key = (n_rec, bound, debug.graph_token())
-            if key not in self._graphs:
+            if key in self._graphs:
+                self._graphs[key] = self._graphs.pop(key)          # kept in the order of last use
+            else:
                 if len(self._graphs) >= 32:
+                    # the step that goes is the one unused for longest; the device may still be running it (steps
+                    # are launched ahead of their results), and its memory goes with it
+                    torch.cuda.current_stream(self.device).synchronize()
                     self._graphs.pop(next(iter(self._graphs)))
                 self._graphs[key] = DecodeGraph(self, n_rec, bound)
             try:
